@@ -1,0 +1,18 @@
+"""MI355X-native hot paths of Causal Trainer: segment-isolated attention and cut cross-entropy.
+
+The directory name contains a hyphen, so the repository root carries the
+symlink ``causal_trainer_dev_amd`` to it; import the package under that name.
+"""
+
+from . import _lib, workloads  # noqa: F401
+from .efficient_attention import (  # noqa: F401
+    AttentionKernelProfile,
+    AttentionMetadata,
+    attention_backward,
+    attention_forward_with_lse,
+    default_attention_scale,
+    efficient_attention,
+    prepare_attention_metadata,
+    resolve_attention_profile,
+    validate_attention_profile,
+)

@@ -1,0 +1,331 @@
+// C ABI of the attention hot path: argument validation and launches.
+#include "ct_attn_bwd_kernels.cuh"
+#include "ct_attn_kernels.cuh"
+#include "ct_error.h"
+
+#include <string.h>
+
+namespace ct {
+
+// ---------------------------------------------------------------------------
+// Tile bounds. One workgroup per batch row; phase 1 summarises every
+// 32-position block, phase 2 turns the summaries into visit ranges.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, const int* end, int S,
+                                                            int* meta) {
+  extern __shared__ int lds_meta[];  // [nrb][3]: min_nz, max_id, end_max
+  const int b = blockIdx.x;
+  const int nrb = S / 32, nt = S / kKeyTile;
+  const int* segb = seg + (size_t)b * S;
+  const int* endb = end ? end + (size_t)b * S : nullptr;
+  int* mb = meta + (size_t)b * nrb * kMetaW;
+
+  for (int rb = threadIdx.x; rb < nrb; rb += blockDim.x) {
+    int min_nz = INT_MAX, max_id = 0, end_min = INT_MAX, end_max = -1;
+    const int first_id = segb[rb * 32];
+    bool same = true;
+    for (int i = 0; i < 32; ++i) {
+      const int pos = rb * 32 + i;
+      const int id = segb[pos];
+      same &= (id == first_id);
+      if (id != 0) {
+        min_nz = min(min_nz, id);
+        max_id = max(max_id, id);
+        const int e = endb ? endb[pos] : pos;
+        end_min = min(end_min, e);
+        end_max = max(end_max, e);
+      }
+    }
+    if (max_id == 0) min_nz = 0;  // reference: all-padding block -> (0, 0)
+    int* m = mb + rb * kMetaW;
+    m[kMinNz] = min_nz;
+    m[kMaxId] = max_id;
+    m[kUniform] = (same && first_id != 0) ? first_id : 0;
+    m[kEndMin] = end_min;
+    m[kEndMax] = end_max;
+    m[9] = 0;
+    m[10] = 0;
+    m[11] = 0;
+    lds_meta[rb * 3 + 0] = min_nz;
+    lds_meta[rb * 3 + 1] = max_id;
+    lds_meta[rb * 3 + 2] = end_max;
+  }
+  __syncthreads();
+
+  for (int rb = threadIdx.x; rb < nrb; rb += blockDim.x) {
+    const int my_min = lds_meta[rb * 3 + 0], my_max = lds_meta[rb * 3 + 1],
+              my_end = lds_meta[rb * 3 + 2];
+    // As queries: which 64-key tiles?
+    int kv_first = INT_MAX, kv_last = -1;
+    if (my_min != 0) {
+      const int t_hi = min(my_end / kKeyTile, nt - 1);
+      for (int t = 0; t <= t_hi; ++t) {
+        const int a_min = lds_meta[(2 * t) * 3], c_min = lds_meta[(2 * t + 1) * 3];
+        const int k_min = a_min == 0 ? c_min : (c_min == 0 ? a_min : min(a_min, c_min));
+        const int k_max = max(lds_meta[(2 * t) * 3 + 1], lds_meta[(2 * t + 1) * 3 + 1]);
+        if (blocks_interact(my_min, my_max, my_end, k_min, k_max, t * kKeyTile)) {
+          kv_first = min(kv_first, t);
+          kv_last = t;
+        }
+      }
+    }
+    // As keys: which 32-row query blocks?
+    int q_first = INT_MAX, q_last = -1;
+    if (my_min != 0) {
+      for (int qb = 0; qb < nrb; ++qb) {
+        if (blocks_interact(lds_meta[qb * 3], lds_meta[qb * 3 + 1], lds_meta[qb * 3 + 2], my_min,
+                            my_max, rb * 32)) {
+          q_first = min(q_first, qb);
+          q_last = qb;
+        }
+      }
+    }
+    int* m = mb + rb * kMetaW;
+    m[kKvFirst] = kv_first;
+    m[kKvLast] = kv_last;
+    m[kQFirst] = q_first;
+    m[kQLast] = q_last;
+  }
+}
+
+__global__ void attn_block_summary_kernel(const int* seg, const int* end, int S, int block,
+                                          int nblocks, int width, int* out) {
+  const int gid = blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= nblocks) return;
+  const int per_row = S / block;
+  const int b = gid / per_row, blk = gid % per_row;
+  const int* segb = seg + (size_t)b * S + (size_t)blk * block;
+  int min_nz = INT_MAX, max_id = 0, end_max = 0;
+  for (int i = 0; i < block; ++i) {
+    const int id = segb[i];
+    if (id != 0) {
+      min_nz = min(min_nz, id);
+      max_id = max(max_id, id);
+    }
+    if (end) end_max = max(end_max, id != 0 ? end[(size_t)b * S + (size_t)blk * block + i] : 0);
+  }
+  if (max_id == 0) min_nz = 0;
+  out[(size_t)gid * width + 0] = min_nz;
+  out[(size_t)gid * width + 1] = max_id;
+  if (end) out[(size_t)gid * width + 2] = end_max;
+}
+
+static float round_to_bf16(float x) {
+  uint32_t u;
+  ::memcpy(&u, &x, 4);
+  const uint32_t lsb = (u >> 16) & 1u;
+  u += 0x7fffu + lsb;
+  u &= 0xffff0000u;
+  float y;
+  ::memcpy(&y, &u, 4);
+  return y;
+}
+
+static int validate_shape(const char* fn, int B, int S, int Hq, int Hkv, int D) {
+  CT_REQUIRE(B > 0 && S > 0 && Hq > 0 && Hkv > 0, "%s: dimensions must be positive", fn);
+  CT_REQUIRE(S % 128 == 0, "%s: sequence length %d has no 128-aligned tiling", fn, S);
+  CT_REQUIRE(Hq % Hkv == 0,
+             "%s: query head count must be divisible by the KV head count, got Hq=%d, Hkv=%d", fn,
+             Hq, Hkv);
+  if (D != 64 && D != 128) return fail(CT_UNSUPPORTED, "%s: head_dim must be 64 or 128, got %d", fn, D);
+  if (S > 262144) return fail(CT_UNSUPPORTED, "%s: sequence length %d exceeds 262144", fn, S);
+  return CT_OK;
+}
+
+// Query heads of one KV head handled by a single workgroup.
+static int heads_per_group(int Hq, int Hkv) {
+  const int g = Hq / Hkv;
+  return g % 4 == 0 ? 4 : (g % 2 == 0 ? 2 : 1);
+}
+
+template <int D, int HS>
+static int launch_fwd(hipStream_t stream, const AttnParams& p) {
+  constexpr int PB = 4 / HS;
+  const size_t smem = KvSmem<D>::kBytes;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, HS>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_fwd: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int grid = (p.S / (32 * PB)) * (p.Hq / HS) * p.B;
+  hipLaunchKernelGGL((attn_fwd_kernel<D, HS>), dim3(grid), dim3(256), smem, stream, p);
+  return check_launch("ct_attn_fwd");
+}
+
+template <int D>
+static int dispatch_fwd(hipStream_t stream, const AttnParams& p) {
+  switch (heads_per_group(p.Hq, p.Hkv)) {
+    case 4: return launch_fwd<D, 4>(stream, p);
+    case 2: return launch_fwd<D, 2>(stream, p);
+    default: return launch_fwd<D, 1>(stream, p);
+  }
+}
+
+template <int D, int HS>
+static int launch_dq(hipStream_t stream, const AttnParams& p) {
+  constexpr int PB = 4 / HS;
+  const size_t smem = KvSmem<D>::kBytes;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dq_kernel<D, HS>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int grid = (p.S / (32 * PB)) * (p.Hq / HS) * p.B;
+  hipLaunchKernelGGL((attn_dq_kernel<D, HS>), dim3(grid), dim3(256), smem, stream, p);
+  return check_launch("ct_attn_bwd (dq)");
+}
+
+template <int D>
+static int launch_dkv(hipStream_t stream, const AttnParams& p) {
+  const size_t smem = DkvSmem<D>::kBytes;
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dkv_kernel<D>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int grid = (p.S / 128) * p.Hkv * p.B;
+  hipLaunchKernelGGL((attn_dkv_kernel<D>), dim3(grid), dim3(256), smem, stream, p);
+  return check_launch("ct_attn_bwd (dkv)");
+}
+
+template <int D>
+static int dispatch_bwd(hipStream_t stream, const AttnParams& p) {
+  const long rows = (long)p.B * p.S * p.Hq;
+  const long threads = rows * (D / 8);
+  hipLaunchKernelGGL((attn_delta_kernel<D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                     stream, p.out, p.dout, p.delta, rows);
+  int rc = check_launch("ct_attn_bwd (delta)");
+  if (rc) return rc;
+  switch (heads_per_group(p.Hq, p.Hkv)) {
+    case 4: rc = launch_dq<D, 4>(stream, p); break;
+    case 2: rc = launch_dq<D, 2>(stream, p); break;
+    default: rc = launch_dq<D, 1>(stream, p); break;
+  }
+  if (rc) return rc;
+  return launch_dkv<D>(stream, p);
+}
+
+}  // namespace ct
+
+using namespace ct;
+
+extern "C" size_t ct_attn_meta_bytes(int32_t batch, int32_t seq) {
+  if (batch <= 0 || seq <= 0) return 0;
+  return (size_t)batch * (size_t)(seq / 32) * kMetaW * sizeof(int32_t);
+}
+
+extern "C" int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
+                                   const int32_t* attention_end, int32_t batch, int32_t seq,
+                                   int32_t* tile_meta) {
+  CT_REQUIRE(segment_ids && tile_meta, "ct_attn_prepare: null pointer");
+  int rc = validate_shape("ct_attn_prepare", batch, seq, 1, 1, 128);
+  if (rc) return rc;
+  const int nrb = seq / 32;
+  const size_t smem = (size_t)nrb * 3 * sizeof(int);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prepare_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 8192 * 3 * 4);
+    if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_prepare: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int threads = nrb >= 1024 ? 1024 : ((nrb + 63) / 64) * 64;
+  hipLaunchKernelGGL(attn_prepare_kernel, dim3(batch), dim3(threads), smem, (hipStream_t)stream,
+                     segment_ids, attention_end, seq, tile_meta);
+  return check_launch("ct_attn_prepare");
+}
+
+extern "C" int32_t ct_attn_block_summary(void* stream, const int32_t* segment_ids,
+                                         const int32_t* attention_end, int32_t batch, int32_t seq,
+                                         int32_t block, int32_t* out) {
+  CT_REQUIRE(segment_ids && out, "ct_attn_block_summary: null pointer");
+  CT_REQUIRE(batch > 0 && seq > 0 && block > 0, "ct_attn_block_summary: dimensions must be positive");
+  CT_REQUIRE(seq % block == 0, "ct_attn_block_summary: sequence %d not divisible by block %d", seq,
+             block);
+  const int nblocks = batch * (seq / block);
+  hipLaunchKernelGGL(attn_block_summary_kernel, dim3((nblocks + 127) / 128), dim3(128), 0,
+                     (hipStream_t)stream, segment_ids, attention_end, seq, block, nblocks,
+                     attention_end ? 3 : 2, out);
+  return check_launch("ct_attn_block_summary");
+}
+
+extern "C" int32_t ct_attn_fwd(void* stream, const ct_attn_fwd_args* a) {
+  CT_REQUIRE(a, "ct_attn_fwd: null args");
+  CT_REQUIRE(a->q && a->k && a->v && a->segment_ids && a->tile_meta && a->out && a->lse,
+             "ct_attn_fwd: null pointer");
+  int rc = validate_shape("ct_attn_fwd", a->batch, a->seq, a->q_heads, a->kv_heads, a->head_dim);
+  if (rc) return rc;
+  CT_REQUIRE(a->scale == a->scale && a->scale - a->scale == 0.f, "ct_attn_fwd: scale must be finite");
+  AttnParams p = {};
+  p.q = reinterpret_cast<const bf16*>(a->q);
+  p.k = reinterpret_cast<const bf16*>(a->k);
+  p.v = reinterpret_cast<const bf16*>(a->v);
+  p.seg = a->segment_ids;
+  p.end = a->attention_end;
+  p.meta = a->tile_meta;
+  p.out = reinterpret_cast<bf16*>(a->out);
+  p.lse = a->lse;
+  p.B = a->batch;
+  p.S = a->seq;
+  p.Hq = a->q_heads;
+  p.Hkv = a->kv_heads;
+  p.scale = round_to_bf16(a->scale);
+  return a->head_dim == 128 ? dispatch_fwd<128>((hipStream_t)stream, p)
+                            : dispatch_fwd<64>((hipStream_t)stream, p);
+}
+
+extern "C" int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16_t* dout,
+                                 float* delta, int64_t rows, int32_t head_dim) {
+  CT_REQUIRE(out && dout && delta, "ct_attn_delta: null pointer");
+  CT_REQUIRE(rows > 0, "ct_attn_delta: rows must be positive");
+  if (head_dim != 64 && head_dim != 128)
+    return fail(CT_UNSUPPORTED, "ct_attn_delta: head_dim must be 64 or 128, got %d", head_dim);
+  const long threads = rows * (head_dim / 8);
+  const dim3 grid((unsigned)((threads + 255) / 256));
+  if (head_dim == 128)
+    hipLaunchKernelGGL((attn_delta_kernel<128>), grid, dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<const bf16*>(out), reinterpret_cast<const bf16*>(dout),
+                       delta, (long)rows);
+  else
+    hipLaunchKernelGGL((attn_delta_kernel<64>), grid, dim3(256), 0, (hipStream_t)stream,
+                       reinterpret_cast<const bf16*>(out), reinterpret_cast<const bf16*>(dout),
+                       delta, (long)rows);
+  return check_launch("ct_attn_delta");
+}
+
+extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
+  CT_REQUIRE(a, "ct_attn_bwd: null args");
+  CT_REQUIRE(a->q && a->k && a->v && a->segment_ids && a->tile_meta && a->out && a->lse &&
+                 a->dout && a->dq && a->dk && a->dv && a->delta,
+             "ct_attn_bwd: null pointer");
+  int rc = validate_shape("ct_attn_bwd", a->batch, a->seq, a->q_heads, a->kv_heads, a->head_dim);
+  if (rc) return rc;
+  CT_REQUIRE(a->scale == a->scale && a->scale - a->scale == 0.f, "ct_attn_bwd: scale must be finite");
+  AttnParams p = {};
+  p.q = reinterpret_cast<const bf16*>(a->q);
+  p.k = reinterpret_cast<const bf16*>(a->k);
+  p.v = reinterpret_cast<const bf16*>(a->v);
+  p.seg = a->segment_ids;
+  p.end = a->attention_end;
+  p.meta = a->tile_meta;
+  p.out = const_cast<bf16*>(reinterpret_cast<const bf16*>(a->out));
+  p.lse = const_cast<float*>(a->lse);
+  p.dout = reinterpret_cast<const bf16*>(a->dout);
+  p.delta = a->delta;
+  p.dq = reinterpret_cast<bf16*>(a->dq);
+  p.dk = reinterpret_cast<bf16*>(a->dk);
+  p.dv = reinterpret_cast<bf16*>(a->dv);
+  p.B = a->batch;
+  p.S = a->seq;
+  p.Hq = a->q_heads;
+  p.Hkv = a->kv_heads;
+  p.scale = round_to_bf16(a->scale);
+  return a->head_dim == 128 ? dispatch_bwd<128>((hipStream_t)stream, p)
+                            : dispatch_bwd<64>((hipStream_t)stream, p);
+}

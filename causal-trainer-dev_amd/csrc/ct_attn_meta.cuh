@@ -1,0 +1,90 @@
+// Tile-bounds buffer shared by the attention kernels.
+//
+// The sequence is cut into 32-position blocks ("row blocks"). For each block
+// the buffer holds CT_ATTN_META_WIDTH int32:
+//   [0] min_nz   smallest nonzero segment id in the block, 0 if none
+//   [1] max_id   largest id among nonzero ids, 0 if none
+//   [2] uniform  the id shared by all 32 positions if they are equal and
+//                nonzero, else 0
+//   [3] end_min  min visible end over positions with id != 0 (INT_MAX if none)
+//   [4] end_max  max visible end over positions with id != 0 (-1 if none)
+//   [5] kv_first first 64-key tile this block (as queries) has to visit
+//   [6] kv_last  last such tile (-1 / INT_MAX pair when there is none)
+//   [7] q_first  first 32-row query block that has to visit this block (as keys)
+//   [8] q_last   last such block
+// [0], [1] and the "has to visit" predicate follow the reference's block
+// summaries and skip test (src/kernels/efficient_attention.py:313-323,
+// :377-412): two blocks interact iff both hold a nonzero id, their id ranges
+// overlap, and the key block starts at or before the query block's largest
+// visible end.
+#pragma once
+
+#include <limits.h>
+
+#include "ct_common.cuh"
+
+namespace ct {
+
+constexpr int kMetaW = 12;
+enum MetaSlot {
+  kMinNz = 0,
+  kMaxId = 1,
+  kUniform = 2,
+  kEndMin = 3,
+  kEndMax = 4,
+  kKvFirst = 5,
+  kKvLast = 6,
+  kQFirst = 7,
+  kQLast = 8,
+};
+
+struct KeyTileBounds {
+  int min_nz;
+  int max_id;
+  int uniform;
+};
+
+// Bounds of the 64-key tile `t` = row blocks 2t and 2t+1 (wave-uniform).
+CT_DEVICE KeyTileBounds key_tile_bounds(const int* meta_b, int t) {
+  const int* a = meta_b + (2 * t) * kMetaW;
+  const int* c = a + kMetaW;
+  const int a_min = a[kMinNz], c_min = c[kMinNz];
+  KeyTileBounds out;
+  out.min_nz = a_min == 0 ? c_min : (c_min == 0 ? a_min : min(a_min, c_min));
+  out.max_id = max(a[kMaxId], c[kMaxId]);
+  out.uniform = (a[kUniform] == c[kUniform]) ? a[kUniform] : 0;
+  return out;
+}
+
+struct QueryBlockBounds {
+  int min_nz, max_id, uniform, end_min, end_max, kv_first, kv_last;
+};
+
+CT_DEVICE QueryBlockBounds query_block_bounds(const int* meta_b, int rb) {
+  const int* m = meta_b + rb * kMetaW;
+  QueryBlockBounds q;
+  q.min_nz = uniform(m[kMinNz]);
+  q.max_id = uniform(m[kMaxId]);
+  q.uniform = uniform(m[kUniform]);
+  q.end_min = uniform(m[kEndMin]);
+  q.end_max = uniform(m[kEndMax]);
+  q.kv_first = uniform(m[kKvFirst]);
+  q.kv_last = uniform(m[kKvLast]);
+  return q;
+}
+
+// Does query block q have any allowed pair in a key range with bounds k that
+// starts at key_start? (conservative: may say yes for a fully masked tile)
+CT_DEVICE bool blocks_interact(int q_min, int q_max, int q_end_max, int k_min, int k_max,
+                               int key_start) {
+  return q_min != 0 && k_min != 0 && max(q_min, k_min) <= min(q_max, k_max) &&
+         key_start <= q_end_max;
+}
+
+// Every (query, key) pair of the tile is allowed: one shared nonzero id and
+// the last key is visible from every query of the block.
+CT_DEVICE bool tile_is_interior(int q_uniform, int q_end_min, int k_uniform, int key_last) {
+  return q_uniform != 0 && q_uniform == k_uniform && key_last <= q_end_min;
+}
+
+}  // namespace ct

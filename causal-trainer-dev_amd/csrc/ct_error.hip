@@ -1,0 +1,28 @@
+#include "ct_error.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+namespace ct {
+
+static thread_local char g_error[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_launch(const char* what) {
+  hipError_t err = hipGetLastError();
+  if (err == hipSuccess) return CT_OK;
+  return fail(CT_LAUNCH_FAILED, "%s: %s", what, hipGetErrorString(err));
+}
+
+}  // namespace ct
+
+extern "C" const char* ct_last_error(void) { return ct::g_error; }
+
+extern "C" int32_t ct_abi_version(void) { return 1; }

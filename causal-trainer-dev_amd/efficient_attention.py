@@ -1,0 +1,464 @@
+"""Host-side mirror of the reference's Efficient attention operator for MI355X.
+
+Same public names, argument meaning and error behaviour as
+``src/causal_trainer/kernels/efficient_attention.py`` (AttentionKernelProfile
+:52-60, AttentionMetadata :63-74, resolve_attention_profile :235-279,
+prepare_attention_metadata :326-374, efficient_attention :1890-1967), with
+torch tensors on a ROCm device instead of jax arrays on TPU, and with the
+kernel work done by libct_hotpath.so through its C ABI.
+
+Differences from the reference, all relaxations:
+  * GQA: any ``Hkv`` dividing ``Hq`` (the reference kernel needs ``Hkv == 1``;
+    the head map ``kv = h // (Hq // Hkv)`` is vanilla_attention's,
+    src/causal_trainer/modeling/attention.py:115-118);
+  * ``head_dim`` 64 or 128;
+  * ``mesh`` may be ``None`` or any mapping / object with ``.shape`` whose axis
+    sizes are all 1: this build runs on one GPU.
+The profile's tile sizes only set the granularity of the summaries kept in
+AttentionMetadata; the HIP kernels use their own 32-row / 64-key tiling and
+read per-tile bounds from ``AttentionMetadata.tile_bounds``.
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import math
+import operator
+from collections.abc import Mapping, Sequence
+from typing import NamedTuple
+
+import torch
+
+from . import _lib
+
+_TILE_ALIGN = 128
+_ROWS_COMMON = 2048
+_ROWS_LONG = 1024
+_ROWS_HYBRID = 1024
+_MAX_QUERY_TOKENS = 512
+_MAX_QUERY_COMPUTE_ELEMENTS = 131_072
+_SUPPORTED_HEAD_DIMS = (64, 128)
+
+
+@dataclasses.dataclass(frozen=True)
+class AttentionKernelProfile:
+    """Static tile choices shared by forward, dQ and dKV (summary granularity here)."""
+
+    block_h: int
+    block_q: int
+    block_kv_outer: int
+    block_kv_compute: int
+    compact_statistics: bool = False
+
+
+class AttentionMetadata(NamedTuple):
+    """Packed metadata reused across layers, optionally with per-query end keys.
+
+    ``attention_end`` holds inclusive global key indices. Hybrid query
+    summaries carry the maximum visible end as a third column. ``tile_bounds``
+    is this build's addition: the opaque per-tile buffer the HIP kernels read.
+    """
+
+    query_segment_ids: torch.Tensor
+    kv_segment_ids: torch.Tensor
+    q_block_segments: torch.Tensor
+    kv_block_segments: torch.Tensor
+    attention_end: torch.Tensor | None = None
+    tile_bounds: torch.Tensor | None = None
+
+
+def _shape_tuple(shape: Sequence[int], name: str) -> tuple[int, ...]:
+    try:
+        result = tuple(operator.index(dimension) for dimension in shape)
+    except TypeError as error:
+        raise TypeError(f"{name} must be a static integer shape") from error
+    if any(dimension <= 0 for dimension in result):
+        raise ValueError(f"{name} dimensions must be positive, got {result}")
+    return result
+
+
+def _mesh_sizes(mesh) -> Mapping[str, int]:
+    if mesh is None:
+        return {}
+    sizes = getattr(mesh, "shape", mesh)
+    if not isinstance(sizes, Mapping):
+        raise TypeError("mesh_shape must be a Mesh or a mapping of named axis sizes")
+    return sizes
+
+
+def _mesh_size(mesh, axis: str) -> int:
+    try:
+        size = operator.index(_mesh_sizes(mesh).get(axis, 1))
+    except TypeError as error:
+        raise TypeError(f"mesh axis {axis!r} must have a static integer size") from error
+    if size <= 0:
+        raise ValueError(f"mesh axis {axis!r} must have a positive size, got {size}")
+    return size
+
+
+def _require_single_device(mesh) -> None:
+    active = {axis: int(size) for axis, size in _mesh_sizes(mesh).items() if int(size) != 1}
+    if active:
+        raise ValueError(f"this build runs on one GPU; mesh axes larger than 1: {active}")
+
+
+def _static_positive_int(value, name: str) -> int:
+    if isinstance(value, bool):
+        raise TypeError(f"{name} must be a static positive integer")
+    try:
+        result = operator.index(value)
+    except TypeError as error:
+        raise TypeError(f"{name} must be a static positive integer") from error
+    if result <= 0:
+        raise ValueError(f"{name} must be positive, got {result}")
+    return result
+
+
+def _validate_qkv_shapes(q_shape, kv_shape, mesh):
+    query_shape = _shape_tuple(q_shape, "q_shape")
+    key_value_shape = _shape_tuple(kv_shape, "kv_shape")
+    if len(query_shape) != 4 or len(key_value_shape) != 4:
+        raise ValueError(
+            "attention shapes must be [batch, sequence, heads, dim], got "
+            f"q={query_shape}, kv={key_value_shape}"
+        )
+    if query_shape[:2] != key_value_shape[:2]:
+        raise ValueError(
+            f"Q and KV batch/sequence dimensions must match, got q={query_shape}, kv={key_value_shape}"
+        )
+    if query_shape[-1] != key_value_shape[-1]:
+        raise ValueError(
+            f"Q and KV head dimensions must match, got q={query_shape[-1]}, kv={key_value_shape[-1]}"
+        )
+    if query_shape[2] % key_value_shape[2]:
+        raise ValueError(
+            "query head count must be divisible by the KV head count, got "
+            f"Hq={query_shape[2]}, Hkv={key_value_shape[2]}"
+        )
+    tp_size = _mesh_size(mesh, "tp")
+    sp_size = _mesh_size(mesh, "sp")
+    data_size = _mesh_size(mesh, "dp") * _mesh_size(mesh, "fsdp")
+    if query_shape[0] % data_size:
+        raise ValueError(f"global batch {query_shape[0]} must be divisible by dp*fsdp={data_size}")
+    if query_shape[2] % tp_size:
+        raise ValueError(f"Hq={query_shape[2]} must be divisible by TP={tp_size}")
+    if query_shape[1] % sp_size:
+        raise ValueError(f"sequence={query_shape[1]} must be divisible by SP={sp_size}")
+    return query_shape, key_value_shape, tp_size, sp_size
+
+
+def validate_attention_profile(profile, q_shape, kv_shape, mesh_shape) -> None:
+    """Check divisibility of the profile against the shapes (reference :159-195)."""
+
+    if not isinstance(profile, AttentionKernelProfile):
+        raise TypeError(f"profile must be AttentionKernelProfile, got {type(profile).__name__}")
+    if not isinstance(profile.compact_statistics, bool):
+        raise TypeError("profile.compact_statistics must be a static bool")
+    query_shape, _, tp_size, sp_size = _validate_qkv_shapes(q_shape, kv_shape, mesh_shape)
+    block_h = _static_positive_int(profile.block_h, "block_h")
+    block_q = _static_positive_int(profile.block_q, "block_q")
+    outer = _static_positive_int(profile.block_kv_outer, "block_kv_outer")
+    compute = _static_positive_int(profile.block_kv_compute, "block_kv_compute")
+    local_heads = query_shape[2] // tp_size
+    local_query = query_shape[1] // sp_size
+    details = (
+        f"q_shape={query_shape}, kv_shape={tuple(kv_shape)}, TP={tp_size}, SP={sp_size}, "
+        f"local_heads={local_heads}, local_query={local_query}, profile={profile}"
+    )
+    if block_h != local_heads:
+        raise ValueError(f"the efficient kernel requires block_h=local_heads; {details}")
+    if block_q % _TILE_ALIGN or local_query % block_q:
+        raise ValueError(f"block_q must be a 128-aligned divisor of local_query; {details}")
+    if outer % _TILE_ALIGN or query_shape[1] % outer:
+        raise ValueError(f"block_kv_outer must be a 128-aligned divisor of sequence; {details}")
+    if compute % _TILE_ALIGN or query_shape[1] % compute:
+        raise ValueError(f"block_kv_compute must be a 128-aligned divisor of sequence; {details}")
+    if compute > outer or outer % compute:
+        raise ValueError(f"block_kv_compute must divide block_kv_outer; {details}")
+
+
+def _aligned_divisors(length: int, limit: int) -> list[int]:
+    return [b for b in range(_TILE_ALIGN, min(length, limit) + 1, _TILE_ALIGN) if length % b == 0]
+
+
+def _nearest_query_tile(local_query, local_heads, preferred_rows, max_query_tokens):
+    candidates = _aligned_divisors(local_query, max_query_tokens)
+    if not candidates:
+        raise ValueError(
+            "SP-local query length has no 128-aligned static divisor: "
+            f"local_query={local_query}, local_heads={local_heads}"
+        )
+    target = preferred_rows / local_heads
+    return min(candidates, key=lambda block: (abs(block - target), block))
+
+
+def _largest_aligned_divisor(length: int, preferred: int) -> int:
+    candidates = _aligned_divisors(length, preferred)
+    if not candidates:
+        raise ValueError(
+            f"length has no 128-aligned static divisor: length={length}, preferred={preferred}"
+        )
+    return max(candidates)
+
+
+def resolve_attention_profile(q_shape, kv_shape, mesh_shape, *, compact_statistics=False,
+                              has_attention_end=False) -> AttentionKernelProfile:
+    """Resolve the static profile from global shapes (reference tiers, :251-276)."""
+
+    query_shape, _, tp_size, sp_size = _validate_qkv_shapes(q_shape, kv_shape, mesh_shape)
+    if not isinstance(has_attention_end, bool):
+        raise TypeError("has_attention_end must be a static bool")
+    local_heads = query_shape[2] // tp_size
+    local_query = query_shape[1] // sp_size
+    sequence = query_shape[1]
+    if sequence <= 16_384:
+        rows, outer_pref, compute_pref = _ROWS_COMMON, 512, 256
+    elif sequence <= 262_144:
+        rows, outer_pref, compute_pref = _ROWS_LONG, 1024, 256
+    else:
+        rows, outer_pref, compute_pref = _ROWS_LONG, 2048, 512
+    if has_attention_end:
+        rows = min(rows, _ROWS_HYBRID)
+    outer = _largest_aligned_divisor(sequence, outer_pref)
+    compute = _largest_aligned_divisor(outer, compute_pref)
+    max_query_tokens = min(_MAX_QUERY_TOKENS, _MAX_QUERY_COMPUTE_ELEMENTS // compute)
+    profile = AttentionKernelProfile(
+        block_h=local_heads,
+        block_q=_nearest_query_tile(local_query, local_heads, rows, max_query_tokens),
+        block_kv_outer=outer,
+        block_kv_compute=compute,
+        compact_statistics=compact_statistics,
+    )
+    validate_attention_profile(profile, q_shape, kv_shape, mesh_shape)
+    return profile
+
+
+def default_attention_scale(head_dim: int) -> float:
+    """``head_dim ** -0.5`` (reference :282-286)."""
+
+    return _static_positive_int(head_dim, "head_dim") ** -0.5
+
+
+def _as_device_int32(value, name: str) -> torch.Tensor:
+    tensor = torch.as_tensor(value)
+    if tensor.dtype != torch.int32:
+        tensor = tensor.to(torch.int32)
+    if not tensor.is_cuda:
+        raise RuntimeError(f"{name} must live on a ROCm device")
+    return tensor.contiguous()
+
+
+def _block_summary(segments: torch.Tensor, ends: torch.Tensor | None, block: int) -> torch.Tensor:
+    batch, sequence = segments.shape
+    width = 3 if ends is not None else 2
+    out = torch.empty((batch, sequence // block, width), dtype=torch.int32, device=segments.device)
+    lib = _lib.load()
+    _lib.check(lib.ct_attn_block_summary(_lib.current_stream(), segments.data_ptr(),
+                                         _lib.pointer(ends), batch, sequence, block,
+                                         out.data_ptr()))
+    return out
+
+
+def prepare_attention_metadata(canonical_segment_ids, *, mesh, profile,
+                               attention_end=None) -> AttentionMetadata:
+    """Build per-tile summaries once, immediately before the decoder loop."""
+
+    if not isinstance(profile, AttentionKernelProfile):
+        raise TypeError("profile must be an AttentionKernelProfile")
+    _require_single_device(mesh)
+    segments = _as_device_int32(canonical_segment_ids, "canonical_segment_ids")
+    if segments.ndim != 2:
+        raise ValueError(f"canonical_segment_ids must be [batch, sequence], got {tuple(segments.shape)}")
+    if segments.shape[0] == 0 or segments.shape[1] == 0:
+        raise ValueError("canonical_segment_ids must have non-empty batch and sequence dimensions")
+    block_q = _static_positive_int(profile.block_q, "profile.block_q")
+    outer = _static_positive_int(profile.block_kv_outer, "profile.block_kv_outer")
+    batch, sequence = segments.shape
+    if sequence % block_q or sequence % outer:
+        raise ValueError(
+            f"metadata sequence must be divisible by profile blocks, got shape={tuple(segments.shape)}, "
+            f"profile={profile}"
+        )
+    ends = None
+    if attention_end is not None:
+        ends = _as_device_int32(attention_end, "attention_end")
+        if ends.shape != segments.shape:
+            raise ValueError("attention_end must match canonical_segment_ids")
+
+    lib = _lib.load()
+    bounds = torch.empty(lib.ct_attn_meta_bytes(batch, sequence) // 4, dtype=torch.int32,
+                         device=segments.device)
+    with torch.cuda.device(segments.device):
+        _lib.check(lib.ct_attn_prepare(_lib.current_stream(), segments.data_ptr(),
+                                       _lib.pointer(ends), batch, sequence, bounds.data_ptr()))
+        q_summary = _block_summary(segments, ends, block_q)
+        kv_summary = _block_summary(segments, None, outer)
+    return AttentionMetadata(
+        query_segment_ids=segments,
+        kv_segment_ids=segments,
+        q_block_segments=q_summary,
+        kv_block_segments=kv_summary,
+        attention_end=ends,
+        tile_bounds=bounds.view(batch, sequence // 32, _lib.ATTN_META_WIDTH),
+    )
+
+
+def _validate_metadata(metadata, query_shape, profile) -> None:
+    if not isinstance(metadata, AttentionMetadata):
+        raise TypeError("metadata must be AttentionMetadata")
+    batch, sequence = query_shape[:2]
+    expected = {
+        "query_segment_ids": (batch, sequence),
+        "kv_segment_ids": (batch, sequence),
+        "q_block_segments": (batch, sequence // profile.block_q,
+                             3 if metadata.attention_end is not None else 2),
+        "kv_block_segments": (batch, sequence // profile.block_kv_outer, 2),
+    }
+    if metadata.attention_end is not None:
+        expected["attention_end"] = (batch, sequence)
+    for name, shape in expected.items():
+        value = getattr(metadata, name)
+        if tuple(value.shape) != shape:
+            raise ValueError(f"metadata.{name} must have shape {shape}, got {tuple(value.shape)}")
+        if value.dtype != torch.int32:
+            raise TypeError(f"metadata.{name} must have dtype int32, got {value.dtype}")
+    if metadata.tile_bounds is None or tuple(metadata.tile_bounds.shape) != (
+        batch, sequence // 32, _lib.ATTN_META_WIDTH
+    ):
+        raise ValueError("metadata.tile_bounds is missing; build it with prepare_attention_metadata")
+
+
+def _attn_forward(query, key, value, metadata, scale):
+    batch, sequence, q_heads, head_dim = query.shape
+    out = torch.empty_like(query)
+    lse = torch.empty((batch, sequence, q_heads), dtype=torch.float32, device=query.device)
+    args = _lib.AttnFwdArgs(
+        q=query.data_ptr(), k=key.data_ptr(), v=value.data_ptr(),
+        segment_ids=metadata.query_segment_ids.data_ptr(),
+        attention_end=_lib.pointer(metadata.attention_end),
+        tile_meta=metadata.tile_bounds.data_ptr(),
+        out=out.data_ptr(), lse=lse.data_ptr(),
+        batch=batch, seq=sequence, q_heads=q_heads, kv_heads=key.shape[2], head_dim=head_dim,
+        scale=scale,
+    )
+    with torch.cuda.device(query.device):
+        _lib.check(_lib.load().ct_attn_fwd(_lib.current_stream(), args))
+    return out, lse
+
+
+def _attn_backward(query, key, value, metadata, out, lse, dout, scale):
+    batch, sequence, q_heads, head_dim = query.shape
+    dq = torch.empty_like(query)
+    dk = torch.empty_like(key)
+    dv = torch.empty_like(value)
+    delta = torch.empty_like(lse)
+    args = _lib.AttnBwdArgs(
+        q=query.data_ptr(), k=key.data_ptr(), v=value.data_ptr(),
+        segment_ids=metadata.query_segment_ids.data_ptr(),
+        attention_end=_lib.pointer(metadata.attention_end),
+        tile_meta=metadata.tile_bounds.data_ptr(),
+        out=out.data_ptr(), lse=lse.data_ptr(), dout=dout.data_ptr(),
+        dq=dq.data_ptr(), dk=dk.data_ptr(), dv=dv.data_ptr(), delta=delta.data_ptr(),
+        batch=batch, seq=sequence, q_heads=q_heads, kv_heads=key.shape[2], head_dim=head_dim,
+        scale=scale,
+    )
+    with torch.cuda.device(query.device):
+        _lib.check(_lib.load().ct_attn_bwd(_lib.current_stream(), args))
+    return dq, dk, dv
+
+
+class _EfficientAttention(torch.autograd.Function):
+    """Custom VJP with the reference's residual (q, k, v, metadata, O, LSE) (:1831-1863)."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, metadata, scale):
+        out, lse = _attn_forward(query, key, value, metadata, scale)
+        ctx.save_for_backward(query, key, value, out, lse)
+        ctx.metadata = metadata
+        ctx.scale = scale
+        return out
+
+    @staticmethod
+    def backward(ctx, output_cotangent):
+        query, key, value, out, lse = ctx.saved_tensors
+        dout = output_cotangent.to(torch.bfloat16).contiguous()
+        dq, dk, dv = _attn_backward(query, key, value, ctx.metadata, out, lse, dout, ctx.scale)
+        return dq, dk, dv, None, None
+
+
+def efficient_attention(query, key, value, metadata, *, mesh=None, profile=None, scale=None,
+                        causal=True):
+    """Segment-isolated causal attention forward with its analytic custom VJP.
+
+    query ``[B, S, Hq, D]``, key / value ``[B, S, Hkv, D]``, all bf16 on a ROCm
+    device; returns ``[B, S, Hq, D]`` bf16. Gradients flow to query, key, value.
+    """
+
+    if not isinstance(causal, bool):
+        raise TypeError("causal must be a compile-time bool")
+    if not causal:
+        raise ValueError("the efficient backend implements causal attention only")
+    if key.shape != value.shape:
+        raise ValueError(f"key and value shapes differ: {tuple(key.shape)} and {tuple(value.shape)}")
+    query_shape, key_shape, _, _ = _validate_qkv_shapes(query.shape, key.shape, mesh)
+    _require_single_device(mesh)
+    if query_shape[-1] not in _SUPPORTED_HEAD_DIMS:
+        raise ValueError(
+            "the efficient attention kernel requires head_dim in (64, 128); "
+            f"got head_dim={query_shape[-1]}"
+        )
+    if any(t.dtype != torch.bfloat16 for t in (query, key, value)):
+        raise TypeError(
+            "efficient_attention requires BF16 query/key/value, got "
+            f"{query.dtype}, {key.dtype}, {value.dtype}"
+        )
+    if not (query.is_cuda and key.is_cuda and value.is_cuda):
+        raise RuntimeError("efficient_attention is available only on a ROCm GPU")
+    has_end = metadata.attention_end is not None if isinstance(metadata, AttentionMetadata) else False
+    resolved_profile = (
+        resolve_attention_profile(query_shape, key_shape, mesh, has_attention_end=has_end)
+        if profile is None else profile
+    )
+    validate_attention_profile(resolved_profile, query_shape, key_shape, mesh)
+    _validate_metadata(metadata, query_shape, resolved_profile)
+    if scale is None:
+        resolved_scale = default_attention_scale(query_shape[-1])
+    else:
+        if isinstance(scale, torch.Tensor):
+            raise TypeError("scale must be a compile-time Python scalar")
+        try:
+            resolved_scale = float(scale)
+        except (TypeError, ValueError) as error:
+            raise TypeError("scale must be a compile-time Python scalar") from error
+        if not math.isfinite(resolved_scale):
+            raise ValueError(f"scale must be finite, got {resolved_scale}")
+    return _EfficientAttention.apply(
+        query.contiguous(), key.contiguous(), value.contiguous(), metadata, resolved_scale
+    )
+
+
+def attention_forward_with_lse(query, key, value, metadata, *, scale=None):
+    """Forward only, returning ``(O, LSE)``: the residual pair the custom VJP saves."""
+
+    resolved = default_attention_scale(query.shape[-1]) if scale is None else float(scale)
+    return _attn_forward(query.contiguous(), key.contiguous(), value.contiguous(), metadata, resolved)
+
+
+def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=None):
+    """Backward only, from the saved residuals: returns ``(dq, dk, dv)``."""
+
+    resolved = default_attention_scale(query.shape[-1]) if scale is None else float(scale)
+    return _attn_backward(query, key, value, metadata, out, lse, dout.contiguous(), resolved)
+
+
+__all__ = [
+    "AttentionKernelProfile",
+    "AttentionMetadata",
+    "attention_backward",
+    "attention_forward_with_lse",
+    "default_attention_scale",
+    "efficient_attention",
+    "prepare_attention_metadata",
+    "resolve_attention_profile",
+    "validate_attention_profile",
+]

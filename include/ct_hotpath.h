@@ -1,0 +1,220 @@
+/*
+ * ct_hotpath.h -- C ABI of the MI355X (gfx950) hot-path library.
+ *
+ * Two hot paths of the Causal Trainer reference are provided:
+ *   1. segment-isolated causal attention with GQA and per-query visibility
+ *      ends (forward, logsumexp residual, custom backward);
+ *   2. projection-fused cut cross-entropy (forward statistics + loss,
+ *      backward dHidden / dHead).
+ *
+ * Conventions
+ *   - Every pointer is a DEVICE pointer unless named host_*. All tensors are
+ *     dense row-major with the last dimension contiguous, exactly the layouts
+ *     the reference passes to its kernels.
+ *   - `stream` is a hipStream_t passed as void*. Work is only enqueued on
+ *     that stream. No entry point synchronises, allocates or frees device
+ *     memory, or keeps state between calls (ct_last_error is thread local).
+ *   - Return value: 0 on success, a negative ct_status otherwise; the text
+ *     for the most recent failure on the calling thread is ct_last_error().
+ *     Argument validation happens before anything is launched.
+ *   - bf16 tensors are passed as uint16_t* (raw bfloat16 bits).
+ *
+ * Reference citations are relative to the reference repository root,
+ * "src/" abbreviating src/causal_trainer/.
+ */
+#ifndef CT_HOTPATH_H_
+#define CT_HOTPATH_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum ct_status {
+  CT_OK = 0,
+  CT_INVALID_ARGUMENT = -1, /* shape / dtype / alignment / null pointer */
+  CT_UNSUPPORTED = -2,      /* valid request the kernels do not implement */
+  CT_WORKSPACE_TOO_SMALL = -3,
+  CT_LAUNCH_FAILED = -4     /* HIP reported an error at launch */
+} ct_status;
+
+/* Text of the last failure on this thread ("" if none). */
+const char* ct_last_error(void);
+
+/* Library ABI version (bumped on any signature change). */
+int32_t ct_abi_version(void);
+
+/* ------------------------------------------------------------------------
+ * Attention
+ * --------------------------------------------------------------------- */
+
+/* Number of int32 per 32-position block in the tile-bounds buffer. */
+#define CT_ATTN_META_WIDTH 12
+
+/* Bytes of the tile-bounds buffer for [batch, seq] segment ids. */
+size_t ct_attn_meta_bytes(int32_t batch, int32_t seq);
+
+/*
+ * Per-tile segment / visibility bounds used by every attention kernel to
+ * skip fully masked tiles and to drop the per-element mask on interior
+ * tiles. Run once per forward, reuse for every layer and for the backward.
+ *
+ * Replaces: prepare_attention_metadata and _segment_block_summary
+ * (src/kernels/efficient_attention.py:313-374) together with the skip
+ * predicates _summary_should_run / _compute_tile_is_causally_reachable
+ * (:377-434), evaluated ahead of time.
+ *
+ *   segment_ids   int32 [batch, seq]  canonical ids, 0 = padding
+ *   attention_end int32 [batch, seq]  inclusive last visible key per query,
+ *                                     or NULL for plain causal (end = q)
+ *   tile_meta     int32 out, ct_attn_meta_bytes(batch, seq) bytes
+ * seq must be a positive multiple of 128 (reference: :221-232).
+ */
+int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
+                        const int32_t* attention_end, int32_t batch, int32_t seq,
+                        int32_t* tile_meta);
+
+/*
+ * Block summaries in the reference's own format, for callers that keep the
+ * AttentionMetadata tuple: out[b, blk] = (min nonzero id, max id) and, when
+ * attention_end != NULL, a third column max(end where id != 0).
+ * Replaces: _segment_block_summary + the hybrid column
+ * (src/kernels/efficient_attention.py:313-323, :359-365).
+ *   out int32 [batch, seq / block, attention_end ? 3 : 2]
+ */
+int32_t ct_attn_block_summary(void* stream, const int32_t* segment_ids,
+                              const int32_t* attention_end, int32_t batch, int32_t seq,
+                              int32_t block, int32_t* out);
+
+typedef struct ct_attn_fwd_args {
+  const uint16_t* q;            /* bf16 [batch, seq, q_heads, head_dim] */
+  const uint16_t* k;            /* bf16 [batch, seq, kv_heads, head_dim] */
+  const uint16_t* v;            /* bf16 [batch, seq, kv_heads, head_dim] */
+  const int32_t* segment_ids;   /* int32 [batch, seq] */
+  const int32_t* attention_end; /* int32 [batch, seq] or NULL */
+  const int32_t* tile_meta;     /* from ct_attn_prepare (same ids / ends) */
+  uint16_t* out;                /* bf16 [batch, seq, q_heads, head_dim] */
+  float* lse;                   /* f32  [batch, seq, q_heads], natural log of
+                                   the scaled scores; 0.0 on rows with no
+                                   visible key */
+  int32_t batch, seq, q_heads, kv_heads, head_dim;
+  float scale;                  /* rounded to bf16 and folded into q in bf16 */
+} ct_attn_fwd_args;
+
+/*
+ * O, LSE = attention(q, k, v). Query head h reads KV head h / (q_heads /
+ * kv_heads). allowed(q, key) = key <= end[q] && seg[q] == seg[key] &&
+ * seg[q] != 0.
+ * Replaces: _local_attention_forward / _attention_forward_kernel
+ * (src/kernels/efficient_attention.py:560-770, :889-982); mask semantics of
+ * _make_causal_segment_mask_precanonicalized (src/modeling/attention.py:67-97);
+ * GQA head map of vanilla_attention (src/modeling/attention.py:115-118).
+ * head_dim in {64, 128}; q_heads % kv_heads == 0; seq % 128 == 0.
+ */
+int32_t ct_attn_fwd(void* stream, const ct_attn_fwd_args* args);
+
+typedef struct ct_attn_bwd_args {
+  const uint16_t* q;
+  const uint16_t* k;
+  const uint16_t* v;
+  const int32_t* segment_ids;
+  const int32_t* attention_end; /* or NULL */
+  const int32_t* tile_meta;
+  const uint16_t* out;          /* forward output (residual) */
+  const float* lse;             /* forward logsumexp (residual) */
+  const uint16_t* dout;         /* bf16 cotangent of out */
+  uint16_t* dq;                 /* bf16 [batch, seq, q_heads, head_dim] */
+  uint16_t* dk;                 /* bf16 [batch, seq, kv_heads, head_dim] */
+  uint16_t* dv;                 /* bf16 [batch, seq, kv_heads, head_dim] */
+  float* delta;                 /* f32 scratch [batch, seq, q_heads] */
+  int32_t batch, seq, q_heads, kv_heads, head_dim;
+  float scale;
+} ct_attn_bwd_args;
+
+/*
+ * dq, dk, dv from the saved (q, k, v, out, lse) and dout. Three launches:
+ * delta = rowsum(out * dout); dq per query tile; dk/dv per key tile (single
+ * owner, no atomics, deterministic).
+ * Replaces: delta at src/kernels/efficient_attention.py:1735-1738,
+ * _local_attention_dq (:985-1267), _local_attention_dkv (:1270-1602) and the
+ * f32 -> bf16 cast at :1774.
+ */
+int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* args);
+
+/* The delta pass alone (exposed so it can be measured by itself). */
+int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16_t* dout,
+                      float* delta, int64_t rows, int32_t head_dim);
+
+/* ------------------------------------------------------------------------
+ * Cut cross-entropy
+ * --------------------------------------------------------------------- */
+
+typedef struct ct_cutce_shape {
+  int32_t rows;   /* N = flattened token rows */
+  int32_t hidden; /* d, multiple of 128 */
+  int32_t vocab;  /* V > 0 */
+} ct_cutce_shape;
+
+/* Bytes of workspace ct_cutce_fwd needs. */
+size_t ct_cutce_fwd_workspace_bytes(const ct_cutce_shape* shape);
+/*
+ * Smallest and preferred workspace for ct_cutce_bwd. With the preferred size
+ * the whole vocabulary is processed as one slab; with less, the vocabulary
+ * is walked in slabs and dHidden is accumulated in f32 in the workspace.
+ */
+size_t ct_cutce_bwd_workspace_min_bytes(const ct_cutce_shape* shape);
+size_t ct_cutce_bwd_workspace_bytes(const ct_cutce_shape* shape);
+
+typedef struct ct_cutce_fwd_args {
+  const uint16_t* hidden;  /* bf16 [rows, hidden] */
+  const uint16_t* head;    /* bf16 [hidden, vocab] (vocab contiguous) */
+  const int32_t* targets;  /* int32 [rows]; never used to index memory */
+  const float* weights;    /* f32 [rows]; a row is ignored iff weight == 0 */
+  float* nll_sum;          /* f32 [1] */
+  float* weight_sum;       /* f32 [1] */
+  float* lse;              /* f32 [rows]; 0.0 on ignored rows */
+  void* workspace;
+  size_t workspace_bytes;
+  ct_cutce_shape shape;
+  int32_t sparse_compaction; /* gather active rows first (same results) */
+} ct_cutce_fwd_args;
+
+/*
+ * nll_sum = sum_i w_i (logsumexp_v(hidden_i . head[:, v]) - hidden_i . head[:, t_i]),
+ * weight_sum = sum_i w_i, lse_i saved for the backward. Logits are never
+ * written to memory.
+ * Replaces: _cut_stats_pallas + _loss_and_lse + _compact_active_rows
+ * (src/kernels/cut_cross_entropy.py:85-222, :474-521, :673-694).
+ */
+int32_t ct_cutce_fwd(void* stream, const ct_cutce_fwd_args* args);
+
+typedef struct ct_cutce_bwd_args {
+  const uint16_t* hidden;
+  const uint16_t* head;
+  const int32_t* targets;
+  const float* weights;
+  const float* lse;        /* from ct_cutce_fwd */
+  const float* dy;         /* f32 [1]: cotangent of nll_sum */
+  uint16_t* dhidden;       /* bf16 [rows, hidden]; exactly 0 on ignored rows */
+  uint16_t* dhead;         /* bf16 [hidden, vocab], or NULL when the head is
+                              frozen (then the dHead kernel is never launched) */
+  void* workspace;
+  size_t workspace_bytes;
+  ct_cutce_shape shape;
+  int32_t sparse_compaction;
+} ct_cutce_bwd_args;
+
+/*
+ * G = w * dy * (softmax(logits) - onehot(target)) rounded to bf16,
+ * dHidden = G @ head^T, dHead = hidden^T @ G, f32 accumulation.
+ * Replaces: _cut_hidden_bwd_pallas and _cut_head_bwd_pallas
+ * (src/kernels/cut_cross_entropy.py:225-471) and the scatter at :638-642.
+ */
+int32_t ct_cutce_bwd(void* stream, const ct_cutce_bwd_args* args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CT_HOTPATH_H_ */
