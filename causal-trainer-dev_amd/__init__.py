@@ -16,3 +16,8 @@ from .efficient_attention import (  # noqa: F401
     resolve_attention_profile,
     validate_attention_profile,
 )
+from .cut_cross_entropy import (  # noqa: F401,E402
+    cutce_backward,
+    cutce_forward,
+    pallas_cut_linear_cross_entropy,
+)

@@ -1,0 +1,163 @@
+"""Host-side mirror of the reference's Cut cross-entropy operator for MI355X.
+
+``pallas_cut_linear_cross_entropy`` keeps the reference's name, argument
+meaning, validation errors and custom-VJP contract
+(src/causal_trainer/kernels/cut_cross_entropy.py:828-958, :524-670): it
+returns ``(nll_sum, weight_sum)`` as f32 scalars, saves
+``(hidden, head, targets, weights, lse)`` and no logits, gives no cotangent to
+targets / weights, ignores the cotangent of ``weight_sum``, and with
+``lm_head_trainable=False`` never launches the dHead kernel and returns no
+head gradient. Tensors are torch tensors on a ROCm device; the work is done by
+libct_hotpath.so through its C ABI.
+
+``loss = nll_sum / max(weight_sum, 1)`` stays with the caller
+(src/causal_trainer/training/losses.py:234-237).
+"""
+
+from __future__ import annotations
+
+import operator
+
+import torch
+
+from . import _lib
+from .efficient_attention import _mesh_sizes
+
+_HIDDEN_ALIGN = 128
+
+
+def _shape_struct(rows: int, hidden: int, vocab: int) -> _lib.CutceShape:
+    return _lib.CutceShape(rows=rows, hidden=hidden, vocab=vocab)
+
+
+def cutce_forward(hidden, head, targets, weights, *, sparse_compaction: bool = False):
+    """Flat forward: hidden [N, d], head [d, V] -> (nll_sum, weight_sum, lse [N])."""
+
+    lib = _lib.load()
+    rows, width = hidden.shape
+    shape = _shape_struct(rows, width, head.shape[1])
+    device = hidden.device
+    workspace = torch.empty(lib.ct_cutce_fwd_workspace_bytes(shape), dtype=torch.uint8, device=device)
+    scalars = torch.empty(2, dtype=torch.float32, device=device)
+    lse = torch.empty(rows, dtype=torch.float32, device=device)
+    args = _lib.CutceFwdArgs(
+        hidden=hidden.data_ptr(), head=head.data_ptr(), targets=targets.data_ptr(),
+        weights=weights.data_ptr(), nll_sum=scalars[0:].data_ptr(),
+        weight_sum=scalars[1:].data_ptr(), lse=lse.data_ptr(),
+        workspace=workspace.data_ptr(), workspace_bytes=workspace.numel(),
+        shape=shape, sparse_compaction=int(bool(sparse_compaction)),
+    )
+    with torch.cuda.device(device):
+        _lib.check(lib.ct_cutce_fwd(_lib.current_stream(), args))
+    return scalars[0], scalars[1], lse
+
+
+def cutce_backward(hidden, head, targets, weights, lse, dy, *, sparse_compaction: bool = False,
+                   lm_head_trainable: bool = True, workspace_bytes: int | None = None):
+    """Flat backward: returns (dhidden [N, d], dhead [d, V] or None)."""
+
+    lib = _lib.load()
+    rows, width = hidden.shape
+    shape = _shape_struct(rows, width, head.shape[1])
+    device = hidden.device
+    if workspace_bytes is None:
+        workspace_bytes = lib.ct_cutce_bwd_workspace_bytes(shape)
+    workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=device)
+    dhidden = torch.empty_like(hidden)
+    dhead = torch.empty_like(head) if lm_head_trainable else None
+    dy = dy.to(device=device, dtype=torch.float32).reshape(1).contiguous()
+    args = _lib.CutceBwdArgs(
+        hidden=hidden.data_ptr(), head=head.data_ptr(), targets=targets.data_ptr(),
+        weights=weights.data_ptr(), lse=lse.data_ptr(), dy=dy.data_ptr(),
+        dhidden=dhidden.data_ptr(), dhead=_lib.pointer(dhead),
+        workspace=workspace.data_ptr(), workspace_bytes=workspace.numel(),
+        shape=shape, sparse_compaction=int(bool(sparse_compaction)),
+    )
+    with torch.cuda.device(device):
+        _lib.check(lib.ct_cutce_bwd(_lib.current_stream(), args))
+    return dhidden, dhead
+
+
+class _CutCE(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, head, targets, weights, lm_head_trainable, sparse_compaction):
+        nll_sum, weight_sum, lse = cutce_forward(hidden, head, targets, weights,
+                                                 sparse_compaction=sparse_compaction)
+        # The complete residual: no logits (reference :587-593).
+        ctx.save_for_backward(hidden, head, targets, weights, lse)
+        ctx.lm_head_trainable = lm_head_trainable
+        ctx.sparse_compaction = sparse_compaction
+        ctx.mark_non_differentiable(weight_sum)
+        return nll_sum, weight_sum
+
+    @staticmethod
+    def backward(ctx, nll_cotangent, _weight_cotangent):
+        hidden, head, targets, weights, lse = ctx.saved_tensors
+        dhidden, dhead = cutce_backward(
+            hidden, head, targets, weights, lse, nll_cotangent,
+            sparse_compaction=ctx.sparse_compaction, lm_head_trainable=ctx.lm_head_trainable,
+        )
+        return dhidden, dhead, None, None, None, None
+
+
+def pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weights, *, mesh=None,
+                                    sparse_compaction: bool = False,
+                                    lm_head_trainable: bool = True, local_chunk_size: int = 0):
+    """Return ``(nll_sum, weight_sum)`` without materialising logits.
+
+    hidden_states ``[B, S, d]``, lm_head_kernel ``[d, V]`` (same float dtype, bf16),
+    targets int32 ``[B, S]``, weights f32 ``[B, S]``; a row is ignored iff its weight is 0.
+    """
+
+    if isinstance(local_chunk_size, bool):
+        raise TypeError("local_chunk_size must be a static non-negative integer")
+    try:
+        local_chunk_size = operator.index(local_chunk_size)
+    except TypeError as error:
+        raise TypeError("local_chunk_size must be a static non-negative integer") from error
+    if local_chunk_size < 0:
+        raise ValueError("local_chunk_size must be non-negative")
+    if hidden_states.ndim != 3:
+        raise ValueError("Cut cross-entropy expects hidden_states [batch, sequence, hidden]")
+    if lm_head_kernel.ndim != 2 or lm_head_kernel.shape[0] != hidden_states.shape[-1]:
+        raise ValueError("lm_head_kernel must have shape [hidden, vocab]")
+    targets = torch.as_tensor(targets, device=hidden_states.device).to(torch.int32)
+    weights = torch.as_tensor(weights, device=hidden_states.device).to(torch.float32)
+    if targets.shape != hidden_states.shape[:-1] or weights.shape != targets.shape:
+        raise ValueError("targets and weights must match hidden_states.shape[:-1]")
+    if hidden_states.shape[0] == 0 or hidden_states.shape[1] == 0:
+        raise ValueError("Cut cross-entropy requires at least one token row")
+    if hidden_states.shape[-1] == 0 or hidden_states.shape[-1] % _HIDDEN_ALIGN:
+        raise ValueError("Cut cross-entropy hidden size must be divisible by 128")
+    if lm_head_kernel.shape[1] == 0:
+        raise ValueError("Cut cross-entropy requires a non-empty vocabulary")
+    if hidden_states.dtype != lm_head_kernel.dtype:
+        raise TypeError("hidden_states and lm_head_kernel must use the same compute dtype")
+    if not hidden_states.dtype.is_floating_point:
+        raise TypeError("Cut cross-entropy inputs must have a floating dtype")
+    if hidden_states.dtype != torch.bfloat16:
+        raise TypeError("this build computes Cut cross-entropy in bfloat16 only")
+    if not hidden_states.is_cuda:
+        raise RuntimeError("Cut cross-entropy is available only on a ROCm GPU")
+    sizes = _mesh_sizes(mesh)
+    unsupported = tuple(axis for axis in ("fsdp", "ep") if int(sizes.get(axis, 1)) != 1)
+    if unsupported:
+        raise ValueError(
+            "Cut cross-entropy currently requires fsdp=ep=1; active unsupported axes: "
+            + ", ".join(unsupported)
+        )
+    active = {axis: int(size) for axis, size in sizes.items() if int(size) != 1}
+    if active:
+        raise ValueError(f"this build runs on one GPU; mesh axes larger than 1: {active}")
+    if local_chunk_size:
+        raise ValueError("local_chunk_size needs a tensor-parallel mesh; this build runs on one GPU")
+
+    width = hidden_states.shape[-1]
+    return _CutCE.apply(
+        hidden_states.reshape(-1, width).contiguous(), lm_head_kernel.contiguous(),
+        targets.reshape(-1).contiguous(), weights.reshape(-1).contiguous(),
+        bool(lm_head_trainable), bool(sparse_compaction),
+    )
+
+
+__all__ = ["cutce_backward", "cutce_forward", "pallas_cut_linear_cross_entropy"]

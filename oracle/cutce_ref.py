@@ -1,0 +1,165 @@
+"""CPU oracle for the cut cross-entropy hot path. TEST INFRASTRUCTURE ONLY.
+
+Imported by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg of
+bench.py, and by nothing else: the product never calls it.
+
+The reference (JAX) cannot be imported in this environment, so parity is
+anchored on this restatement, pinned by tests/test_oracle_cutce.py against
+  * the reference's closed forms (zero hidden => nll = sum(w) * log V),
+  * the known answers of its shifted-target tests,
+  * torch.nn.functional.cross_entropy / log_softmax and autograd,
+  * the per-row identity sum_v dlogits = 0.
+Citations are relative to the reference root; "src/" = src/causal_trainer/.
+
+Functions and what they follow:
+  shifted_targets_and_weights   src/training/losses.py:21-85
+  mean_loss                     src/training/losses.py:234-237
+  compact_active_rows           src/kernels/cut_cross_entropy.py:673-694
+  cut_forward                   src/kernels/cut_cross_entropy.py:85-156, :474-521
+  cut_backward                  src/kernels/cut_cross_entropy.py:225-278, :349-403, :597-667
+  xla_sparse_cross_entropy(+vjp)  src/kernels/fused_cross_entropy.py:64-109
+  cut_f64                       float64 evaluation of the same mathematics
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from .attention_ref import canonicalize_segment_ids
+
+
+def shifted_targets_and_weights(input_ids, attention_mask, segment_ids=None, assistant_mask=None,
+                                loss_mask=None, labels=None, *, ignore_index: int = -100):
+    tokens = np.asarray(input_ids).astype(np.int32)
+    if tokens.ndim != 2:
+        raise ValueError(f"input_ids must have shape [batch, sequence], got {tokens.shape}")
+    labels = tokens if labels is None else np.asarray(labels).astype(np.int32)
+    valid_tokens = (np.ones(tokens.shape, bool) if attention_mask is None
+                    else np.asarray(attention_mask) == 1)
+    targets = labels[:, 1:]
+    valid = valid_tokens[:, :-1] & valid_tokens[:, 1:] & (targets != ignore_index)
+    if segment_ids is not None:
+        segments = canonicalize_segment_ids(valid_tokens, np.asarray(segment_ids))
+        valid &= (segments[:, :-1] == segments[:, 1:]) & (segments[:, 1:] != 0)
+    weights = valid.astype(np.float32)
+    if assistant_mask is not None:
+        weights = weights * (np.asarray(assistant_mask) != 0)[:, 1:].astype(np.float32)
+    if loss_mask is not None:
+        weights = weights * np.asarray(loss_mask, dtype=np.float32)[:, 1:]
+    safe_targets = np.where(weights > 0.0, targets, 0).astype(np.int32)
+    return safe_targets, weights.astype(np.float32)
+
+
+def mean_loss(nll_sum, weight_sum):
+    return nll_sum / max(float(weight_sum), 1.0)
+
+
+def compact_active_rows(hidden, targets, weights):
+    """Stable fixed-shape gather: active rows first; returns the reference's 5-tuple."""
+
+    weights = torch.as_tensor(weights)
+    rows = weights.shape[0]
+    active = weights != 0
+    nonzero = torch.nonzero(active).flatten()
+    indices = torch.zeros(rows, dtype=torch.long)
+    indices[: nonzero.numel()] = nonzero
+    slot_valid = torch.arange(rows) < nonzero.numel()
+    compact_hidden = hidden[indices]
+    compact_targets = torch.where(slot_valid, torch.as_tensor(targets)[indices], 0)
+    compact_weights = torch.where(slot_valid, weights[indices], 0.0)
+    return compact_hidden, compact_targets, compact_weights, indices, slot_valid
+
+
+def _logits_f32(hidden, head):
+    # bf16 x bf16 products are exact in f32; accumulation in f32.
+    return hidden.float() @ head.float()
+
+
+def cut_forward(hidden, head, targets, weights):
+    """(nll_sum f32, weight_sum f32, lse f32 [N]) for hidden [N, d], head [d, V]."""
+
+    targets = torch.as_tensor(targets).long()
+    weights = torch.as_tensor(weights).float()
+    logits = _logits_f32(hidden, head)
+    valid = weights != 0
+    vocab = logits.shape[1]
+    lse = torch.where(valid, torch.logsumexp(logits, dim=-1), 0.0)
+    in_range = (targets >= 0) & (targets < vocab)
+    gathered = logits.gather(1, targets.clamp(0, vocab - 1)[:, None])[:, 0]
+    target_logit = torch.where(in_range, gathered, 0.0)
+    losses = torch.where(valid, weights * (lse - target_logit), 0.0)
+    return losses.sum(dtype=torch.float32), weights.sum(dtype=torch.float32), lse
+
+
+def cut_backward(hidden, head, targets, weights, lse, dy: float, *, head_trainable: bool = True):
+    """(dhidden bf16 [N, d], dhead bf16 [d, V] or None). G is rounded to bf16 before both products."""
+
+    targets = torch.as_tensor(targets).long()
+    weights = torch.as_tensor(weights).float()
+    logits = _logits_f32(hidden, head)
+    valid = (weights != 0)[:, None]
+    vocab = logits.shape[1]
+    prob = torch.where(valid, torch.exp(logits - lse[:, None]), 0.0)
+    onehot = torch.zeros_like(prob)
+    in_range = (targets >= 0) & (targets < vocab) & (weights != 0)
+    rows = torch.nonzero(in_range).flatten()
+    onehot[rows, targets[rows]] = 1.0
+    g = ((weights * float(dy))[:, None] * (prob - onehot)).to(torch.bfloat16)
+    dhidden = (g.float() @ head.float().T).to(hidden.dtype)
+    dhead = (hidden.float().T @ g.float()).to(head.dtype) if head_trainable else None
+    return dhidden, dhead
+
+
+def xla_sparse_cross_entropy(logits, targets, weights):
+    """Per-row weighted CE on materialised logits, differentiable via torch autograd."""
+
+    compute = logits.float()
+    log_normalizer = torch.logsumexp(compute, dim=-1)
+    target_logits = compute.gather(-1, torch.as_tensor(targets).long()[..., None])[..., 0]
+    return ((log_normalizer - target_logits) * torch.as_tensor(weights).float()).float()
+
+
+def xla_sparse_cross_entropy_vjp(logits, targets, weights, cotangent):
+    """Analytic logits cotangent: (softmax - onehot) * w * dy, cast to the logits dtype."""
+
+    compute = logits.float()
+    log_normalizer = torch.logsumexp(compute, dim=-1)
+    prob = torch.exp(compute - log_normalizer[..., None])
+    onehot = torch.nn.functional.one_hot(torch.as_tensor(targets).long(), logits.shape[-1]).float()
+    factor = (torch.as_tensor(weights).float() * torch.as_tensor(cotangent).float())[..., None]
+    return ((prob - onehot) * factor).to(logits.dtype)
+
+
+def full_logits_loss_and_grads(hidden, head, targets, weights, dy: float):
+    """The reference's pure path: materialise f32 logits, sparse CE, autograd to hidden / head."""
+
+    h = hidden.detach().clone().requires_grad_(True)
+    w = head.detach().clone().requires_grad_(True)
+    logits = (h.float() @ w.float())
+    safe_targets = torch.as_tensor(targets).long().clamp(0, head.shape[1] - 1)
+    losses = xla_sparse_cross_entropy(logits, safe_targets, weights)
+    nll = losses.sum()
+    (nll * dy).backward()
+    return nll.detach(), h.grad, w.grad
+
+
+def cut_f64(hidden, head, targets, weights, dy: float):
+    """float64 (nll_sum, weight_sum, lse, dhidden, dhead) from the bf16 inputs, no intermediate rounding."""
+
+    targets = torch.as_tensor(targets).long()
+    weights64 = torch.as_tensor(weights).double()
+    logits = hidden.double() @ head.double()
+    valid = weights64 != 0
+    vocab = logits.shape[1]
+    lse = torch.where(valid, torch.logsumexp(logits, dim=-1), 0.0)
+    in_range = (targets >= 0) & (targets < vocab)
+    gathered = logits.gather(1, targets.clamp(0, vocab - 1)[:, None])[:, 0]
+    target_logit = torch.where(in_range, gathered, 0.0)
+    nll = torch.where(valid, weights64 * (lse - target_logit), 0.0).sum()
+    prob = torch.where(valid[:, None], torch.exp(logits - lse[:, None]), 0.0)
+    onehot = torch.zeros_like(prob)
+    rows = torch.nonzero(in_range & valid).flatten()
+    onehot[rows, targets[rows]] = 1.0
+    g = (weights64 * dy)[:, None] * (prob - onehot)
+    return nll, weights64.sum(), lse, g @ head.double().T, hidden.double().T @ g
