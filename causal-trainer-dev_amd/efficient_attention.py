@@ -374,7 +374,7 @@ class _EfficientAttention(torch.autograd.Function):
     def forward(ctx, query, key, value, metadata, scale):
         out, lse = _attn_forward(query, key, value, metadata, scale)
         ctx.save_for_backward(query, key, value, out, lse)
-        ctx.metadata = metadata
+        ctx.attention_metadata = metadata
         ctx.scale = scale
         return out
 
@@ -382,7 +382,7 @@ class _EfficientAttention(torch.autograd.Function):
     def backward(ctx, output_cotangent):
         query, key, value, out, lse = ctx.saved_tensors
         dout = output_cotangent.to(torch.bfloat16).contiguous()
-        dq, dk, dv = _attn_backward(query, key, value, ctx.metadata, out, lse, dout, ctx.scale)
+        dq, dk, dv = _attn_backward(query, key, value, ctx.attention_metadata, out, lse, dout, ctx.scale)
         return dq, dk, dv, None, None
 
 

@@ -1,0 +1,312 @@
+"""GPU parity of the attention hot path (through the C ABI) against oracle/attention_ref.py.
+
+Tolerances are the stated ones: O max-abs <= 2e-2 (bf16), LSE max-abs <= 1e-3 (f32),
+dQ / dK / dV relative L2 <= 2e-2; mask handling is exact (zeros are bitwise zeros).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attention_ref as ref
+
+pytestmark = pytest.mark.gpu
+
+O_ATOL, LSE_ATOL, GRAD_RTOL = 2e-2, 1e-3, 2e-2
+
+
+def _bf16(array):
+    return torch.from_numpy(np.asarray(array, dtype=np.float32)).to(torch.bfloat16)
+
+
+def _layout(rng, batch, seq, *, holes=False, max_len=200):
+    ids = np.zeros((batch, seq), np.int32)
+    for row in range(batch):
+        position, segment = (int(rng.integers(0, 70)) if holes else 0), 1
+        while position < seq:
+            length = int(rng.integers(1, max_len))
+            if holes and rng.random() < 0.25:
+                position += length
+                continue
+            ids[row, position:position + length] = segment
+            position += length
+            segment += 1
+    return ids
+
+
+def _random_ends(rng, ids, blocks_per_row=5):
+    batch, seq = ids.shape
+    ends = np.broadcast_to(np.arange(seq, dtype=np.int32), ids.shape).copy()
+    for row in range(batch):
+        for _ in range(blocks_per_row):
+            start = int(rng.integers(0, seq - 2))
+            sid = ids[row, start]
+            if sid == 0:
+                continue
+            stop = start
+            limit = start + int(rng.integers(2, 150))
+            while stop < seq and stop < limit and ids[row, stop] == sid:
+                stop += 1
+            ends[row, start:stop] = stop - 1
+    return ends
+
+
+def _run_gpu(ct, device, q, k, v, dout, ids, ends, scale):
+    profile = ct.resolve_attention_profile(q.shape, k.shape, None, has_attention_end=ends is not None)
+    metadata = ct.prepare_attention_metadata(
+        torch.from_numpy(ids).to(device), mesh=None, profile=profile,
+        attention_end=None if ends is None else torch.from_numpy(ends).to(device))
+    qd, kd, vd, dod = (t.to(device) for t in (q, k, v, dout))
+    out, lse = ct.attention_forward_with_lse(qd, kd, vd, metadata, scale=scale)
+    dq, dk, dv = ct.attention_backward(qd, kd, vd, metadata, out, lse, dod, scale=scale)
+    torch.cuda.synchronize()
+    return tuple(t.cpu() for t in (out, lse, dq, dk, dv))
+
+
+def _check_against_oracle(results, q, k, v, dout, ids, ends, scale):
+    out, lse, dq, dk, dv = results
+    allowed = ref.allowed_from_canonical(ids, ends)
+    out_ref, dq_ref, dk_ref, dv_ref = ref.vanilla_attention_vjp(q, k, v, allowed, dout, scale=scale)
+    lse_ref = ref.efficient_lse(q, k, allowed, scale=scale)
+    assert float((out.float() - out_ref.float()).abs().max()) <= O_ATOL
+    assert float((lse - lse_ref).abs().max()) <= LSE_ATOL
+    for name, got, want in (("dq", dq, dq_ref), ("dk", dk, dk_ref), ("dv", dv, dv_ref)):
+        assert ref.relative_l2(got, want) <= GRAD_RTOL, name
+    # and against the analytic backward of the kernel being replaced
+    for got, want in zip((dq, dk, dv), ref.efficient_backward(q, k, v, allowed, out, lse, dout, scale=scale)):
+        assert ref.relative_l2(got, want) <= GRAD_RTOL
+    pad = torch.from_numpy(ids == 0)
+    assert (out[pad] == 0).all() and (lse[pad] == 0).all()
+    assert (dq[pad] == 0).all() and (dk[pad] == 0).all() and (dv[pad] == 0).all()
+    for tensor in results:
+        assert torch.isfinite(tensor.float()).all()
+
+
+CASES = [
+    # batch, seq, Hq, Hkv, D, holes, ends
+    (1, 128, 1, 1, 128, False, False),
+    (2, 256, 4, 1, 128, False, False),    # MQA as in the reference kernel
+    (2, 512, 8, 2, 128, True, False),     # GQA group 4, padding holes and leading padding
+    (1, 512, 2, 2, 128, True, True),      # MHA with bidirectional blocks
+    (2, 256, 8, 8, 64, False, False),     # head_dim 64
+    (1, 384, 6, 3, 128, True, True),      # group 2
+    (1, 256, 3, 1, 64, False, True),      # group 3 (one head per workgroup)
+    (1, 384, 16, 2, 128, True, False),    # group 8
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_S%d_Hq%d_Hkv%d_D%d_%s%s" % (
+    c[0], c[1], c[2], c[3], c[4], "holes" if c[5] else "packed", "_ends" if c[6] else ""))
+def test_forward_backward_match_oracle(ct, gpu, case):
+    batch, seq, q_heads, kv_heads, dim, holes, with_ends = case
+    rng = np.random.default_rng(hash(case) % (2 ** 31))
+    ids = _layout(rng, batch, seq, holes=holes)
+    ends = _random_ends(rng, ids) if with_ends else None
+    q = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    k = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    v = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    dout = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    scale = dim ** -0.5
+    print("case", case, flush=True)
+    results = _run_gpu(ct, gpu, q, k, v, dout, ids, ends, scale)
+    _check_against_oracle(results, q, k, v, dout, ids, ends, scale)
+
+
+def test_edge_layouts(ct, gpu):
+    rng = np.random.default_rng(11)
+    batch, seq, q_heads, kv_heads, dim = 4, 256, 4, 2, 128
+    ids = np.zeros((batch, seq), np.int32)
+    ids[1, :] = 1                       # one full-length segment
+    ids[2, 200:] = 1                    # whole leading tiles of padding
+    ids[3] = np.arange(seq) % 7 + 1     # ids that are not contiguous runs: length-1 "segments"
+    ids[3, 100:160] = 9                 # ... with one real run; row 0 stays all padding
+    q = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    k = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    v = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    dout = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    results = _run_gpu(ct, gpu, q, k, v, dout, ids, None, dim ** -0.5)
+    _check_against_oracle(results, q, k, v, dout, ids, None, dim ** -0.5)
+    assert not results[0][0].any() and not results[2][0].any()
+
+
+def test_reference_seeded_fixture(ct, gpu):
+    # inputs of the reference's tests/kernels/test_efficient_attention.py:187-223; its own bar is
+    # relative L2 < 0.03 against vanilla attention
+    golden = np.load("tests/golden/attention_rng931.npz")
+
+    def tensor(name):
+        return torch.from_numpy(golden[name]).view(torch.bfloat16)
+
+    q, k, v, dout = (tensor(n) for n in ("q", "k", "v", "dout"))
+    ids = golden["segment_ids"]
+    out, lse, dq, dk, dv = _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5)
+    for name, got in (("out", out), ("dq", dq), ("dk", dk), ("dv", dv)):
+        assert ref.relative_l2(got, tensor(name)) < 0.02, name
+        assert (got[:, ids[0] == 0] == 0).all()
+    assert float((lse - torch.from_numpy(golden["lse"])).abs().max()) <= LSE_ATOL
+    for grad in (dk, dv):
+        assert grad[0, 71:128].float().abs().sum() > 0
+        assert (grad[:, ids[0] != 2] == 0).all()
+
+
+def test_neighbour_perturbation_leaves_other_segment_bitwise_unchanged(ct, gpu):
+    # reference: tests/kernels/test_efficient_attention_tpu.py:395-424
+    rng = np.random.default_rng(21)
+    batch, seq, q_heads, kv_heads, dim = 1, 512, 4, 2, 128
+    ids = np.zeros((batch, seq), np.int32)
+    ids[0, 10:230], ids[0, 230:500] = 1, 2
+    q = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    k = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    v = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    dout = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    base = _run_gpu(ct, gpu, q, k, v, dout, ids, None, dim ** -0.5)
+    q2, k2, v2, d2 = q.clone(), k.clone(), v.clone(), dout.clone()
+    q2[:, 10:230], k2[:, 10:230], v2[:, 10:230], d2[:, 10:230] = 3.0, -2.0, 5.0, -1.0
+    other = _run_gpu(ct, gpu, q2, k2, v2, d2, ids, None, dim ** -0.5)
+    for a, b in zip(base, other):
+        assert torch.equal(a[:, 230:500], b[:, 230:500])
+    again = _run_gpu(ct, gpu, q, k, v, dout, ids, None, dim ** -0.5)
+    for a, b in zip(base, again):
+        assert torch.equal(a, b)        # fixed summation order: bitwise reproducible
+
+
+def test_zero_cross_segment_mass(ct, gpu):
+    # V carries a one-hot of the key's segment id: any attention mass that leaks to another
+    # segment shows up as a nonzero in a column that must be exactly 0.
+    rng = np.random.default_rng(31)
+    batch, seq, q_heads, kv_heads, dim = 2, 1024, 8, 2, 128
+    ids = _layout(rng, batch, seq, holes=True, max_len=120)
+    assert ids.max() < dim
+    ends = _random_ends(rng, ids, 8)
+    q = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    k = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    onehot = np.zeros((batch, seq, kv_heads, dim), np.float32)
+    b_idx, s_idx = np.nonzero(ids)
+    onehot[b_idx, s_idx, :, ids[b_idx, s_idx]] = 1.0
+    v = _bf16(onehot)
+    out = _run_gpu(ct, gpu, q, k, v, torch.zeros_like(q), ids, ends, dim ** -0.5)[0].float()
+    own = torch.zeros((batch, seq, dim), dtype=torch.bool)
+    own[torch.from_numpy(b_idx), torch.from_numpy(s_idx), torch.from_numpy(ids[b_idx, s_idx]).long()] = True
+    own = own[:, :, None, :].expand_as(out)
+    assert (out[~own] == 0).all()
+    valid = torch.from_numpy(ids != 0)
+    assert float((out[own].reshape(-1) - 1).abs().max()) <= 2 ** -7     # probabilities sum to 1
+    assert own.sum() == valid.sum() * q_heads
+
+
+def test_custom_vjp_through_autograd(ct, gpu):
+    rng = np.random.default_rng(41)
+    batch, seq, q_heads, kv_heads, dim = 1, 256, 4, 2, 128
+    ids = _layout(rng, batch, seq)
+    q, k, v, dout = (_bf16(rng.standard_normal(s)).to(gpu) for s in (
+        (batch, seq, q_heads, dim), (batch, seq, kv_heads, dim), (batch, seq, kv_heads, dim),
+        (batch, seq, q_heads, dim)))
+    profile = ct.resolve_attention_profile(q.shape, k.shape, None)
+    metadata = ct.prepare_attention_metadata(torch.from_numpy(ids).to(gpu), mesh=None, profile=profile)
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    out = ct.efficient_attention(q, k, v, metadata, mesh=None)
+    out.backward(dout)
+    lse_out, lse = ct.attention_forward_with_lse(q.detach(), k.detach(), v.detach(), metadata)
+    assert torch.equal(out.detach(), lse_out)
+    dq, dk, dv = ct.attention_backward(q.detach(), k.detach(), v.detach(), metadata, lse_out, lse, dout)
+    assert torch.equal(q.grad, dq) and torch.equal(k.grad, dk) and torch.equal(v.grad, dv)
+    with pytest.raises(ValueError, match="metadata.q_block_segments must have shape"):
+        ct.efficient_attention(q, k, v, metadata, profile=ct.AttentionKernelProfile(4, 128, 128, 128))
+
+
+def test_metadata_matches_oracle_bit_exact(ct, gpu):
+    rng = np.random.default_rng(51)
+    # known answers of the reference first (tests/kernels/test_efficient_attention.py:446-480)
+    ids = np.concatenate((np.zeros(130), np.ones(49), np.full(122, 2), np.full(211, 3))).astype(np.int32)[None]
+    metadata = ct.prepare_attention_metadata(torch.from_numpy(ids).to(gpu), mesh=None,
+                                             profile=ct.AttentionKernelProfile(1, 128, 256, 128))
+    assert metadata.q_block_segments.cpu().tolist() == [[[0, 0], [1, 2], [2, 3], [3, 3]]]
+    assert metadata.kv_block_segments.cpu().tolist() == [[[1, 2], [2, 3]]]
+    for _ in range(5):
+        ids = _layout(rng, 2, 1024, holes=True)
+        ends = _random_ends(rng, ids, 10)
+        metadata = ct.prepare_attention_metadata(
+            torch.from_numpy(ids).to(gpu), mesh=None, profile=ct.AttentionKernelProfile(1, 128, 256, 128),
+            attention_end=torch.from_numpy(ends).to(gpu))
+        q_summary, kv_summary = ref.block_summaries(ids, 128, 256, ends)
+        np.testing.assert_array_equal(metadata.q_block_segments.cpu().numpy(), q_summary)
+        np.testing.assert_array_equal(metadata.kv_block_segments.cpu().numpy(), kv_summary)
+        # tile bounds: every allowed pair lies inside the advertised visit ranges
+        bounds = metadata.tile_bounds.cpu().numpy()
+        allowed = ref.allowed_from_canonical(ids, ends)
+        for b in range(2):
+            for rb in range(1024 // 32):
+                rows = allowed[b, rb * 32:(rb + 1) * 32]
+                keys = np.flatnonzero(rows.any(0))
+                if len(keys):
+                    assert bounds[b, rb, 5] <= keys[0] // 64 and keys[-1] // 64 <= bounds[b, rb, 6]
+                cols = allowed[b, :, rb * 32:(rb + 1) * 32]
+                queries = np.flatnonzero(cols.any(1))
+                if len(queries):
+                    assert bounds[b, rb, 7] <= queries[0] // 32 and queries[-1] // 32 <= bounds[b, rb, 8]
+                block = ids[b, rb * 32:(rb + 1) * 32]
+                assert bounds[b, rb, 2] == (block[0] if (block == block[0]).all() and block[0] != 0 else 0)
+
+
+def test_delta_pass_matches_torch(ct, gpu):
+    rng = np.random.default_rng(61)
+    rows = 4 * 300 * 3
+    for dim in (64, 128):
+        out = _bf16(rng.standard_normal((rows, dim))).to(gpu)
+        dout = _bf16(rng.standard_normal((rows, dim))).to(gpu)
+        delta = torch.empty(rows, dtype=torch.float32, device=gpu)
+        ct._lib.check(ct._lib.load().ct_attn_delta(ct._lib.current_stream(), out.data_ptr(), dout.data_ptr(),
+                                                   delta.data_ptr(), rows, dim))
+        expected = (out.float() * dout.float()).sum(-1)
+        torch.testing.assert_close(delta, expected, atol=1e-4, rtol=1e-5)
+
+
+def _self_contained_window(ids_row, limit):
+    """Largest run of whole segments (and padding) of at most `limit` positions: (start, stop)."""
+
+    seq = len(ids_row)
+    cuts = [0] + [i for i in range(1, seq) if ids_row[i] != ids_row[i - 1]] + [seq]
+    best = (0, 0)
+    for a in range(len(cuts) - 1):
+        for c in range(a + 1, len(cuts)):
+            if cuts[c] - cuts[a] > limit:
+                break
+            if cuts[c] - cuts[a] > best[1] - best[0]:
+                best = (cuts[a], cuts[c])
+    return best
+
+
+@pytest.mark.parametrize("name", ["packed_small", "llama3_8b", "maskgit", "long_70b"])
+def test_benchmark_shapes(ct, gpu, name):
+    """Full benchmark shapes: size-independent properties everywhere, and the oracle on a
+    self-contained window (whole segments) of one KV head with its query group."""
+
+    W = ct.workloads
+    config = W.ATTENTION_CONFIGS[name]
+    inputs = W.make_attention_inputs(config)
+    ids = inputs["segment_ids"].numpy()
+    ends = None if inputs["attention_end"] is None else inputs["attention_end"].numpy()
+    print("shape", name, flush=True)
+    out, lse, dq, dk, dv = _run_gpu(ct, gpu, inputs["q"], inputs["k"], inputs["v"], inputs["dout"], ids, ends,
+                                    config.scale)
+    pad = torch.from_numpy(ids == 0)
+    for tensor in (out, lse, dq, dk, dv):
+        assert torch.isfinite(tensor.float()).all()
+        assert (tensor[pad] == 0).all()
+    assert (lse[~pad] != 0).any()
+
+    group = config.q_heads // config.kv_heads
+    b, kvh = config.batch - 1, config.kv_heads - 1
+    heads = slice(kvh * group, (kvh + 1) * group)
+    start, stop = _self_contained_window(ids[b], 4096)
+    assert stop - start >= 512, "no whole segment short enough for the oracle"
+    window = slice(start, stop)
+    w_ids = ids[b:b + 1, window]
+    w_ends = None if ends is None else ends[b:b + 1, window] - start
+    q = inputs["q"][b:b + 1, window, heads]
+    k = inputs["k"][b:b + 1, window, kvh:kvh + 1]
+    v = inputs["v"][b:b + 1, window, kvh:kvh + 1]
+    dout = inputs["dout"][b:b + 1, window, heads]
+    got = (out[b:b + 1, window, heads], lse[b:b + 1, window, heads], dq[b:b + 1, window, heads],
+           dk[b:b + 1, window, kvh:kvh + 1], dv[b:b + 1, window, kvh:kvh + 1])
+    _check_against_oracle(got, q, k, v, dout, w_ids, w_ends, config.scale)

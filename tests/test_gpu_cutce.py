@@ -1,0 +1,199 @@
+"""GPU parity of the cut cross-entropy hot path (through the C ABI) against oracle/cutce_ref.py.
+
+Tolerances are the stated ones: scalar loss relative error <= 1e-4, dHidden / dHead relative
+L2 <= 2e-2; the ignored-token set is exact (lse and dHidden are bitwise zero on ignored rows).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import cutce_ref as ref
+from oracle.attention_ref import relative_l2
+
+pytestmark = pytest.mark.gpu
+
+LOSS_RTOL, GRAD_RTOL, LSE_ATOL = 1e-4, 2e-2, 1e-3
+
+
+def _bf16(array):
+    return torch.from_numpy(np.asarray(array, dtype=np.float32)).to(torch.bfloat16)
+
+
+def _case(seed, rows, width, vocab, pattern="random", hidden_scale=1.0, head_scale=0.05):
+    rng = np.random.default_rng(seed)
+    hidden = _bf16(rng.normal(scale=hidden_scale, size=(rows, width)))
+    head = _bf16(rng.normal(scale=head_scale, size=(width, vocab)))
+    targets = rng.integers(vocab, size=rows).astype(np.int32)
+    weights = rng.choice(np.asarray([0.25, 1.0, 2.0], np.float32), size=rows).astype(np.float32)
+    position = np.arange(rows)
+    if pattern == "random":
+        weights[rng.random(rows) < 0.3] = 0
+    elif pattern == "trailing":
+        weights[position >= rows // 3] = 0
+    elif pattern == "alternating":
+        weights[position % 2 == 1] = 0
+    elif pattern == "middle":
+        weights[(position < rows // 3) | (position >= rows // 2)] = 0
+    elif pattern == "inactive":
+        weights[:] = 0
+    targets[weights == 0] = -100     # raw ignore labels do reach the kernel on zero-weight rows
+    return hidden, head, torch.from_numpy(targets), torch.from_numpy(weights)
+
+
+def _gpu(ct, device, hidden, head, targets, weights, dy, *, compaction, trainable=True, workspace=None):
+    hd, wd, td, ws = hidden.to(device), head.to(device), targets.to(device), weights.to(device)
+    nll, weight_sum, lse = ct.cutce_forward(hd, wd, td, ws, sparse_compaction=compaction)
+    dhidden, dhead = ct.cutce_backward(hd, wd, td, ws, lse, torch.tensor(dy), sparse_compaction=compaction,
+                                       lm_head_trainable=trainable, workspace_bytes=workspace)
+    torch.cuda.synchronize()
+    return float(nll), float(weight_sum), lse.cpu(), dhidden.cpu(), None if dhead is None else dhead.cpu()
+
+
+def _check(results, hidden, head, targets, weights, dy):
+    nll, weight_sum, lse, dhidden, dhead = results
+    nll_ref, weight_ref, lse_ref = ref.cut_forward(hidden, head, targets, weights)
+    assert nll == pytest.approx(float(nll_ref), rel=LOSS_RTOL, abs=1e-6)
+    assert weight_sum == float(weight_ref)
+    assert float((lse - lse_ref).abs().max()) <= LSE_ATOL
+    ignored = weights == 0
+    assert (lse[ignored] == 0).all() and (lse[~ignored] != 0).all()     # identical ignored-token set
+    assert (dhidden[ignored] == 0).all()
+    dh_ref, dw_ref = ref.cut_backward(hidden, head, targets, weights, lse_ref, dy)
+    assert relative_l2(dhidden, dh_ref) <= GRAD_RTOL
+    if dhead is not None:
+        assert relative_l2(dhead, dw_ref) <= GRAD_RTOL
+    # and against the pure path (materialised logits + autograd)
+    _, dh_pure, dw_pure = ref.full_logits_loss_and_grads(hidden, head, targets, weights, dy)
+    assert relative_l2(dhidden, dh_pure) <= GRAD_RTOL
+    if dhead is not None:
+        assert relative_l2(dhead, dw_pure) <= GRAD_RTOL
+
+
+@pytest.mark.parametrize("rows,width,vocab", [(256, 128, 256), (300, 128, 258), (1000, 256, 1500),
+                                              (513, 384, 1031), (64, 128, 40)])
+@pytest.mark.parametrize("compaction", [True, False])
+def test_forward_backward_match_oracle(ct, gpu, rows, width, vocab, compaction):
+    print("case", rows, width, vocab, compaction, flush=True)
+    case = _case(rows + vocab, rows, width, vocab)
+    _check(_gpu(ct, gpu, *case, 0.37, compaction=compaction), *case, 0.37)
+
+
+@pytest.mark.parametrize("pattern", ["trailing", "alternating", "middle", "inactive"])
+def test_weight_patterns(ct, gpu, pattern):
+    # reference: tests/kernels/test_cross_entropy_tpu.py:166-239
+    case = _case(7, 700, 128, 300, pattern)
+    with_c = _gpu(ct, gpu, *case, 1.0, compaction=True)
+    without = _gpu(ct, gpu, *case, 1.0, compaction=False)
+    _check(with_c, *case, 1.0)
+    _check(without, *case, 1.0)
+    assert with_c[0] == pytest.approx(without[0], rel=1e-6, abs=1e-6) and with_c[1] == without[1]
+    if pattern == "inactive":
+        # reference: tests/kernels/test_tiled_cut.py:138-155
+        assert with_c[0] == 0 and with_c[1] == 0
+        assert not with_c[3].any() and not with_c[4].any()
+
+
+def test_small_workspace_walks_vocabulary_slabs(ct, gpu):
+    case = _case(9, 900, 256, 1500)
+    lib = ct._lib.load()
+    shape = ct._lib.CutceShape(900, 256, 1500)
+    import ctypes
+    least = lib.ct_cutce_bwd_workspace_min_bytes(ctypes.byref(shape))
+    full = lib.ct_cutce_bwd_workspace_bytes(ctypes.byref(shape))
+    assert least < full
+    one_slab = _gpu(ct, gpu, *case, 0.5, compaction=True)
+    for workspace in (least, least + 2 * 1024 * 256 * 2):     # 1 and 3 tile columns per slab
+        slabs = _gpu(ct, gpu, *case, 0.5, compaction=True, workspace=workspace)
+        _check(slabs, *case, 0.5)
+        assert torch.equal(slabs[4], one_slab[4])             # dHead does not depend on the slab walk
+    with pytest.raises(ct._lib.CtError, match="workspace"):
+        _gpu(ct, gpu, *case, 0.5, compaction=True, workspace=least - 256)
+
+
+def test_reference_seeded_fixture_and_frozen_head(ct, gpu):
+    # inputs of the reference's tests/kernels/test_tiled_cut.py:66-128 (cotangent 0.37)
+    golden = np.load("tests/golden/cutce_rng460.npz")
+    hidden = torch.from_numpy(golden["hidden"]).view(torch.bfloat16)        # [2, 386, 128]
+    head = torch.from_numpy(golden["head"]).view(torch.bfloat16)
+    targets, weights = torch.from_numpy(golden["targets"]), torch.from_numpy(golden["weights"])
+    hd = hidden.to(gpu).requires_grad_(True)
+    wd = head.to(gpu).requires_grad_(True)
+    for compaction in (False, True):
+        hd.grad = wd.grad = None
+        nll, weight_sum = ct.pallas_cut_linear_cross_entropy(hd, wd, targets.to(gpu), weights.to(gpu), mesh=None,
+                                                             sparse_compaction=compaction)
+        (nll * 0.37 + weight_sum * 0.0).backward()
+        assert float(nll) == pytest.approx(float(golden["nll_sum"]), rel=2e-5, abs=2e-3)
+        assert float(weight_sum) == float(golden["weight_sum"])
+        expected_dh = torch.from_numpy(golden["dhidden"]).view(torch.bfloat16).reshape(hidden.shape)
+        expected_dw = torch.from_numpy(golden["dhead"]).view(torch.bfloat16)
+        assert relative_l2(hd.grad.cpu(), expected_dh) < GRAD_RTOL
+        assert relative_l2(wd.grad.cpu(), expected_dw) < GRAD_RTOL
+        assert (hd.grad.cpu()[weights == 0] == 0).all()
+    # frozen head: no head gradient is produced at all (reference :645-667)
+    hd.grad = wd.grad = None
+    nll, _ = ct.pallas_cut_linear_cross_entropy(hd, wd, targets.to(gpu), weights.to(gpu), mesh=None,
+                                                lm_head_trainable=False)
+    nll.backward()
+    assert wd.grad is None and hd.grad is not None
+    with pytest.raises(ValueError, match="fsdp=ep=1"):
+        ct.pallas_cut_linear_cross_entropy(hd, wd, targets.to(gpu), weights.to(gpu), mesh={"fsdp": 2})
+
+
+def test_closed_form_uniform_logits(ct, gpu):
+    # zero hidden => nll = sum(w) log V (reference: tests/training/test_losses.py:125-252)
+    rows, vocab = 300, 1000
+    hidden = torch.zeros((rows, 128), dtype=torch.bfloat16)
+    head = _bf16(np.random.default_rng(0).normal(size=(128, vocab)))
+    weights = torch.from_numpy(np.random.default_rng(1).choice([0.0, 0.25, 1.0], size=rows).astype(np.float32))
+    targets = torch.arange(rows, dtype=torch.int32) % vocab
+    nll, weight_sum, lse, dhidden, _ = _gpu(ct, gpu, hidden, head, targets, weights, 1.0, compaction=True)
+    assert nll == pytest.approx(float(weights.sum()) * np.log(vocab), rel=1e-6)
+    assert weight_sum == float(weights.sum())
+    assert float((lse[weights != 0] - np.log(vocab)).abs().max()) < 1e-5
+
+
+def test_benchmark_shape(ct, gpu):
+    """N=16384, d=4096, V=128256, 30% ignored: oracle on samples + size-independent properties."""
+
+    W = ct.workloads
+    config = W.CUTCE_CONFIGS["llama3_8b_head"]
+    inputs = W.make_cutce_inputs(config)
+    hidden, head, targets, weights = (inputs[n] for n in ("hidden", "head", "targets", "weights"))
+    active = int((weights != 0).sum())
+    dy = 1.0 / active
+    print("shape", config, "active", active, flush=True)
+    nll, weight_sum, lse, dhidden, dhead = _gpu(ct, gpu, hidden, head, targets, weights, dy, compaction=True)
+    assert weight_sum == float(active)
+    ignored = weights == 0
+    assert (lse[ignored] == 0).all() and (lse[~ignored] != 0).all()
+    assert (dhidden[ignored] == 0).all()
+    assert torch.isfinite(dhidden.float()).all() and torch.isfinite(dhead.float()).all()
+
+    # rows: oracle on a sample of 512 rows (full vocabulary)
+    rng = np.random.default_rng(0)
+    sample = torch.from_numpy(np.sort(rng.choice(config.rows, size=512, replace=False)))
+    head_f32 = head.float()
+    logits = hidden[sample].float() @ head_f32
+    lse_ref = torch.where(weights[sample] != 0, torch.logsumexp(logits, -1), 0.0)
+    assert float((lse[sample] - lse_ref).abs().max()) <= LSE_ATOL
+    dh_ref, _ = ref.cut_backward(hidden[sample], head, targets[sample], weights[sample], lse_ref, dy,
+                                 head_trainable=False)
+    assert relative_l2(dhidden[sample], dh_ref) <= GRAD_RTOL
+
+    # scalar loss: f64 sum of per-row losses with the device lse (verified on the sample above)
+    # and target logits recomputed on the host for every active row
+    rows = torch.nonzero(~ignored).flatten()
+    target_logit = (hidden[rows].float() * head_f32[:, targets[rows].long()].T).sum(-1).double()
+    nll_ref = float(((lse[rows].double() - target_logit) * weights[rows].double()).sum())
+    assert nll == pytest.approx(nll_ref, rel=LOSS_RTOL)
+
+    # columns: dHead on 256 sampled vocabulary columns, G rebuilt on the host from the device lse
+    cols = torch.from_numpy(np.sort(rng.choice(config.vocab, size=256, replace=False)))
+    col_logits = hidden.float() @ head_f32[:, cols]
+    prob = torch.where(~ignored[:, None], torch.exp(col_logits - lse[:, None]), 0.0)
+    onehot = (targets[:, None].long() == cols[None, :]) & ~ignored[:, None]
+    g = ((weights * dy)[:, None] * (prob - onehot.float())).to(torch.bfloat16).float()
+    dw_ref = hidden.float().T @ g
+    assert relative_l2(dhead[:, cols], dw_ref) <= GRAD_RTOL

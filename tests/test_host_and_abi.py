@@ -1,0 +1,144 @@
+"""CPU-only checks of the host-side mirror and of the C ABI surface (no compute calls)."""
+
+import ctypes
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def test_library_exports_every_declared_symbol(ct):
+    header = (ROOT / "include" / "ct_hotpath.h").read_text()
+    declared = set(re.findall(r"\b(ct_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(ct._lib.SYMBOLS), declared ^ set(ct._lib.SYMBOLS)
+    library = ct._lib.load()
+    for name in declared:
+        assert hasattr(library, name), name
+    assert library.ct_abi_version() == ct._lib.ABI_VERSION
+    assert library.ct_last_error() == b"" or isinstance(library.ct_last_error(), bytes)
+
+
+def test_size_queries_need_no_gpu(ct):
+    library = ct._lib.load()
+    assert library.ct_attn_meta_bytes(4, 4096) == 4 * (4096 // 32) * 12 * 4
+    assert library.ct_attn_meta_bytes(0, 128) == 0
+    shape = ct._lib.CutceShape(16384, 4096, 128256)
+    fwd = library.ct_cutce_fwd_workspace_bytes(ctypes.byref(shape))
+    full = library.ct_cutce_bwd_workspace_bytes(ctypes.byref(shape))
+    least = library.ct_cutce_bwd_workspace_min_bytes(ctypes.byref(shape))
+    assert 0 < fwd < 64 << 20
+    assert full >= 16384 * 128256 * 2
+    assert 0 < least < full
+
+
+def test_argument_validation_happens_before_any_launch(ct):
+    library = ct._lib.load()
+    args = ct._lib.AttnFwdArgs(batch=1, seq=100, q_heads=4, kv_heads=2, head_dim=128, scale=0.1)
+    assert library.ct_attn_fwd(None, ctypes.byref(args)) == ct._lib.CT_INVALID_ARGUMENT
+    assert b"null pointer" in library.ct_last_error()
+    for field in ("q", "k", "v", "segment_ids", "tile_meta", "out", "lse"):
+        setattr(args, field, 4096)       # never dereferenced: validation fails first
+    assert library.ct_attn_fwd(None, ctypes.byref(args)) == ct._lib.CT_INVALID_ARGUMENT
+    assert b"128-aligned" in library.ct_last_error()
+    args.seq, args.q_heads, args.kv_heads = 128, 5, 2
+    assert library.ct_attn_fwd(None, ctypes.byref(args)) == ct._lib.CT_INVALID_ARGUMENT
+    assert b"divisible by the KV head count" in library.ct_last_error()
+    args.q_heads, args.head_dim = 4, 96
+    assert library.ct_attn_fwd(None, ctypes.byref(args)) == ct._lib.CT_UNSUPPORTED
+    shape = ct._lib.CutceShape(10, 100, 50)
+    cargs = ct._lib.CutceFwdArgs(shape=shape)
+    for field in ("hidden", "head", "targets", "weights", "nll_sum", "weight_sum", "lse", "workspace"):
+        setattr(cargs, field, 4096)
+    assert library.ct_cutce_fwd(None, ctypes.byref(cargs)) == ct._lib.CT_INVALID_ARGUMENT
+    assert b"divisible by 128" in library.ct_last_error()
+    cargs.shape = ct._lib.CutceShape(10, 128, 50)
+    cargs.workspace_bytes = 16
+    assert library.ct_cutce_fwd(None, ctypes.byref(cargs)) == ct._lib.CT_WORKSPACE_TOO_SMALL
+
+
+def test_profile_resolution_matches_reference_tiers(ct):
+    # tests/kernels/test_efficient_attention.py:226-249: S=4096, 32 heads, tp=4 -> h8, q256, kv 512/256
+    profile = ct.resolve_attention_profile((4, 4096, 32, 128), (4, 4096, 1, 128), {"tp": 4})
+    assert (profile.block_h, profile.block_q, profile.block_kv_outer, profile.block_kv_compute) == (8, 256, 512, 256)
+    long_profile = ct.resolve_attention_profile((1, 32768, 64, 128), (1, 32768, 8, 128), None)
+    assert (long_profile.block_kv_outer, long_profile.block_kv_compute) == (1024, 256)
+    hybrid = ct.resolve_attention_profile((2, 8192, 16, 128), (2, 8192, 16, 128), None, has_attention_end=True)
+    assert hybrid.block_h * hybrid.block_q <= 2048 and hybrid.block_q % 128 == 0
+    assert ct.default_attention_scale(128) == 128 ** -0.5
+    with pytest.raises(ValueError, match="128-aligned"):
+        ct.resolve_attention_profile((1, 100, 2, 128), (1, 100, 1, 128), None)
+    with pytest.raises(ValueError, match="divisible by the KV head count"):
+        ct.resolve_attention_profile((1, 128, 3, 128), (1, 128, 2, 128), None)
+
+
+def test_attention_argument_errors(ct):
+    q = torch.zeros((1, 128, 2, 128), dtype=torch.bfloat16)
+    k = torch.zeros((1, 128, 1, 128), dtype=torch.bfloat16)
+    meta = ct.AttentionMetadata(*(torch.zeros((1, 128), dtype=torch.int32),) * 2,
+                                torch.zeros((1, 1, 2), dtype=torch.int32),
+                                torch.zeros((1, 1, 2), dtype=torch.int32))
+    # tests/kernels/test_efficient_attention.py:420-441: non-causal is rejected
+    with pytest.raises(ValueError, match="implements causal attention only"):
+        ct.efficient_attention(q, k, k, meta, causal=False)
+    with pytest.raises(TypeError, match="compile-time bool"):
+        ct.efficient_attention(q, k, k, meta, causal=1)
+    with pytest.raises(TypeError, match="requires BF16"):
+        ct.efficient_attention(q.float(), k.float(), k.float(), meta)
+    with pytest.raises(ValueError, match="key and value shapes differ"):
+        ct.efficient_attention(q, k, k[:, :64], meta)
+    with pytest.raises(ValueError, match="head_dim"):
+        ct.efficient_attention(q[..., :32], k[..., :32], k[..., :32], meta)
+    with pytest.raises(ValueError, match="one GPU"):
+        ct.efficient_attention(q, k, k, meta, mesh={"tp": 2})
+    with pytest.raises(RuntimeError, match="only on a ROCm GPU"):
+        ct.efficient_attention(q, k, k, meta)
+
+
+def test_cutce_argument_errors(ct):
+    fn = ct.pallas_cut_linear_cross_entropy
+    hidden = torch.zeros((1, 4, 128), dtype=torch.bfloat16)
+    head = torch.zeros((128, 10), dtype=torch.bfloat16)
+    targets = torch.zeros((1, 4), dtype=torch.int32)
+    weights = torch.ones((1, 4))
+    with pytest.raises(ValueError, match=r"\[batch, sequence, hidden\]"):
+        fn(hidden[0], head, targets, weights)
+    with pytest.raises(ValueError, match=r"\[hidden, vocab\]"):
+        fn(hidden, head.T, targets, weights)
+    with pytest.raises(ValueError, match="must match hidden_states"):
+        fn(hidden, head, targets[:, :2], weights)
+    with pytest.raises(ValueError, match="divisible by 128"):
+        fn(hidden[..., :100], head[:100], targets, weights)
+    with pytest.raises(TypeError, match="same compute dtype"):
+        fn(hidden, head.float(), targets, weights)
+    with pytest.raises(TypeError, match="non-negative integer"):
+        fn(hidden, head, targets, weights, local_chunk_size=True)
+    with pytest.raises(ValueError, match="non-negative"):
+        fn(hidden, head, targets, weights, local_chunk_size=-1)
+    with pytest.raises(RuntimeError, match="only on a ROCm GPU"):
+        fn(hidden, head, targets, weights)
+
+
+def test_workload_generators_and_flop_accounting(ct):
+    from oracle import attention_ref
+
+    W = ct.workloads
+    config = W.ATTENTION_CONFIGS["packed_small"]
+    inputs = W.make_attention_inputs(config)
+    ids = inputs["segment_ids"].numpy()
+    assert ids.shape == (2, 1024) and inputs["q"].shape == (2, 1024, 8, 64)
+    np.testing.assert_array_equal(attention_ref.canonicalize_segment_ids(ids != 0, ids), ids)
+    pairs = W.count_allowed_pairs(ids)
+    assert pairs == attention_ref.count_allowed_pairs(ids)
+    assert W.attention_flops(config, pairs)["total"] == 14 * 64 * 8 * pairs
+    rng = np.random.default_rng(0)
+    seg, end = W.maskgit_layout(rng, 1, 4096)
+    assert W.count_allowed_pairs(seg, end) == attention_ref.count_allowed_pairs(seg, end)
+    blocks = np.flatnonzero(end[0] != np.arange(4096))
+    assert len(blocks) % 1055 == 0 and len(blocks) > 0  # the last token of a block keeps end == itself
+    cfg = W.CUTCE_CONFIGS["llama3_8b_head"]
+    assert W.cutce_flops(cfg, 16384)["total"] == 6 * 16384 * 4096 * 128256
+    assert W.attention_delta_bytes(W.ATTENTION_CONFIGS["llama3_8b"]) == 2 * 4 * 4096 * 32 * 128 * 2 + 4 * 4 * 4096 * 32
