@@ -1,0 +1,248 @@
+#!/usr/bin/env python3
+"""Benchmark of the two hot paths on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one forward + backward of packed GQA attention at the Llama-3-8B shape
+(B=4, S=4096, Hq=32, Hkv=8, D=128, log-uniform packed segments) on synthetic inputs already
+resident in HBM. The headline value is mask-aware TFLOP/s over K steps: 14 * D * Hq * pairs
+FLOPs per step, pairs = exact number of allowed (query, key) pairs. The same JSON line carries
+the cut cross-entropy forward + backward at N=16384, d=4096, V=128256 (tokens/s), the roofline
+of the dominant kernel from stream events recorded around each kernel in the timed region, the
+HBM rate of the delta pass, and a CPU baseline: this repository's CPU restatement of the
+reference's pure path, timed on the host cores on a bounded sample.
+
+Exactly one JSON line is printed on stdout.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
+
+
+def parse_args():
+    parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=20)
+    parser.add_argument("--warmup", type=int, default=5)
+    parser.add_argument("--cutce-steps", type=int, default=None, help="default: min(steps, 5)")
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-cutce", action="store_true")
+    return parser.parse_args()
+
+
+def timed_region(torch, step, steps, warmup, timer_factory):
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    with timer_factory() as timer:
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - start
+    return elapsed, timer.durations_ms()
+
+
+def mean(values):
+    return sum(values) / len(values)
+
+
+def bench_attention(ct, torch, steps, warmup):
+    W = ct.workloads
+    config = W.ATTENTION_CONFIGS["llama3_8b"]
+    inputs = W.make_attention_inputs(config, "cuda")
+    pairs = W.count_allowed_pairs(inputs["segment_ids"], inputs["attention_end"])
+    flops = W.attention_flops(config, pairs)
+    profile = ct.resolve_attention_profile(inputs["q"].shape, inputs["k"].shape, None)
+    metadata = ct.prepare_attention_metadata(inputs["segment_ids"], mesh=None, profile=profile)
+    q, k, v, dout = inputs["q"], inputs["k"], inputs["v"], inputs["dout"]
+
+    def step():
+        out, lse = ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
+        ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=config.scale)
+
+    elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
+    ms_per_step = elapsed / steps * 1e3
+    per_kernel_flops = {
+        "attn_fwd_kernel": flops["fwd"],
+        # backward = 5 GEMMs: dQ owns S recompute share + dP share + dQ; counted as executed-free
+        # algorithmic split: dq kernel 4*D*Hq*pairs (dP, dQ), dkv kernel 6*D*Hq*pairs (S, dV, dK)
+        "attn_dq_kernel": 4 * config.head_dim * config.q_heads * pairs,
+        "attn_dkv_kernel": 6 * config.head_dim * config.q_heads * pairs,
+    }
+    table = []
+    for name, durations in kernels.items():
+        entry = {"kernel": name, "launches": len(durations), "avg_ms": mean(durations)}
+        if name in per_kernel_flops:
+            entry["algorithmic_tflops"] = per_kernel_flops[name] / (entry["avg_ms"] * 1e-3) / 1e12
+        if name == "attn_delta_kernel":
+            entry["algorithmic_gbps"] = W.attention_delta_bytes(config) / (entry["avg_ms"] * 1e-3) / 1e9
+        table.append(entry)
+    return {
+        "config": config, "pairs": pairs, "flops": flops, "ms_per_step": ms_per_step,
+        "tflops": flops["total"] / (ms_per_step * 1e-3) / 1e12, "kernels": table,
+        "inputs": inputs,
+    }
+
+
+def bench_cutce(ct, torch, steps, warmup):
+    W = ct.workloads
+    config = W.CUTCE_CONFIGS["llama3_8b_head"]
+    inputs = W.make_cutce_inputs(config, "cuda")
+    hidden, head, targets, weights = (inputs[n] for n in ("hidden", "head", "targets", "weights"))
+    active = int((weights != 0).sum())
+    flops = W.cutce_flops(config, active)
+    dy = torch.tensor(1.0 / max(active, 1))
+
+    state = {}
+
+    def step():
+        nll, weight_sum, lse = ct.cutce_forward(hidden, head, targets, weights, sparse_compaction=True)
+        ct.cutce_backward(hidden, head, targets, weights, lse, dy, sparse_compaction=True)
+        state["loss"] = (nll, weight_sum)
+
+    elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
+    ms_per_step = elapsed / steps * 1e3
+    gemm = 2 * active * config.hidden * config.vocab
+    per_kernel_flops = {"cutce_stats_kernel": gemm, "cutce_dhidden_kernel": gemm, "cutce_dhead_kernel": gemm}
+    table = []
+    for name, durations in kernels.items():
+        entry = {"kernel": name, "launches": len(durations), "avg_ms": mean(durations)}
+        if name in per_kernel_flops:
+            entry["algorithmic_tflops"] = per_kernel_flops[name] / (entry["avg_ms"] * 1e-3) / 1e12
+        table.append(entry)
+    nll, weight_sum = state["loss"]
+    return {
+        "workload": "cut-CE fwd+bwd N=16384 d=4096 V=128256 bf16, 30% ignored, head [d, V], compaction on",
+        "active_rows": active,
+        "ms_per_step": ms_per_step,
+        "tokens_per_s": config.rows / (ms_per_step * 1e-3),
+        "mask_aware_tflops": flops["total"] / (ms_per_step * 1e-3) / 1e12,
+        "mfma_frac_mask_aware": flops["total"] / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        "dense_flops": flops["dense_total"], "mask_aware_flops": flops["total"],
+        "mean_loss": float(nll) / max(float(weight_sum), 1.0),
+        "steps": steps,
+        "kernels": table,
+    }
+
+
+def cpu_baseline(ct, torch, attention):
+    """The oracle (a port of the reference's pure JAX path) on the host cores, bounded sample."""
+
+    from oracle import attention_ref
+
+    config = attention["config"]
+    inputs = attention["inputs"]
+    group = config.q_heads // config.kv_heads
+    budget_s, flops, pairs, elapsed, slices = 12.0, 0, 0, 0.0, 0
+    for b in range(config.batch):
+        ids = inputs["segment_ids"][b:b + 1].cpu().numpy()
+        allowed = attention_ref.allowed_from_canonical(ids)
+        for kvh in range(config.kv_heads):
+            heads = slice(kvh * group, (kvh + 1) * group)
+            q = inputs["q"][b:b + 1, :, heads].cpu()
+            k = inputs["k"][b:b + 1, :, kvh:kvh + 1].cpu()
+            v = inputs["v"][b:b + 1, :, kvh:kvh + 1].cpu()
+            dout = inputs["dout"][b:b + 1, :, heads].cpu()
+            start = time.perf_counter()
+            attention_ref.vanilla_attention_vjp(q, k, v, allowed, dout, scale=config.scale)
+            elapsed += time.perf_counter() - start
+            slices += 1
+            pairs += int(allowed.sum())
+            flops += 14 * config.head_dim * group * int(allowed.sum())
+            if elapsed >= budget_s:
+                break
+        if elapsed >= budget_s:
+            break
+    return {
+        "value": flops / elapsed / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": (f"{slices} (batch row, KV head) slices of the same workload, each one KV head with its "
+                   f"{group} query heads at S={config.seq} ({pairs} allowed pairs in all), vanilla attention "
+                   f"fwd + autograd bwd, {elapsed:.2f} s on {torch.get_num_threads()} threads of "
+                   f"{os.cpu_count()} logical CPUs"),
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported in this build "
+              "(nothing here uses a second GPU).", file=sys.stderr)
+        return 2
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    import torch
+
+    import causal_trainer_dev_amd as ct
+    from causal_trainer_dev_amd import profiling  # noqa: F401  (ct.profiling)
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    ct._lib.load()
+
+    attention = bench_attention(ct, torch, args.steps, args.warmup)
+    config = attention["config"]
+    dominant = max((k for k in attention["kernels"] if "algorithmic_tflops" in k),
+                   key=lambda k: k["avg_ms"] * k["launches"])
+    delta = next((k for k in attention["kernels"] if k["kernel"] == "attn_delta_kernel"), None)
+    result = {
+        "metric": "attn fwd+bwd TFLOP/s (mask-aware), Llama-3-8B shape",
+        "value": attention["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": attention["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": ("packed GQA attention fwd+bwd, Llama-3-8B shape: B=4 S=4096 Hq=32 Hkv=8 D=128 bf16, "
+                         "segment lengths log-uniform [64,4096], tail padding, scale 128^-0.5"),
+            "allowed_pairs": attention["pairs"],
+            "flops_per_step": attention["flops"]["total"],
+            "seed": config.seed,
+        },
+        "pct_bf16_mfma_peak": 100.0 * attention["tflops"] / PEAK_BF16_TFLOPS,
+        "roofline": {
+            "bound": "mfma",
+            "kernel": dominant["kernel"],
+            "achieved": dominant["algorithmic_tflops"],
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": dominant["algorithmic_tflops"] / PEAK_BF16_TFLOPS,
+            "avg_launch_ms": dominant["avg_ms"],
+            "traffic": None,
+        },
+        "kernels": attention["kernels"],
+    }
+    if delta is not None:
+        result["delta_pass"] = {
+            "bound": "hbm", "achieved": delta["algorithmic_gbps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+            "frac": delta["algorithmic_gbps"] / PEAK_HBM_GBPS, "avg_launch_ms": delta["avg_ms"],
+        }
+    if not args.no_cutce:
+        cut_steps = args.cutce_steps or min(args.steps, 5)
+        result["cutce"] = bench_cutce(ct, torch, cut_steps, min(args.warmup, 2))
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(ct, torch, attention)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

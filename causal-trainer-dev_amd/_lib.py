@@ -75,8 +75,11 @@ class CutceBwdArgs(Structure):
     ]
 
 
+LAUNCH_HOOK = ctypes.CFUNCTYPE(None, c_void_p, ctypes.c_char_p, c_int32, c_void_p)
+
 # name -> (restype, argtypes); every symbol include/ct_hotpath.h declares.
 SYMBOLS = {
+    "ct_set_launch_hook": (None, [LAUNCH_HOOK, c_void_p]),
     "ct_last_error": (ctypes.c_char_p, []),
     "ct_abi_version": (c_int32, []),
     "ct_attn_meta_bytes": (c_size_t, [c_int32, c_int32]),

@@ -142,16 +142,15 @@ template <int D, int HS>
 static int launch_fwd(hipStream_t stream, const AttnParams& p) {
   constexpr int PB = 4 / HS;
   const size_t smem = KvSmem<D>::kBytes;
-  static bool configured = false;
-  if (!configured) {
+  {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, HS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_fwd: %s", hipGetErrorString(e));
-    configured = true;
   }
   const int grid = (p.S / (32 * PB)) * (p.Hq / HS) * p.B;
+  LaunchScope scope1("attn_fwd_kernel", stream);
   hipLaunchKernelGGL((attn_fwd_kernel<D, HS>), dim3(grid), dim3(256), smem, stream, p);
-  return check_launch("ct_attn_fwd");
+  return scope1.done();
 }
 
 template <int D>
@@ -167,40 +166,44 @@ template <int D, int HS>
 static int launch_dq(hipStream_t stream, const AttnParams& p) {
   constexpr int PB = 4 / HS;
   const size_t smem = KvSmem<D>::kBytes;
-  static bool configured = false;
-  if (!configured) {
+  {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dq_kernel<D, HS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
-    configured = true;
   }
   const int grid = (p.S / (32 * PB)) * (p.Hq / HS) * p.B;
+  LaunchScope scope2("attn_dq_kernel", stream);
   hipLaunchKernelGGL((attn_dq_kernel<D, HS>), dim3(grid), dim3(256), smem, stream, p);
-  return check_launch("ct_attn_bwd (dq)");
+  return scope2.done();
 }
 
 template <int D>
 static int launch_dkv(hipStream_t stream, const AttnParams& p) {
   const size_t smem = DkvSmem<D>::kBytes;
-  static bool configured = false;
-  if (!configured) {
+  {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dkv_kernel<D>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
-    configured = true;
   }
   const int grid = (p.S / 128) * p.Hkv * p.B;
+  LaunchScope scope3("attn_dkv_kernel", stream);
   hipLaunchKernelGGL((attn_dkv_kernel<D>), dim3(grid), dim3(256), smem, stream, p);
-  return check_launch("ct_attn_bwd (dkv)");
+  return scope3.done();
+}
+
+template <int D>
+static int launch_delta(hipStream_t stream, const bf16* out, const bf16* dout, float* delta,
+                        long rows) {
+  const long threads = rows * (D / 8);
+  LaunchScope scope4("attn_delta_kernel", stream);
+  hipLaunchKernelGGL((attn_delta_kernel<D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
+                     stream, out, dout, delta, rows);
+  return scope4.done();
 }
 
 template <int D>
 static int dispatch_bwd(hipStream_t stream, const AttnParams& p) {
-  const long rows = (long)p.B * p.S * p.Hq;
-  const long threads = rows * (D / 8);
-  hipLaunchKernelGGL((attn_delta_kernel<D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
-                     stream, p.out, p.dout, p.delta, rows);
-  int rc = check_launch("ct_attn_bwd (delta)");
+  int rc = launch_delta<D>(stream, p.out, p.dout, p.delta, (long)p.B * p.S * p.Hq);
   if (rc) return rc;
   switch (heads_per_group(p.Hq, p.Hkv)) {
     case 4: rc = launch_dq<D, 4>(stream, p); break;
@@ -228,17 +231,16 @@ extern "C" int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
   if (rc) return rc;
   const int nrb = seq / 32;
   const size_t smem = (size_t)nrb * 3 * sizeof(int);
-  static bool configured = false;
-  if (!configured) {
+  {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prepare_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 8192 * 3 * 4);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_prepare: %s", hipGetErrorString(e));
-    configured = true;
   }
   const int threads = nrb >= 1024 ? 1024 : ((nrb + 63) / 64) * 64;
+  LaunchScope scope5("attn_prepare_kernel", (hipStream_t)stream);
   hipLaunchKernelGGL(attn_prepare_kernel, dim3(batch), dim3(threads), smem, (hipStream_t)stream,
                      segment_ids, attention_end, seq, tile_meta);
-  return check_launch("ct_attn_prepare");
+  return scope5.done();
 }
 
 extern "C" int32_t ct_attn_block_summary(void* stream, const int32_t* segment_ids,
@@ -249,10 +251,11 @@ extern "C" int32_t ct_attn_block_summary(void* stream, const int32_t* segment_id
   CT_REQUIRE(seq % block == 0, "ct_attn_block_summary: sequence %d not divisible by block %d", seq,
              block);
   const int nblocks = batch * (seq / block);
+  LaunchScope scope6("attn_block_summary_kernel", (hipStream_t)stream);
   hipLaunchKernelGGL(attn_block_summary_kernel, dim3((nblocks + 127) / 128), dim3(128), 0,
                      (hipStream_t)stream, segment_ids, attention_end, seq, block, nblocks,
                      attention_end ? 3 : 2, out);
-  return check_launch("ct_attn_block_summary");
+  return scope6.done();
 }
 
 extern "C" int32_t ct_attn_fwd(void* stream, const ct_attn_fwd_args* a) {
@@ -286,17 +289,10 @@ extern "C" int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16
   CT_REQUIRE(rows > 0, "ct_attn_delta: rows must be positive");
   if (head_dim != 64 && head_dim != 128)
     return fail(CT_UNSUPPORTED, "ct_attn_delta: head_dim must be 64 or 128, got %d", head_dim);
-  const long threads = rows * (head_dim / 8);
-  const dim3 grid((unsigned)((threads + 255) / 256));
-  if (head_dim == 128)
-    hipLaunchKernelGGL((attn_delta_kernel<128>), grid, dim3(256), 0, (hipStream_t)stream,
-                       reinterpret_cast<const bf16*>(out), reinterpret_cast<const bf16*>(dout),
-                       delta, (long)rows);
-  else
-    hipLaunchKernelGGL((attn_delta_kernel<64>), grid, dim3(256), 0, (hipStream_t)stream,
-                       reinterpret_cast<const bf16*>(out), reinterpret_cast<const bf16*>(dout),
-                       delta, (long)rows);
-  return check_launch("ct_attn_delta");
+  const bf16* o = reinterpret_cast<const bf16*>(out);
+  const bf16* g = reinterpret_cast<const bf16*>(dout);
+  return head_dim == 128 ? launch_delta<128>((hipStream_t)stream, o, g, delta, (long)rows)
+                         : launch_delta<64>((hipStream_t)stream, o, g, delta, (long)rows);
 }
 
 extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {

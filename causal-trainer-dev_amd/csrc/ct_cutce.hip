@@ -574,22 +574,26 @@ extern "C" int32_t ct_cutce_fwd(void* stream_, const ct_cutce_fwd_args* a) {
   const int chunks = stats_chunks(p.V);
   const int row_blocks = p.n_pad / kGemmTile;
 
+  LaunchScope scope1("cutce_index_kernel", stream);
   hipLaunchKernelGGL(cutce_index_kernel, dim3(1), dim3(1024), 0, stream, p.weights, p.N, p.n_pad,
                      a->sparse_compaction ? 1 : 0, p.idx, p.header);
-  if ((rc = check_launch("ct_cutce_fwd (index)"))) return rc;
+  if ((rc = scope1.done())) return rc;
 
   const size_t smem = GemmSmem<kBK>::kBytes;
   if ((rc = set_smem(cutce_stats_kernel, smem, "ct_cutce_fwd"))) return rc;
   const int persistent = min(device_cu_count(), chunks * row_blocks);
+  LaunchScope scope2("cutce_stats_kernel", stream);
   hipLaunchKernelGGL(cutce_stats_kernel, dim3(persistent), dim3(256), smem, stream, p, part, chunks);
-  if ((rc = check_launch("ct_cutce_fwd (stats)"))) return rc;
+  if ((rc = scope2.done())) return rc;
 
+  LaunchScope scope3("cutce_merge_kernel", stream);
   hipLaunchKernelGGL(cutce_merge_kernel, dim3(row_blocks), dim3(256), 0, stream, p, part, chunks,
                      a->lse, sums);
-  if ((rc = check_launch("ct_cutce_fwd (merge)"))) return rc;
+  if ((rc = scope3.done())) return rc;
+  LaunchScope scope4("cutce_finalize_kernel", stream);
   hipLaunchKernelGGL(cutce_finalize_kernel, dim3(1), dim3(64), 0, stream, sums, row_blocks,
                      a->nll_sum, a->weight_sum);
-  return check_launch("ct_cutce_fwd (finalize)");
+  return scope4.done();
 }
 
 extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
@@ -619,12 +623,14 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
   if ((rc = set_smem(cutce_dhidden_kernel, smem, "ct_cutce_bwd"))) return rc;
   if ((rc = set_smem(cutce_dhead_kernel, smem, "ct_cutce_bwd"))) return rc;
 
+  LaunchScope scope5("cutce_index_kernel", stream);
   hipLaunchKernelGGL(cutce_index_kernel, dim3(1), dim3(1024), 0, stream, p.weights, p.N, p.n_pad,
                      a->sparse_compaction ? 1 : 0, p.idx, p.header);
-  if ((rc = check_launch("ct_cutce_bwd (index)"))) return rc;
+  if ((rc = scope5.done())) return rc;
+  LaunchScope scope6("cutce_zero_rows_kernel", stream);
   hipLaunchKernelGGL(cutce_zero_rows_kernel, dim3(p.N), dim3(256), 0, stream, p.weights, p.N, p.d,
                      dhidden);
-  if ((rc = check_launch("ct_cutce_bwd (zero rows)"))) return rc;
+  if ((rc = scope6.done())) return rc;
 
   const int tiles = vocab_tile_count(p.V);
   const int tiles_per_slab = L.slab_cols / kGemmTile;
@@ -632,17 +638,20 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
     const int slab0 = s * L.slab_cols;
     const int slab_tiles = min(tiles_per_slab, tiles - s * tiles_per_slab);
     const int slab_width = slab_tiles * kGemmTile;
+    LaunchScope scope7("cutce_dlogits_kernel", stream);
     hipLaunchKernelGGL(cutce_dlogits_kernel, dim3(slab_tiles * row_blocks), dim3(256), smem, stream,
                        p, a->lse, a->dy, slab0, slab_tiles, G, ldg);
-    if ((rc = check_launch("ct_cutce_bwd (dlogits)"))) return rc;
+    if ((rc = scope7.done())) return rc;
     const int mode = L.slabs == 1 ? 0 : (s == 0 ? 1 : (s == L.slabs - 1 ? 3 : 2));
+    LaunchScope scope8("cutce_dhidden_kernel", stream);
     hipLaunchKernelGGL(cutce_dhidden_kernel, dim3(row_blocks * ((p.d + kGemmTile - 1) / kGemmTile)), dim3(256), smem,
                        stream, p, G, ldg, slab0, slab_width, mode, dh_acc, dhidden);
-    if ((rc = check_launch("ct_cutce_bwd (dhidden)"))) return rc;
+    if ((rc = scope8.done())) return rc;
     if (dhead) {
+      LaunchScope scope9("cutce_dhead_kernel", stream);
       hipLaunchKernelGGL(cutce_dhead_kernel, dim3(((p.d + kGemmTile - 1) / kGemmTile) * slab_tiles), dim3(256), smem,
                          stream, p, G, ldg, slab0, slab_tiles, dhead);
-      if ((rc = check_launch("ct_cutce_bwd (dhead)"))) return rc;
+      if ((rc = scope9.done())) return rc;
     }
   }
   return CT_OK;

@@ -1,0 +1,51 @@
+"""Per-kernel timing with stream events, through the library's launch hook.
+
+``KernelTimer`` brackets every kernel the C ABI launches on the calling thread
+with a pair of events recorded on the launch stream, so durations are those of
+the individual kernels, measured in the same run and on the same stream as the
+work being timed.
+"""
+
+from __future__ import annotations
+
+import collections
+import ctypes
+
+import torch
+
+from . import _lib
+
+
+class KernelTimer:
+    """Context manager: collects (kernel name -> list of durations in ms)."""
+
+    def __init__(self):
+        self._pending = []
+        self._open = {}
+        self._callback = _lib.LAUNCH_HOOK(self._on_launch)
+
+    def _on_launch(self, _user, kernel, phase, stream):
+        name = kernel.decode()
+        event = torch.cuda.Event(enable_timing=True)
+        event.record(torch.cuda.ExternalStream(stream) if stream else torch.cuda.current_stream())
+        if phase == 0:
+            self._open[name] = event
+        else:
+            self._pending.append((name, self._open.pop(name), event))
+
+    def __enter__(self):
+        _lib.load().ct_set_launch_hook(self._callback, None)
+        return self
+
+    def __exit__(self, *exc):
+        _lib.load().ct_set_launch_hook(ctypes.cast(None, _lib.LAUNCH_HOOK), None)
+        return False
+
+    def durations_ms(self) -> dict[str, list[float]]:
+        """Synchronises and returns every recorded launch, grouped by kernel name."""
+
+        torch.cuda.synchronize()
+        result = collections.defaultdict(list)
+        for name, begin, end in self._pending:
+            result[name].append(begin.elapsed_time(end))
+        return dict(result)

@@ -46,6 +46,17 @@ const char* ct_last_error(void);
 /* Library ABI version (bumped on any signature change). */
 int32_t ct_abi_version(void);
 
+/*
+ * Measurement hook, no counterpart in the reference. When set (per calling
+ * thread), every kernel launch made by an entry point on that thread is
+ * bracketed by hook(user, kernel_name, 0, stream) and hook(user, kernel_name,
+ * 1, stream), called on the host, so a harness can record stream events
+ * around individual kernels. NULL removes it. The hook must not call back
+ * into this library.
+ */
+typedef void (*ct_launch_hook)(void* user, const char* kernel, int32_t phase, void* stream);
+void ct_set_launch_hook(ct_launch_hook hook, void* user);
+
 /* ------------------------------------------------------------------------
  * Attention
  * --------------------------------------------------------------------- */
