@@ -1,0 +1,229 @@
+// XLA FFI handlers: a thin second entry into the C ABI of ct_hotpath.h.
+//
+// Built only where jaxlib's headers exist (jax.ffi.include_dir()); nothing in
+// libct_hotpath.so depends on this file:
+//   hipcc -O2 -fPIC -shared -std=c++17 -D__HIP_PLATFORM_AMD__ \
+//         -I$(python -c "import jax.ffi; print(jax.ffi.include_dir())") \
+//         -Iinclude causal-trainer-dev_amd/csrc/ct_ffi.cc \
+//         -Lcausal-trainer-dev_amd -lct_hotpath -o causal-trainer-dev_amd/libct_ffi.so
+// Every handler unpacks buffers, attributes and the platform stream and calls
+// the C ABI; scratch memory is requested from XLA as extra results, so the
+// handlers allocate nothing and are safe under command-buffer capture.
+#include <hip/hip_runtime.h>
+
+#include "ct_hotpath.h"
+#include "xla/ffi/api/ffi.h"
+
+namespace ffi = xla::ffi;
+
+namespace {
+
+ffi::Error status_to_error(int32_t status) {
+  if (status == CT_OK) return ffi::Error::Success();
+  const auto code = (status == CT_LAUNCH_FAILED) ? ffi::ErrorCode::kInternal
+                                                 : ffi::ErrorCode::kInvalidArgument;
+  return ffi::Error(code, ct_last_error());
+}
+
+template <typename T>
+const uint16_t* bits(const T& buffer) {
+  return reinterpret_cast<const uint16_t*>(buffer.untyped_data());
+}
+template <typename T>
+uint16_t* bits_out(T& buffer) {
+  return reinterpret_cast<uint16_t*>(buffer->untyped_data());
+}
+
+// segment ids / attention_end / tile bounds are int32 [B, S] (...); q is [B, S, Hq, D].
+ffi::Error AttnPrepare(hipStream_t stream, ffi::Buffer<ffi::S32> segment_ids,
+                       ffi::Buffer<ffi::S32> attention_end, ffi::ResultBuffer<ffi::S32> tile_meta,
+                       bool has_end) {
+  const auto dims = segment_ids.dimensions();
+  if (dims.size() != 2) return ffi::Error::InvalidArgument("segment_ids must be [batch, sequence]");
+  return status_to_error(ct_attn_prepare(stream, segment_ids.typed_data(),
+                                         has_end ? attention_end.typed_data() : nullptr,
+                                         (int32_t)dims[0], (int32_t)dims[1], tile_meta->typed_data()));
+}
+
+ffi::Error AttnFwd(hipStream_t stream, ffi::Buffer<ffi::BF16> q, ffi::Buffer<ffi::BF16> k,
+                   ffi::Buffer<ffi::BF16> v, ffi::Buffer<ffi::S32> segment_ids,
+                   ffi::Buffer<ffi::S32> attention_end, ffi::Buffer<ffi::S32> tile_meta,
+                   ffi::ResultBuffer<ffi::BF16> out, ffi::ResultBuffer<ffi::F32> lse, float scale,
+                   bool has_end) {
+  const auto qd = q.dimensions();
+  const auto kd = k.dimensions();
+  if (qd.size() != 4 || kd.size() != 4)
+    return ffi::Error::InvalidArgument("attention shapes must be [batch, sequence, heads, dim]");
+  ct_attn_fwd_args a = {};
+  a.q = bits(q);
+  a.k = bits(k);
+  a.v = bits(v);
+  a.segment_ids = segment_ids.typed_data();
+  a.attention_end = has_end ? attention_end.typed_data() : nullptr;
+  a.tile_meta = tile_meta.typed_data();
+  a.out = bits_out(out);
+  a.lse = lse->typed_data();
+  a.batch = (int32_t)qd[0];
+  a.seq = (int32_t)qd[1];
+  a.q_heads = (int32_t)qd[2];
+  a.kv_heads = (int32_t)kd[2];
+  a.head_dim = (int32_t)qd[3];
+  a.scale = scale;
+  return status_to_error(ct_attn_fwd(stream, &a));
+}
+
+ffi::Error AttnBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> q, ffi::Buffer<ffi::BF16> k,
+                   ffi::Buffer<ffi::BF16> v, ffi::Buffer<ffi::S32> segment_ids,
+                   ffi::Buffer<ffi::S32> attention_end, ffi::Buffer<ffi::S32> tile_meta,
+                   ffi::Buffer<ffi::BF16> out, ffi::Buffer<ffi::F32> lse,
+                   ffi::Buffer<ffi::BF16> dout, ffi::ResultBuffer<ffi::BF16> dq,
+                   ffi::ResultBuffer<ffi::BF16> dk, ffi::ResultBuffer<ffi::BF16> dv,
+                   ffi::ResultBuffer<ffi::F32> delta_scratch, float scale, bool has_end) {
+  const auto qd = q.dimensions();
+  const auto kd = k.dimensions();
+  if (qd.size() != 4 || kd.size() != 4)
+    return ffi::Error::InvalidArgument("attention shapes must be [batch, sequence, heads, dim]");
+  ct_attn_bwd_args a = {};
+  a.q = bits(q);
+  a.k = bits(k);
+  a.v = bits(v);
+  a.segment_ids = segment_ids.typed_data();
+  a.attention_end = has_end ? attention_end.typed_data() : nullptr;
+  a.tile_meta = tile_meta.typed_data();
+  a.out = bits(out);
+  a.lse = lse.typed_data();
+  a.dout = bits(dout);
+  a.dq = bits_out(dq);
+  a.dk = bits_out(dk);
+  a.dv = bits_out(dv);
+  a.delta = delta_scratch->typed_data();
+  a.batch = (int32_t)qd[0];
+  a.seq = (int32_t)qd[1];
+  a.q_heads = (int32_t)qd[2];
+  a.kv_heads = (int32_t)kd[2];
+  a.head_dim = (int32_t)qd[3];
+  a.scale = scale;
+  return status_to_error(ct_attn_bwd(stream, &a));
+}
+
+ct_cutce_shape cut_shape(const ffi::Buffer<ffi::BF16>& hidden, const ffi::Buffer<ffi::BF16>& head) {
+  ct_cutce_shape s;
+  s.rows = (int32_t)hidden.dimensions()[0];
+  s.hidden = (int32_t)hidden.dimensions()[1];
+  s.vocab = (int32_t)head.dimensions()[1];
+  return s;
+}
+
+ffi::Error CutceFwd(hipStream_t stream, ffi::Buffer<ffi::BF16> hidden, ffi::Buffer<ffi::BF16> head,
+                    ffi::Buffer<ffi::S32> targets, ffi::Buffer<ffi::F32> weights,
+                    ffi::ResultBuffer<ffi::F32> nll_sum, ffi::ResultBuffer<ffi::F32> weight_sum,
+                    ffi::ResultBuffer<ffi::F32> lse, ffi::ResultBuffer<ffi::U8> workspace,
+                    bool sparse_compaction) {
+  if (hidden.dimensions().size() != 2 || head.dimensions().size() != 2)
+    return ffi::Error::InvalidArgument("hidden must be [rows, hidden] and head [hidden, vocab]");
+  ct_cutce_fwd_args a = {};
+  a.hidden = bits(hidden);
+  a.head = bits(head);
+  a.targets = targets.typed_data();
+  a.weights = weights.typed_data();
+  a.nll_sum = nll_sum->typed_data();
+  a.weight_sum = weight_sum->typed_data();
+  a.lse = lse->typed_data();
+  a.workspace = workspace->untyped_data();
+  a.workspace_bytes = workspace->size_bytes();
+  a.shape = cut_shape(hidden, head);
+  a.sparse_compaction = sparse_compaction ? 1 : 0;
+  return status_to_error(ct_cutce_fwd(stream, &a));
+}
+
+ffi::Error CutceBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> hidden, ffi::Buffer<ffi::BF16> head,
+                    ffi::Buffer<ffi::S32> targets, ffi::Buffer<ffi::F32> weights,
+                    ffi::Buffer<ffi::F32> lse, ffi::Buffer<ffi::F32> dy,
+                    ffi::ResultBuffer<ffi::BF16> dhidden, ffi::ResultBuffer<ffi::BF16> dhead,
+                    ffi::ResultBuffer<ffi::U8> workspace, bool sparse_compaction,
+                    bool head_trainable) {
+  if (hidden.dimensions().size() != 2 || head.dimensions().size() != 2)
+    return ffi::Error::InvalidArgument("hidden must be [rows, hidden] and head [hidden, vocab]");
+  ct_cutce_bwd_args a = {};
+  a.hidden = bits(hidden);
+  a.head = bits(head);
+  a.targets = targets.typed_data();
+  a.weights = weights.typed_data();
+  a.lse = lse.typed_data();
+  a.dy = dy.typed_data();
+  a.dhidden = bits_out(dhidden);
+  a.dhead = head_trainable ? bits_out(dhead) : nullptr;  // frozen head: dHead never launched
+  a.workspace = workspace->untyped_data();
+  a.workspace_bytes = workspace->size_bytes();
+  a.shape = cut_shape(hidden, head);
+  a.sparse_compaction = sparse_compaction ? 1 : 0;
+  return status_to_error(ct_cutce_bwd(stream, &a));
+}
+
+}  // namespace
+
+#define CT_STREAM Ctx<ffi::PlatformStream<hipStream_t>>()
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_attn_prepare, AttnPrepare,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::S32>>()
+                                  .Attr<bool>("has_end"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_attn_fwd, AttnFwd,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Attr<float>("scale")
+                                  .Attr<bool>("has_end"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_attn_bwd, AttnBwd,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Attr<float>("scale")
+                                  .Attr<bool>("has_end"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_cutce_fwd, CutceFwd,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<bool>("sparse_compaction"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_cutce_bwd, CutceBwd,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<bool>("sparse_compaction")
+                                  .Attr<bool>("head_trainable"));
