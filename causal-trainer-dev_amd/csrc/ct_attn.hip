@@ -12,13 +12,14 @@ namespace ct {
 // 32-position block, phase 2 turns the summaries into visit ranges.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, const int* end, int S,
-                                                            int* meta) {
+                                                            int* meta, int* sched_all) {
   extern __shared__ int lds_meta[];  // [nrb][3]: min_nz, max_id, end_max
   const int b = blockIdx.x;
   const int nrb = S / 32, nt = S / kKeyTile;
   const int* segb = seg + (size_t)b * S;
   const int* endb = end ? end + (size_t)b * S : nullptr;
   int* mb = meta + (size_t)b * nrb * kMetaW;
+  int* sched = sched_all + (size_t)b * schedule_ints(nrb);
 
   for (int rb = threadIdx.x; rb < nrb; rb += blockDim.x) {
     int min_nz = INT_MAX, max_id = 0, end_min = INT_MAX, end_max = -1;
@@ -86,6 +87,58 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, cons
     m[kQFirst] = q_first;
     m[kQLast] = q_last;
   }
+  __threadfence_block();
+  __syncthreads();
+
+  // Phase 3: amount of work per tile, for the four schedules, into LDS (the
+  // summaries are no longer needed): [0, nrb) query tiles of 1 row block,
+  // then tiles of 2, of 4, then 128-key tiles.
+  int* work = lds_meta;
+  const int off2 = nrb, off4 = nrb + nrb / 2, offk = nrb + nrb / 2 + nrb / 4;
+  for (int i = threadIdx.x; i < nrb; i += blockDim.x) {
+    const int* m = mb + i * kMetaW;
+    work[i] = m[kKvLast] >= m[kKvFirst] ? m[kKvLast] - m[kKvFirst] + 1 : 0;
+  }
+  for (int pb = 2; pb <= 4; pb *= 2) {
+    int* dst = work + (pb == 2 ? off2 : off4);
+    for (int i = threadIdx.x; i < nrb / pb; i += blockDim.x) {
+      int first = INT_MAX, last = -1;
+      for (int k = 0; k < pb; ++k) {
+        const int* m = mb + (i * pb + k) * kMetaW;
+        first = min(first, m[kKvFirst]);
+        last = max(last, m[kKvLast]);
+      }
+      dst[i] = last >= first ? last - first + 1 : 0;
+    }
+  }
+  for (int i = threadIdx.x; i < nrb / 4; i += blockDim.x) {
+    int first = INT_MAX, last = -1;
+    for (int k = 0; k < 4; ++k) {
+      const int* m = mb + (i * 4 + k) * kMetaW;
+      first = min(first, m[kQFirst]);
+      last = max(last, m[kQLast]);
+    }
+    work[offk + i] = last >= first ? last - first + 1 : 0;
+  }
+  __syncthreads();
+
+  // Phase 4: rank sort (descending work, ties by index) -> schedules.
+  const int counts[4] = {nrb, nrb / 2, nrb / 4, nrb / 4};
+  const int offsets[4] = {0, off2, off4, offk};
+  for (int sidx = 0; sidx < 4; ++sidx) {
+    const int n = counts[sidx];
+    const int* wk = work + offsets[sidx];
+    int* out = sched + offsets[sidx];
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+      const int wi = wk[i];
+      int rank = 0;
+      for (int k = 0; k < n; ++k) {
+        const int wv = wk[k];
+        rank += (wv > wi) || (wv == wi && k < i);
+      }
+      out[rank] = i;
+    }
+  }
 }
 
 __global__ void attn_block_summary_kernel(const int* seg, const int* end, int S, int block,
@@ -141,7 +194,7 @@ static int heads_per_group(int Hq, int Hkv) {
 template <int D, int HS>
 static int launch_fwd(hipStream_t stream, const AttnParams& p) {
   constexpr int PB = 4 / HS;
-  const size_t smem = KvSmem<D>::kBytes;
+  const size_t smem = 2 * KvStage<D>::kBytes;
   {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, HS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -165,7 +218,7 @@ static int dispatch_fwd(hipStream_t stream, const AttnParams& p) {
 template <int D, int HS>
 static int launch_dq(hipStream_t stream, const AttnParams& p) {
   constexpr int PB = 4 / HS;
-  const size_t smem = KvSmem<D>::kBytes;
+  const size_t smem = 2 * KvStage<D>::kBytes;
   {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dq_kernel<D, HS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -179,13 +232,13 @@ static int launch_dq(hipStream_t stream, const AttnParams& p) {
 
 template <int D>
 static int launch_dkv(hipStream_t stream, const AttnParams& p) {
-  const size_t smem = DkvSmem<D>::kBytes;
+  const size_t smem = QdoStage<D>::kTotalBytes;
   {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dkv_kernel<D>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
   }
-  const int grid = (p.S / 128) * p.Hkv * p.B;
+  const int grid = (p.S / 128) * p.Hkv * p.B;  // rank-major, see attn_dkv_kernel
   LaunchScope scope3("attn_dkv_kernel", stream);
   hipLaunchKernelGGL((attn_dkv_kernel<D>), dim3(grid), dim3(256), smem, stream, p);
   return scope3.done();
@@ -220,7 +273,7 @@ using namespace ct;
 
 extern "C" size_t ct_attn_meta_bytes(int32_t batch, int32_t seq) {
   if (batch <= 0 || seq <= 0) return 0;
-  return (size_t)batch * (size_t)(seq / 32) * kMetaW * sizeof(int32_t);
+  return (size_t)batch * (size_t)(seq / 32) * (kMetaW + 2) * sizeof(int32_t);
 }
 
 extern "C" int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
@@ -239,7 +292,8 @@ extern "C" int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
   const int threads = nrb >= 1024 ? 1024 : ((nrb + 63) / 64) * 64;
   LaunchScope scope5("attn_prepare_kernel", (hipStream_t)stream);
   hipLaunchKernelGGL(attn_prepare_kernel, dim3(batch), dim3(threads), smem, (hipStream_t)stream,
-                     segment_ids, attention_end, seq, tile_meta);
+                     segment_ids, attention_end, seq, tile_meta,
+                     tile_meta + (size_t)batch * nrb * kMetaW);
   return scope5.done();
 }
 
@@ -272,6 +326,7 @@ extern "C" int32_t ct_attn_fwd(void* stream, const ct_attn_fwd_args* a) {
   p.seg = a->segment_ids;
   p.end = a->attention_end;
   p.meta = a->tile_meta;
+  p.sched = a->tile_meta + (size_t)a->batch * (a->seq / 32) * kMetaW;
   p.out = reinterpret_cast<bf16*>(a->out);
   p.lse = a->lse;
   p.B = a->batch;
@@ -310,6 +365,7 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   p.seg = a->segment_ids;
   p.end = a->attention_end;
   p.meta = a->tile_meta;
+  p.sched = a->tile_meta + (size_t)a->batch * (a->seq / 32) * kMetaW;
   p.out = const_cast<bf16*>(reinterpret_cast<const bf16*>(a->out));
   p.lse = const_cast<float*>(a->lse);
   p.dout = reinterpret_cast<const bf16*>(a->dout);

@@ -22,94 +22,79 @@ namespace ct {
 // ---------------------------------------------------------------------------
 template <int D, int HS>
 __global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
-  constexpr int PB = 4 / HS;
   extern __shared__ __align__(16) char smem_raw[];
-  KvSmem<D> sm(smem_raw);
+  const lds_addr lds0 = lds_address_of(smem_raw);
+  constexpr int kStage = KvStage<D>::kBytes;
 
-  const QueryWork<HS> work(p);
-  const int l = lane_id(), j = l & 31, half = l >> 5, w = threadIdx.x >> 6;
-  const int nrb = p.S / 32;
-  const int* meta_b = p.meta + (size_t)work.b * nrb * kMetaW;
-  const int pos = work.rb * 32 + j;
-
-  QueryBlockBounds wq[PB];
-#pragma unroll
-  for (int i = 0; i < PB; ++i) wq[i] = query_block_bounds(meta_b, work.qt * PB + i);
-  const QueryBlockBounds mine = query_block_bounds(meta_b, work.rb);
-  int first = INT_MAX, last = -1;
-#pragma unroll
-  for (int i = 0; i < PB; ++i) {
-    first = min(first, wq[i].kv_first);
-    last = max(last, wq[i].kv_last);
-  }
-
+  const QueryTileContext<D, HS> ctx(p);
+  const int l = lane_id(), half = l >> 5, w = threadIdx.x >> 6;
+  const RowFragOffsets<D / 8> ro;
+  const TrFragOffsets<D / 8, KSlots::kAccum> to;
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
-  const size_t q_off = (((size_t)work.b * p.S + pos) * p.Hq + work.h) * D;
-  const size_t stat_off = ((size_t)work.b * p.S + pos) * p.Hq + work.h;
-  const int seg_q = p.seg[(size_t)work.b * p.S + pos];
-  const int end_q = p.end ? p.end[(size_t)work.b * p.S + pos] : pos;
-  const bool row_valid = seg_q != 0;
-  const float lse2 = p.lse[stat_off] * kLog2e;
-  const float delta_q = p.delta[stat_off];
+  const float lse2 = p.lse[ctx.stat_off] * kLog2e;
+  const float delta_q = p.delta[ctx.stat_off];
 
   bf16x8 qf[D / 16], dof[D / 16];
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) {
-    qf[ks] = scale_bf16x8(as_bf16x8(load_global16(p.q + q_off + 16 * ks + 8 * half)), p.scale);
-    dof[ks] = as_bf16x8(load_global16(p.dout + q_off + 16 * ks + 8 * half));
+    qf[ks] = scale_bf16x8(as_bf16x8(load_global16(p.q + ctx.q_off + 16 * ks + 8 * half)), p.scale);
+    dof[ks] = as_bf16x8(load_global16(p.dout + ctx.q_off + 16 * ks + 8 * half));
   }
-
   f32x16 dqacc[D / 32];
 #pragma unroll
   for (int db = 0; db < D / 32; ++db) dqacc[db] = zero16();
 
-  const bf16* kbase = p.k + ((size_t)work.b * p.S * p.Hkv + work.kvh) * D;
-  const bf16* vbase = p.v + ((size_t)work.b * p.S * p.Hkv + work.kvh) * D;
-  const int* segb = p.seg + (size_t)work.b * p.S;
-
-  int t = (first <= last) ? next_tile<PB>(meta_b, wq, first, last) : last + 1;
-  if (t <= last) {
+  int t = ctx.first;
+  KeyTileBounds kb = {0, 0, 0};
+  if (t <= ctx.last) {
     KvRegs<D> regs;
-    kv_fetch<D>(regs, kbase, vbase, segb, kv_row_stride, t);
-    kv_commit<D>(regs, sm.k[0], sm.v[0], sm.seg[0]);
+    kv_fetch<D>(regs, ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride, t);
+    kb = key_tile_bounds(ctx.meta_b, t);
+    kv_commit<D>(regs, lds0);
   }
   __syncthreads();
-  int cur = 0;
-  while (t <= last) {
-    const int tn = next_tile<PB>(meta_b, wq, t + 1, last);
-    KvRegs<D> regs;
-    if (tn <= last) kv_fetch<D>(regs, kbase, vbase, segb, kv_row_stride, tn);
 
-    const KeyTileBounds kb = key_tile_bounds(meta_b, t);
-    if (blocks_interact(mine.min_nz, mine.max_id, mine.end_max, uniform(kb.min_nz),
-                        uniform(kb.max_id), t * kKeyTile)) {
+  auto step = [&](auto stage_tag) {
+    constexpr int CUR = decltype(stage_tag)::value;
+    const lds_addr stage = lds0 + CUR * kStage;
+    const bool more = t + 1 <= ctx.last;
+    KvRegs<D> regs;
+    KeyTileBounds nb = kb;
+    if (more) {
+      kv_fetch<D>(regs, ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride, t + 1);
+      nb = key_tile_bounds(ctx.meta_b, t + 1);
+    }
+    if (ctx.wave_visits(kb, t)) {
       f32x16 s[2], dp[2];
-      scores_t<D>(sm.k[cur], qf, s);
-      scores_t<D>(sm.v[cur], dof, dp);
-      const bool interior = tile_is_interior(mine.uniform, mine.end_min, uniform(kb.uniform),
-                                             t * kKeyTile + kKeyTile - 1);
+      scores_t<D>(stage + KvStage<D>::kK, ro, qf, s);
+      scores_t<D>(stage + KvStage<D>::kV, ro, dof, dp);
       unsigned allow[2] = {0xffffffffu, 0xffffffffu};
-      if (!interior) tile_mask(sm.seg[cur], t, seg_q, end_q, row_valid, allow);
+      if (!ctx.interior(kb, t))
+        tile_mask(stage + KvStage<D>::kSeg, t, ctx.seg_q, ctx.end_q, ctx.row_valid, allow);
 #pragma unroll
       for (int kbk = 0; kbk < 2; ++kbk)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float prob =
-              ((allow[kbk] >> r) & 1u) ? exp2_fast(s[kbk][r] * kLog2e - lse2) : 0.f;
+              ((allow[kbk] >> r) & 1u) ? exp2_fast(fmaf(s[kbk][r], kLog2e, -lse2)) : 0.f;
           s[kbk][r] = prob * (dp[kbk][r] - delta_q);
         }
-      accumulate_t<D>(sm.k[cur], s, dqacc);
+      accumulate_t<D>(stage + KvStage<D>::kK, to, s, dqacc);
     }
-
-    if (tn <= last) kv_commit<D>(regs, sm.k[cur ^ 1], sm.v[cur ^ 1], sm.seg[cur ^ 1]);
+    if (more) kv_commit<D>(regs, lds0 + (CUR ^ 1) * kStage);
     __syncthreads();
-    t = tn;
-    cur ^= 1;
+    kb = nb;
+    ++t;
+  };
+  while (t <= ctx.last) {
+    step(std::integral_constant<int, 0>{});
+    if (t > ctx.last) break;
+    step(std::integral_constant<int, 1>{});
   }
 
-  bf16* patch = reinterpret_cast<bf16*>(smem_raw) + w * 32 * D;
-  bf16* gbase = p.dq + (((size_t)work.b * p.S + work.rb * 32) * p.Hq + work.h) * D;
+  const lds_addr patch = lds0 + w * 32 * D * 2;
+  bf16* gbase = p.dq + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
   store_rows_t<D>(dqacc, p.scale, patch, gbase, q_row_stride);
 }
 
@@ -118,39 +103,27 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
 // ---------------------------------------------------------------------------
 constexpr int kQueryTile = 32;
 
+// LDS stage: Q tile, dO tile (32 x D bf16 each), then lse2 / delta (f32) and
+// seg / end (i32), 32 entries each.
 template <int D>
-struct DkvSmem {
-  static constexpr int kTileElems = kQueryTile * D;
-  // per stage: Q tile, dO tile, then lse2 / delta (f32) and seg / end (i32) rows
-  static constexpr size_t kStageBytes = 2 * kTileElems * sizeof(bf16) + 4 * kQueryTile * 4;
-  static constexpr size_t kPatchBytes = 4 * 32 * D * sizeof(bf16);
-  static constexpr size_t kBytes =
-      (2 * kStageBytes > kPatchBytes) ? 2 * kStageBytes : kPatchBytes;
-  bf16* q[2];
-  bf16* dout[2];
-  float* lse2[2];
-  float* delta[2];
-  int* seg[2];
-  int* end[2];
-  CT_DEVICE explicit DkvSmem(char* base) {
-#pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      char* b = base + s * kStageBytes;
-      q[s] = reinterpret_cast<bf16*>(b);
-      dout[s] = q[s] + kTileElems;
-      lse2[s] = reinterpret_cast<float*>(dout[s] + kTileElems);
-      delta[s] = lse2[s] + kQueryTile;
-      seg[s] = reinterpret_cast<int*>(delta[s] + kQueryTile);
-      end[s] = seg[s] + kQueryTile;
-    }
-  }
+struct QdoStage {
+  static constexpr int kTileBytes = kQueryTile * D * 2;
+  static constexpr int kQ = 0;
+  static constexpr int kDo = kTileBytes;
+  static constexpr int kLse = 2 * kTileBytes;
+  static constexpr int kDelta = kLse + kQueryTile * 4;
+  static constexpr int kSeg = kDelta + kQueryTile * 4;
+  static constexpr int kEnd = kSeg + kQueryTile * 4;
+  static constexpr int kBytes = kEnd + kQueryTile * 4;
+  static constexpr int kPatchBytes = 4 * 32 * D * 2;
+  static constexpr int kTotalBytes = (2 * kBytes > kPatchBytes) ? 2 * kBytes : kPatchBytes;
 };
 
 template <int D>
 struct QdoRegs {
   static constexpr int kChunks = kQueryTile * (D / 8) / 256;
-  uint4 q[kChunks];
-  uint4 dout[kChunks];
+  u32x4 q[kChunks];
+  u32x4 dout[kChunks];
   float lse2, delta;
   int seg, end;
 };
@@ -178,107 +151,93 @@ CT_DEVICE void qdo_fetch(QdoRegs<D>& r, const AttnParams& p, int b, int h, int q
 }
 
 template <int D>
-CT_DEVICE void qdo_commit(const QdoRegs<D>& r, const DkvSmem<D>& sm, int stage, float scale) {
+CT_DEVICE void qdo_commit(const QdoRegs<D>& r, lds_addr stage, float scale) {
   constexpr int CPR = D / 8;
   const int tid = threadIdx.x;
 #pragma unroll
   for (int n = 0; n < QdoRegs<D>::kChunks; ++n) {
     const int e = tid + 256 * n;
-    const int row = e / CPR, c = e % CPR;
-    tile_store_chunk<CPR>(sm.q[stage], row, c, as_uint4(scale_bf16x8(as_bf16x8(r.q[n]), scale)));
-    tile_store_chunk<CPR>(sm.dout[stage], row, c, r.dout[n]);
+    const int off = tile_byte_offset<CPR>(e / CPR, e % CPR);
+    lds_store<u32x4>(stage + QdoStage<D>::kQ + off, as_u32x4(scale_bf16x8(as_bf16x8(r.q[n]), scale)));
+    lds_store<u32x4>(stage + QdoStage<D>::kDo + off, r.dout[n]);
   }
   if (tid < kQueryTile) {
-    sm.lse2[stage][tid] = r.lse2;
-    sm.delta[stage][tid] = r.delta;
-    sm.seg[stage][tid] = r.seg;
-    sm.end[stage][tid] = r.end;
+    lds_store<float>(stage + QdoStage<D>::kLse + tid * 4, r.lse2);
+    lds_store<float>(stage + QdoStage<D>::kDelta + tid * 4, r.delta);
+    lds_store<int>(stage + QdoStage<D>::kSeg + tid * 4, r.seg);
+    lds_store<int>(stage + QdoStage<D>::kEnd + tid * 4, r.end);
   }
 }
 
 // X (32 rows of an LDS tile) times register fragments: C[row, key] = sum_d X[row, d] F[key, d].
 template <int D>
-CT_DEVICE f32x16 rows_times_frags(const bf16* tile, const bf16x8* frags) {
-  constexpr int CPR = D / 8;
-  const int l = lane_id(), j = l & 31, half = l >> 5;
+CT_DEVICE f32x16 rows_times_frags(lds_addr tile, const RowFragOffsets<D / 8>& ro,
+                                  const bf16x8* frags) {
   f32x16 c = zero16();
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) {
-    const bf16x8 a = tile_read_row8<CPR>(tile, j, 2 * ks + half);
-    c = mfma32(a, frags[ks], c);
-  }
+  for (int ks = 0; ks < D / 16; ++ks) c = mfma32(lds_load<bf16x8>(tile + ro.off[ks]), frags[ks], c);
   return c;
 }
 
 // acc (32 keys x D) += W^T X, W in accumulator layout (rows = the 32 tile rows,
 // cols = keys), X the 32-row LDS tile read transposed.
 template <int D>
-CT_DEVICE void accumulate_keys(const bf16* tile, const f32x16& wt, f32x16* acc) {
-  constexpr int CPR = D / 8;
-  const int half = lane_id() >> 5;
+CT_DEVICE void accumulate_keys(lds_addr tile, const TrFragOffsets<D / 8, KSlots::kAccum>& to,
+                               const f32x16& wt, f32x16* acc) {
 #pragma unroll
   for (int step = 0; step < 2; ++step) {
     const bf16x8 aop = pack_acc8(wt, step);
-    int rowA, rowB;
-    kslot_rows_accum(16 * step, half, rowA, rowB);
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db) {
-      const bf16x8 bop = tile_read_tr8<CPR>(tile, rowA, rowB, db * 32);
-      acc[db] = mfma32(aop, bop, acc[db]);
-    }
+    for (int db = 0; db < D / 32; ++db) acc[db] = mfma32(aop, to.load(tile, step, db), acc[db]);
   }
 }
 
 // Store a (32 rows x D) accumulator (lanes along D) as bf16 rows via an LDS patch.
 template <int D>
-CT_DEVICE void store_rows(const f32x16* acc, bf16* patch, bf16* gbase, size_t row_stride) {
+CT_DEVICE void store_rows(const f32x16* acc, lds_addr patch, bf16* gbase, size_t row_stride) {
   constexpr int CPR = D / 8;
   const int l = lane_id(), j = l & 31, half = l >> 5;
 #pragma unroll
   for (int db = 0; db < D / 32; ++db) {
     const int col = db * 32 + j;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int row = acc_row(r, half);
-      patch[tile_offset<CPR>(row, col >> 3) + (col & 7)] = (bf16)acc[db][r];
-    }
+    for (int r = 0; r < 16; ++r)
+      lds_store<bf16>(patch + tile_byte_offset<CPR>(acc_row(r, half), col >> 3) + (col & 7) * 2,
+                      (bf16)acc[db][r]);
   }
   __builtin_amdgcn_wave_barrier();
 #pragma unroll
   for (int n = 0; n < 32 * CPR / 64; ++n) {
     const int e = l + 64 * n;
     const int row = e / CPR, c = e % CPR;
-    const bf16x8 val = tile_read_row8<CPR>(patch, row, c);
-    *reinterpret_cast<uint4*>(gbase + (size_t)row * row_stride + c * 8) = as_uint4(val);
+    const u32x4 val = lds_load<u32x4>(patch + tile_byte_offset<CPR>(row, c));
+    store_global16(gbase + (size_t)row * row_stride + c * 8, val);
   }
 }
 
 template <int D>
 __global__ __launch_bounds__(256) void attn_dkv_kernel(AttnParams p) {
   extern __shared__ __align__(16) char smem_raw[];
-  DkvSmem<D> sm(smem_raw);
+  const lds_addr lds0 = lds_address_of(smem_raw);
+  constexpr int kStage = QdoStage<D>::kBytes;
 
   const int l = lane_id(), j = l & 31, half = l >> 5, w = threadIdx.x >> 6;
-  const int nkt = p.S / 128;
-  const int total = nkt * p.Hkv * p.B;
-  int id = xcd_remap(blockIdx.x, total);
-  const int kt = id % nkt;  // early key tiles are seen by the most queries
-  id /= nkt;
-  const int kvh = id % p.Hkv;
-  const int b = id / p.Hkv;
-  const int g = p.Hq / p.Hkv;
   const int nrb = p.S / 32;
+  const int groups = p.B * p.Hkv;
+  const int group = blockIdx.x % groups, rank = blockIdx.x / groups;
+  const int kvh = group % p.Hkv;
+  const int b = group / p.Hkv;
+  const int kt =
+      uniform(p.sched[(size_t)b * schedule_ints(nrb) + key_schedule_offset(nrb) + rank]);
+  const int g = p.Hq / p.Hkv;
   const int* meta_b = p.meta + (size_t)b * nrb * kMetaW;
+  const RowFragOffsets<D / 8> ro;
+  const TrFragOffsets<D / 8, KSlots::kAccum> to;
 
-  // Key-side bounds of the 4 row blocks of this workgroup; [4] is this wavefront's.
-  int k_min[4], k_max[4], k_uni[4];
   int q_lo = INT_MAX, q_hi = -1;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int* m = meta_b + (kt * 4 + i) * kMetaW;
-    k_min[i] = uniform(m[kMinNz]);
-    k_max[i] = uniform(m[kMaxId]);
-    k_uni[i] = uniform(m[kUniform]);
     q_lo = min(q_lo, uniform(m[kQFirst]));
     q_hi = max(q_hi, uniform(m[kQLast]));
   }
@@ -305,75 +264,73 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(AttnParams p) {
     dvacc[db] = zero16();
   }
 
-  // Work items: (head of the group, query block) pairs, flattened.
+  // Work items: (head of the group, query block) pairs, flattened; query block fastest.
   const int nq = (q_lo <= q_hi) ? (q_hi - q_lo + 1) : 0;
   const int items = nq * g;
-  auto item_needed = [&](int it) -> bool {
-    const int* m = meta_b + (q_lo + it % nq) * kMetaW;
-    const int q_min = m[kMinNz], q_max = m[kMaxId], q_end = m[kEndMax];
-    bool any = false;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      any |= blocks_interact(q_min, q_max, q_end, k_min[i], k_max[i], (kt * 4 + i) * 32);
-    return any;
-  };
-  auto next_item = [&](int it) -> int {
-    while (it < items && !item_needed(it)) ++it;
-    return uniform(it);
-  };
-
-  int it = next_item(0);
+  int it = 0, qb = q_lo, head = kvh * g;
   if (it < items) {
     QdoRegs<D> regs;
-    qdo_fetch<D>(regs, p, b, kvh * g + it / nq, q_lo + it % nq);
-    qdo_commit<D>(regs, sm, 0, p.scale);
+    qdo_fetch<D>(regs, p, b, head, qb);
+    qdo_commit<D>(regs, lds0, p.scale);
   }
   __syncthreads();
-  int cur = 0;
-  while (it < items) {
-    const int itn = next_item(it + 1);
-    QdoRegs<D> regs;
-    if (itn < items) qdo_fetch<D>(regs, p, b, kvh * g + itn / nq, q_lo + itn % nq);
 
-    const int qb = q_lo + it % nq;
+  auto step = [&](auto stage_tag) {
+    constexpr int CUR = decltype(stage_tag)::value;
+    const lds_addr stage = lds0 + CUR * kStage;
+    const bool more = it + 1 < items;
+    int qb_next = qb + 1, head_next = head;
+    if (qb_next > q_hi) {
+      qb_next = q_lo;
+      ++head_next;
+    }
+    QdoRegs<D> regs;
+    if (more) qdo_fetch<D>(regs, p, b, head_next, qb_next);
+
     const int* qm = meta_b + qb * kMetaW;
     const int q_min = uniform(qm[kMinNz]), q_max = uniform(qm[kMaxId]),
               q_end_max = uniform(qm[kEndMax]), q_end_min = uniform(qm[kEndMin]),
               q_uni = uniform(qm[kUniform]);
     if (blocks_interact(q_min, q_max, q_end_max, my_min, my_max, my_rb * 32)) {
-      f32x16 s = rows_times_frags<D>(sm.q[cur], kf);
-      f32x16 dp = rows_times_frags<D>(sm.dout[cur], vf);
+      f32x16 s = rows_times_frags<D>(stage + QdoStage<D>::kQ, ro, kf);
+      f32x16 dp = rows_times_frags<D>(stage + QdoStage<D>::kDo, ro, vf);
       const bool interior = tile_is_interior(q_uni, q_end_min, my_uni, my_rb * 32 + 31);
       f32x16 prob;
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
         const int r0 = 8 * qd + 4 * half;  // first of 4 consecutive query rows
-        const f32x4 lse4 = *reinterpret_cast<const f32x4*>(sm.lse2[cur] + r0);
-        const f32x4 del4 = *reinterpret_cast<const f32x4*>(sm.delta[cur] + r0);
-        const int4 seg4 = *reinterpret_cast<const int4*>(sm.seg[cur] + r0);
-        const int4 end4 = *reinterpret_cast<const int4*>(sm.end[cur] + r0);
-        const int segs[4] = {seg4.x, seg4.y, seg4.z, seg4.w};
-        const int ends[4] = {end4.x, end4.y, end4.z, end4.w};
+        const f32x4 lse4 = lds_load<f32x4>(stage + QdoStage<D>::kLse + r0 * 4);
+        const f32x4 del4 = lds_load<f32x4>(stage + QdoStage<D>::kDelta + r0 * 4);
+        i32x4 seg4, end4;
+        if (!interior) {
+          seg4 = lds_load<i32x4>(stage + QdoStage<D>::kSeg + r0 * 4);
+          end4 = lds_load<i32x4>(stage + QdoStage<D>::kEnd + r0 * 4);
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = 4 * qd + e;
-          const bool ok = interior || (segs[e] == seg_k && seg_k != 0 && key <= ends[e]);
-          const float pr = ok ? exp2_fast(s[r] * kLog2e - lse4[e]) : 0.f;
+          const bool ok = interior || (seg4[e] == seg_k && seg_k != 0 && key <= end4[e]);
+          const float pr = ok ? exp2_fast(fmaf(s[r], kLog2e, -lse4[e])) : 0.f;
           prob[r] = pr;
           dp[r] = pr * (dp[r] - del4[e]);
         }
       }
-      accumulate_keys<D>(sm.dout[cur], prob, dvacc);
-      accumulate_keys<D>(sm.q[cur], dp, dkacc);
+      accumulate_keys<D>(stage + QdoStage<D>::kDo, to, prob, dvacc);
+      accumulate_keys<D>(stage + QdoStage<D>::kQ, to, dp, dkacc);
     }
-
-    if (itn < items) qdo_commit<D>(regs, sm, cur ^ 1, p.scale);
+    if (more) qdo_commit<D>(regs, lds0 + (CUR ^ 1) * kStage, p.scale);
     __syncthreads();
-    it = itn;
-    cur ^= 1;
+    ++it;
+    qb = qb_next;
+    head = head_next;
+  };
+  while (it < items) {
+    step(std::integral_constant<int, 0>{});
+    if (it >= items) break;
+    step(std::integral_constant<int, 1>{});
   }
 
-  bf16* patch = reinterpret_cast<bf16*>(smem_raw) + w * 32 * D;
+  const lds_addr patch = lds0 + w * 32 * D * 2;
   const size_t out_off = (((size_t)b * p.S + my_rb * 32) * p.Hkv + kvh) * D;
   store_rows<D>(dkacc, patch, p.dk + out_off, kv_row_stride);
   __builtin_amdgcn_wave_barrier();

@@ -1,4 +1,4 @@
-// Attention kernels for gfx950: forward, delta, dQ and dK/dV.
+// Attention kernels for gfx950: forward and delta (shared pieces for dQ too).
 //
 // Common structure. A workgroup is 4 wavefronts. In the forward and dQ
 // kernels every wavefront owns 32 query rows of one query head (a "row
@@ -22,6 +22,8 @@
 // (src/modeling/attention.py:138).
 #pragma once
 
+#include <type_traits>
+
 #include "ct_attn_meta.cuh"
 #include "ct_common.cuh"
 
@@ -36,7 +38,8 @@ struct AttnParams {
   const bf16* v;
   const int* seg;
   const int* end;   // may be null
-  const int* meta;
+  const int* meta;  // [B][nrb][kMetaW]
+  const int* sched; // [B][schedule_ints(nrb)]
   bf16* out;        // forward: written; backward: forward output
   float* lse;
   const bf16* dout;
@@ -50,12 +53,22 @@ struct AttnParams {
 
 // ---------------------------------------------------------------------------
 // K/V tile staging: global -> registers -> swizzled LDS.
+// LDS stage layout: K tile, V tile (64 x D bf16 each), 64 segment ids.
 // ---------------------------------------------------------------------------
+template <int D>
+struct KvStage {
+  static constexpr int kTileBytes = kKeyTile * D * 2;
+  static constexpr int kK = 0;
+  static constexpr int kV = kTileBytes;
+  static constexpr int kSeg = 2 * kTileBytes;
+  static constexpr int kBytes = 2 * kTileBytes + kKeyTile * 4;
+};
+
 template <int D>
 struct KvRegs {
   static constexpr int kChunks = kKeyTile * (D / 8) / 256;
-  uint4 k[kChunks];
-  uint4 v[kChunks];
+  u32x4 k[kChunks];
+  u32x4 v[kChunks];
   int seg;
 };
 
@@ -76,87 +89,59 @@ CT_DEVICE void kv_fetch(KvRegs<D>& r, const bf16* kbase, const bf16* vbase, cons
 }
 
 template <int D>
-CT_DEVICE void kv_commit(const KvRegs<D>& r, bf16* ktile, bf16* vtile, int* segk) {
+CT_DEVICE void kv_commit(const KvRegs<D>& r, lds_addr stage) {
   constexpr int CPR = D / 8;
   const int tid = threadIdx.x;
 #pragma unroll
   for (int n = 0; n < KvRegs<D>::kChunks; ++n) {
     const int e = tid + 256 * n;
-    const int row = e / CPR, c = e % CPR;
-    tile_store_chunk<CPR>(ktile, row, c, r.k[n]);
-    tile_store_chunk<CPR>(vtile, row, c, r.v[n]);
+    const int off = tile_byte_offset<CPR>(e / CPR, e % CPR);
+    lds_store<u32x4>(stage + KvStage<D>::kK + off, r.k[n]);
+    lds_store<u32x4>(stage + KvStage<D>::kV + off, r.v[n]);
   }
-  if (tid < kKeyTile) segk[tid] = r.seg;
+  if (tid < kKeyTile) lds_store<int>(stage + KvStage<D>::kSeg + tid * 4, r.seg);
 }
 
-// LDS carve-up for the forward / dQ kernels.
-template <int D>
-struct KvSmem {
-  static constexpr int kTileElems = kKeyTile * D;
-  static constexpr size_t kBytes = 2 * (2 * kTileElems * sizeof(bf16)) + 2 * kKeyTile * sizeof(int);
-  bf16* k[2];
-  bf16* v[2];
-  int* seg[2];
-  CT_DEVICE explicit KvSmem(char* base) {
-    bf16* t = reinterpret_cast<bf16*>(base);
-    k[0] = t;
-    v[0] = t + kTileElems;
-    k[1] = t + 2 * kTileElems;
-    v[1] = t + 3 * kTileElems;
-    seg[0] = reinterpret_cast<int*>(t + 4 * kTileElems);
-    seg[1] = seg[0] + kKeyTile;
-  }
-};
-
-// Decoded position of a workgroup / wavefront in the (batch, head, row block) space.
+// Decoded position of a workgroup / wavefront in the (batch, head, row block)
+// space. Hardware workgroup ids run over (rank, group): the group (batch,
+// head slice, KV head) is the fast index, so a group always lands on the same
+// XCD (ids are dealt round robin to the 8 XCDs) and keeps its K/V in that L2;
+// the rank is the position in the batch row's work-sorted schedule, longest
+// tiles first.
 template <int HS>
 struct QueryWork {
   static constexpr int PB = 4 / HS;  // row blocks per workgroup
   int b, h, kvh, qt, rb;
   CT_DEVICE QueryWork(const AttnParams& p) {
-    const int nqt = p.S / (32 * PB);
-    const int hgroups = p.Hq / HS;
-    const int total = nqt * hgroups * p.B;
-    int id = xcd_remap(blockIdx.x, total);
-    qt = nqt - 1 - (id % nqt);  // longest key ranges first
-    id /= nqt;
-    const int hg = id % hgroups;
-    b = id / hgroups;
+    const int nrb = p.S / 32;
+    const int g = p.Hq / p.Hkv;
+    const int slices = g / HS;
+    const int groups = p.B * slices * p.Hkv;
+    const int group = blockIdx.x % groups, rank = blockIdx.x / groups;
+    kvh = group % p.Hkv;
+    const int rest = group / p.Hkv;
+    const int slice = rest % slices;
+    b = rest / slices;
+    const int* sched = p.sched + (size_t)b * schedule_ints(nrb) + query_schedule_offset(nrb, PB);
+    qt = uniform(sched[rank]);
     const int w = threadIdx.x >> 6;
-    h = hg * HS + (w % HS);
-    kvh = (hg * HS) / (p.Hq / p.Hkv);
+    h = kvh * g + slice * HS + (w % HS);
     rb = qt * PB + (w / HS);
   }
 };
 
-// Next tile >= t (and <= last) that any row block of the workgroup visits;
-// last + 1 if none.
-template <int PB>
-CT_DEVICE int next_tile(const int* meta_b, const QueryBlockBounds* wq, int t, int last) {
-  for (; t <= last; ++t) {
-    const KeyTileBounds kb = key_tile_bounds(meta_b, t);
-    bool any = false;
-#pragma unroll
-    for (int i = 0; i < PB; ++i)
-      any |= blocks_interact(wq[i].min_nz, wq[i].max_id, wq[i].end_max, kb.min_nz, kb.max_id,
-                             t * kKeyTile);
-    if (any) break;
-  }
-  return uniform(t);
-}
-
 // S^T (two 32-key blocks) = K_tile Q^T for this wavefront's 32 queries.
 template <int D>
-CT_DEVICE void scores_t(const bf16* ktile, const bf16x8* qf, f32x16* s) {
-  constexpr int CPR = D / 8;
-  const int l = lane_id(), j = l & 31, half = l >> 5;
+CT_DEVICE void scores_t(lds_addr tile, const RowFragOffsets<D / 8>& ro, const bf16x8* qf,
+                        f32x16* s) {
   s[0] = zero16();
   s[1] = zero16();
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) {
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
-      const bf16x8 a = tile_read_row8<CPR>(ktile, kb * 32 + j, 2 * ks + half);
+      const bf16x8 a =
+          lds_load<bf16x8>(tile + kb * RowFragOffsets<D / 8>::kRowBlockBytes + ro.off[ks]);
       s[kb] = mfma32(a, qf[ks], s[kb]);
     }
   }
@@ -164,7 +149,7 @@ CT_DEVICE void scores_t(const bf16* ktile, const bf16x8* qf, f32x16* s) {
 
 // allowed(query of this lane, key held by register r of block kb)?  Writes a
 // 32-bit mask per block: bit r set = allowed.
-CT_DEVICE void tile_mask(const int* segk, int tile, int seg_q, int end_q, bool row_valid,
+CT_DEVICE void tile_mask(lds_addr segk, int tile, int seg_q, int end_q, bool row_valid,
                          unsigned* allow) {
   const int half = lane_id() >> 5;
 #pragma unroll
@@ -173,33 +158,26 @@ CT_DEVICE void tile_mask(const int* segk, int tile, int seg_q, int end_q, bool r
 #pragma unroll
     for (int qd = 0; qd < 4; ++qd) {
       const int k0 = kb * 32 + 8 * qd + 4 * half;
-      const int4 sk = *reinterpret_cast<const int4*>(segk + k0);
+      const i32x4 sk = lds_load<i32x4>(segk + k0 * 4);
       const int key = tile * kKeyTile + k0;
-      bits |= (unsigned)(sk.x == seg_q && key + 0 <= end_q) << (4 * qd + 0);
-      bits |= (unsigned)(sk.y == seg_q && key + 1 <= end_q) << (4 * qd + 1);
-      bits |= (unsigned)(sk.z == seg_q && key + 2 <= end_q) << (4 * qd + 2);
-      bits |= (unsigned)(sk.w == seg_q && key + 3 <= end_q) << (4 * qd + 3);
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        bits |= (unsigned)(sk[e] == seg_q && key + e <= end_q) << (4 * qd + e);
     }
     allow[kb] = row_valid ? bits : 0u;
   }
 }
 
 // acc (D x 32 queries, transposed) += X^T W^T where X is a 64-row LDS tile read
-// transposed and W^T are the packed accumulator-layout weights wt[2].
+// transposed and W^T are the accumulator-layout weights wt[2].
 template <int D>
-CT_DEVICE void accumulate_t(const bf16* tile, const f32x16* wt, f32x16* acc) {
-  constexpr int CPR = D / 8;
-  const int half = lane_id() >> 5;
+CT_DEVICE void accumulate_t(lds_addr tile, const TrFragOffsets<D / 8, KSlots::kAccum>& to,
+                            const f32x16* wt, f32x16* acc) {
 #pragma unroll
   for (int step = 0; step < 4; ++step) {
     const bf16x8 bop = pack_acc8(wt[step >> 1], step & 1);
-    int rowA, rowB;
-    kslot_rows_accum(16 * step, half, rowA, rowB);
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db) {
-      const bf16x8 a = tile_read_tr8<CPR>(tile, rowA, rowB, db * 32);
-      acc[db] = mfma32(a, bop, acc[db]);
-    }
+    for (int db = 0; db < D / 32; ++db) acc[db] = mfma32(to.load(tile, step, db), bop, acc[db]);
   }
 }
 
@@ -207,7 +185,7 @@ CT_DEVICE void accumulate_t(const bf16* tile, const f32x16* wt, f32x16* acc) {
 // global memory, staged through this wavefront's private LDS patch so that
 // the global stores are 16 bytes per lane and contiguous per row.
 template <int D>
-CT_DEVICE void store_rows_t(const f32x16* acc, float row_scale, bf16* patch, bf16* gbase,
+CT_DEVICE void store_rows_t(const f32x16* acc, float row_scale, lds_addr patch, bf16* gbase,
                             size_t row_stride) {
   constexpr int CPR = D / 8;
   const int l = lane_id(), j = l & 31, half = l >> 5;
@@ -219,7 +197,7 @@ CT_DEVICE void store_rows_t(const f32x16* acc, float row_scale, bf16* patch, bf1
       bf16x4 pk;
 #pragma unroll
       for (int e = 0; e < 4; ++e) pk[e] = (bf16)(acc[db][4 * qd + e] * row_scale);
-      *reinterpret_cast<bf16x4*>(patch + tile_offset<CPR>(j, d0 >> 3) + (d0 & 4)) = pk;
+      lds_store<bf16x4>(patch + tile_byte_offset<CPR>(j, d0 >> 3) + (d0 & 4) * 2, pk);
     }
   }
   __builtin_amdgcn_wave_barrier();
@@ -227,48 +205,78 @@ CT_DEVICE void store_rows_t(const f32x16* acc, float row_scale, bf16* patch, bf1
   for (int n = 0; n < 32 * CPR / 64; ++n) {
     const int e = l + 64 * n;
     const int row = e / CPR, c = e % CPR;
-    const bf16x8 val = tile_read_row8<CPR>(patch, row, c);
-    *reinterpret_cast<uint4*>(gbase + (size_t)row * row_stride + c * 8) = as_uint4(val);
+    const u32x4 val = lds_load<u32x4>(patch + tile_byte_offset<CPR>(row, c));
+    store_global16(gbase + (size_t)row * row_stride + c * 8, val);
   }
 }
+
+// Shared prologue of the forward and dQ kernels.
+template <int D, int HS>
+struct QueryTileContext {
+  static constexpr int PB = 4 / HS;
+  QueryWork<HS> work;
+  const int* meta_b;
+  QueryBlockBounds mine;
+  int first, last;
+  int pos, seg_q, end_q;
+  bool row_valid;
+  size_t q_off, stat_off;
+  const bf16* kbase;
+  const bf16* vbase;
+  const int* segb;
+  CT_DEVICE explicit QueryTileContext(const AttnParams& p) : work(p) {
+    const int nrb = p.S / 32;
+    meta_b = p.meta + (size_t)work.b * nrb * kMetaW;
+    mine = query_block_bounds(meta_b, work.rb);
+    first = INT_MAX;
+    last = -1;
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+      const int* m = meta_b + (work.qt * PB + i) * kMetaW;
+      first = min(first, uniform(m[kKvFirst]));
+      last = max(last, uniform(m[kKvLast]));
+    }
+    pos = work.rb * 32 + (lane_id() & 31);
+    seg_q = p.seg[(size_t)work.b * p.S + pos];
+    end_q = p.end ? p.end[(size_t)work.b * p.S + pos] : pos;
+    row_valid = seg_q != 0;
+    q_off = (((size_t)work.b * p.S + pos) * p.Hq + work.h) * D;
+    stat_off = ((size_t)work.b * p.S + pos) * p.Hq + work.h;
+    kbase = p.k + ((size_t)work.b * p.S * p.Hkv + work.kvh) * D;
+    vbase = p.v + ((size_t)work.b * p.S * p.Hkv + work.kvh) * D;
+    segb = p.seg + (size_t)work.b * p.S;
+  }
+  // does this wavefront's row block have anything in key tile t (bounds kb)?
+  CT_DEVICE bool wave_visits(const KeyTileBounds& kb, int t) const {
+    return blocks_interact(mine.min_nz, mine.max_id, mine.end_max, uniform(kb.min_nz),
+                           uniform(kb.max_id), t * kKeyTile);
+  }
+  CT_DEVICE bool interior(const KeyTileBounds& kb, int t) const {
+    return tile_is_interior(mine.uniform, mine.end_min, uniform(kb.uniform),
+                            t * kKeyTile + kKeyTile - 1);
+  }
+};
 
 // ---------------------------------------------------------------------------
 // Forward
 // ---------------------------------------------------------------------------
 template <int D, int HS>
 __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
-  constexpr int PB = 4 / HS;
   extern __shared__ __align__(16) char smem_raw[];
-  KvSmem<D> sm(smem_raw);
+  const lds_addr lds0 = lds_address_of(smem_raw);
+  constexpr int kStage = KvStage<D>::kBytes;
 
-  const QueryWork<HS> work(p);
-  const int l = lane_id(), j = l & 31, half = l >> 5, w = threadIdx.x >> 6;
-  const int nrb = p.S / 32;
-  const int* meta_b = p.meta + (size_t)work.b * nrb * kMetaW;
-  const int pos = work.rb * 32 + j;
-
-  QueryBlockBounds wq[PB];
-#pragma unroll
-  for (int i = 0; i < PB; ++i) wq[i] = query_block_bounds(meta_b, work.qt * PB + i);
-  const QueryBlockBounds mine = query_block_bounds(meta_b, work.rb);
-  int first = INT_MAX, last = -1;
-#pragma unroll
-  for (int i = 0; i < PB; ++i) {
-    first = min(first, wq[i].kv_first);
-    last = max(last, wq[i].kv_last);
-  }
-
+  const QueryTileContext<D, HS> ctx(p);
+  const int l = lane_id(), half = l >> 5, w = threadIdx.x >> 6;
+  const RowFragOffsets<D / 8> ro;
+  const TrFragOffsets<D / 8, KSlots::kAccum> to;
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
-  const size_t q_off = (((size_t)work.b * p.S + pos) * p.Hq + work.h) * D;
-  const int seg_q = p.seg[(size_t)work.b * p.S + pos];
-  const int end_q = p.end ? p.end[(size_t)work.b * p.S + pos] : pos;
-  const bool row_valid = seg_q != 0;
 
   bf16x8 qf[D / 16];
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks)
-    qf[ks] = scale_bf16x8(as_bf16x8(load_global16(p.q + q_off + 16 * ks + 8 * half)), p.scale);
+    qf[ks] = scale_bf16x8(as_bf16x8(load_global16(p.q + ctx.q_off + 16 * ks + 8 * half)), p.scale);
 
   f32x16 oacc[D / 32];
 #pragma unroll
@@ -276,86 +284,83 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
   float m_run = kNegInf;  // running max, log2 domain
   float l_run = 0.f;      // this lane's share of the running sum
 
-  const bf16* kbase = p.k + ((size_t)work.b * p.S * p.Hkv + work.kvh) * D;
-  const bf16* vbase = p.v + ((size_t)work.b * p.S * p.Hkv + work.kvh) * D;
-  const int* segb = p.seg + (size_t)work.b * p.S;
-
-  int t = (first <= last) ? next_tile<PB>(meta_b, wq, first, last) : last + 1;
-  if (t <= last) {
+  int t = ctx.first;
+  KeyTileBounds kb = {0, 0, 0};
+  if (t <= ctx.last) {
     KvRegs<D> regs;
-    kv_fetch<D>(regs, kbase, vbase, segb, kv_row_stride, t);
-    kv_commit<D>(regs, sm.k[0], sm.v[0], sm.seg[0]);
+    kv_fetch<D>(regs, ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride, t);
+    kb = key_tile_bounds(ctx.meta_b, t);
+    kv_commit<D>(regs, lds0);
   }
   __syncthreads();
-  int cur = 0;
-  while (t <= last) {
-    const int tn = next_tile<PB>(meta_b, wq, t + 1, last);
-    KvRegs<D> regs;
-    if (tn <= last) kv_fetch<D>(regs, kbase, vbase, segb, kv_row_stride, tn);
 
-    const KeyTileBounds kb = key_tile_bounds(meta_b, t);
-    if (blocks_interact(mine.min_nz, mine.max_id, mine.end_max, uniform(kb.min_nz),
-                        uniform(kb.max_id), t * kKeyTile)) {
+  auto step = [&](auto stage_tag) {
+    constexpr int CUR = decltype(stage_tag)::value;
+    const lds_addr stage = lds0 + CUR * kStage;
+    const bool more = t + 1 <= ctx.last;
+    KvRegs<D> regs;
+    KeyTileBounds nb = kb;
+    if (more) {
+      kv_fetch<D>(regs, ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride, t + 1);
+      nb = key_tile_bounds(ctx.meta_b, t + 1);
+    }
+    if (ctx.wave_visits(kb, t)) {
       f32x16 s[2];
-      scores_t<D>(sm.k[cur], qf, s);
-      const bool interior = tile_is_interior(mine.uniform, mine.end_min, uniform(kb.uniform),
-                                             t * kKeyTile + kKeyTile - 1);
+      scores_t<D>(stage + KvStage<D>::kK, ro, qf, s);
       float mx = kNegInf;
-      if (interior) {
-#pragma unroll
-        for (int kbk = 0; kbk < 2; ++kbk)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            s[kbk][r] *= kLog2e;
-            mx = fmaxf(mx, s[kbk][r]);
-          }
-      } else {
+      if (!ctx.interior(kb, t)) {
         unsigned allow[2];
-        tile_mask(sm.seg[cur], t, seg_q, end_q, row_valid, allow);
+        tile_mask(stage + KvStage<D>::kSeg, t, ctx.seg_q, ctx.end_q, ctx.row_valid, allow);
 #pragma unroll
         for (int kbk = 0; kbk < 2; ++kbk)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            s[kbk][r] = ((allow[kbk] >> r) & 1u) ? s[kbk][r] * kLog2e : kNegInf;
-            mx = fmaxf(mx, s[kbk][r]);
-          }
+          for (int r = 0; r < 16; ++r)
+            s[kbk][r] = ((allow[kbk] >> r) & 1u) ? s[kbk][r] : kNegInf;
       }
-      mx = fmaxf(mx, xor32(mx));
+#pragma unroll
+      for (int kbk = 0; kbk < 2; ++kbk)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kbk][r]);
+      mx = fmaxf(mx, xor32(mx)) * kLog2e;
       const float m_new = fmaxf(m_run, mx);
       const float m_use = (m_new == kNegInf) ? 0.f : m_new;
-      const float alpha = exp2_fast(m_run - m_use);
       float psum = 0.f;
 #pragma unroll
       for (int kbk = 0; kbk < 2; ++kbk)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          s[kbk][r] = exp2_fast(s[kbk][r] - m_use);
+          s[kbk][r] = exp2_fast(fmaf(s[kbk][r], kLog2e, -m_use));
           psum += s[kbk][r];
         }
-      l_run = l_run * alpha + psum;
-      m_run = m_new;
+      if (__any(m_new != m_run)) {
+        const float alpha = exp2_fast(m_run - m_use);
+        l_run *= alpha;
 #pragma unroll
-      for (int db = 0; db < D / 32; ++db)
+        for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-      accumulate_t<D>(sm.v[cur], s, oacc);
+          for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+        m_run = m_new;
+      }
+      l_run += psum;
+      accumulate_t<D>(stage + KvStage<D>::kV, to, s, oacc);
     }
-
-    if (tn <= last) kv_commit<D>(regs, sm.k[cur ^ 1], sm.v[cur ^ 1], sm.seg[cur ^ 1]);
+    if (more) kv_commit<D>(regs, lds0 + (CUR ^ 1) * kStage);
     __syncthreads();
-    t = tn;
-    cur ^= 1;
+    kb = nb;
+    ++t;
+  };
+  while (t <= ctx.last) {
+    step(std::integral_constant<int, 0>{});
+    if (t > ctx.last) break;
+    step(std::integral_constant<int, 1>{});
   }
 
   const float l_tot = l_run + xor32(l_run);
   const bool has = l_tot > 0.f;
   const float inv = has ? 1.f / l_tot : 0.f;
-  if (half == 0)
-    p.lse[((size_t)work.b * p.S + pos) * p.Hq + work.h] =
-        has ? (__logf(l_tot) + m_run * kLn2) : 0.f;
-  bf16* patch = reinterpret_cast<bf16*>(smem_raw) + w * 32 * D;
-  bf16* obase = p.out + (((size_t)work.b * p.S + work.rb * 32) * p.Hq + work.h) * D;
-  // store_rows_t applies one scale per lane = per query row (lane j <-> row j).
+  if (half == 0) p.lse[ctx.stat_off] = has ? (__logf(l_tot) + m_run * kLn2) : 0.f;
+  const lds_addr patch = lds0 + w * 32 * D * 2;
+  bf16* obase = p.out + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
   store_rows_t<D>(oacc, inv, patch, obase, q_row_stride);
 }
 

@@ -1,7 +1,7 @@
 // Tile-bounds buffer shared by the attention kernels.
 //
 // The sequence is cut into 32-position blocks ("row blocks"). For each block
-// the buffer holds CT_ATTN_META_WIDTH int32:
+// the buffer holds kMetaW int32:
 //   [0] min_nz   smallest nonzero segment id in the block, 0 if none
 //   [1] max_id   largest id among nonzero ids, 0 if none
 //   [2] uniform  the id shared by all 32 positions if they are equal and
@@ -9,7 +9,7 @@
 //   [3] end_min  min visible end over positions with id != 0 (INT_MAX if none)
 //   [4] end_max  max visible end over positions with id != 0 (-1 if none)
 //   [5] kv_first first 64-key tile this block (as queries) has to visit
-//   [6] kv_last  last such tile (-1 / INT_MAX pair when there is none)
+//   [6] kv_last  last such tile (INT_MAX / -1 pair when there is none)
 //   [7] q_first  first 32-row query block that has to visit this block (as keys)
 //   [8] q_last   last such block
 // [0], [1] and the "has to visit" predicate follow the reference's block
@@ -17,6 +17,13 @@
 // :377-412): two blocks interact iff both hold a nonzero id, their id ranges
 // overlap, and the key block starts at or before the query block's largest
 // visible end.
+//
+// After the [batch][nrb][kMetaW] table come four work-sorted schedules per
+// batch row, each a permutation that lists tiles by decreasing amount of
+// work, so that the hardware's in-order workgroup dispatch places the longest
+// tiles first:
+//   query tiles of 1, 2 and 4 row blocks (by number of key tiles to visit),
+//   128-key tiles (by number of query blocks to visit).
 #pragma once
 
 #include <limits.h>
@@ -37,6 +44,14 @@ enum MetaSlot {
   kQFirst = 7,
   kQLast = 8,
 };
+
+// ints of schedule data per batch row (nrb + nrb/2 + nrb/4 + nrb/4)
+__host__ __device__ inline int schedule_ints(int nrb) { return 2 * nrb; }
+// offset of the schedule for query tiles of pb row blocks (pb = 1, 2, 4) inside a row's schedules
+__host__ __device__ inline int query_schedule_offset(int nrb, int pb) {
+  return pb == 1 ? 0 : (pb == 2 ? nrb : nrb + nrb / 2);
+}
+__host__ __device__ inline int key_schedule_offset(int nrb) { return nrb + nrb / 2 + nrb / 4; }
 
 struct KeyTileBounds {
   int min_nz;

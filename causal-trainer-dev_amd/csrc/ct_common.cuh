@@ -13,6 +13,11 @@
 //   * "transposed" reads (ds_read_b64_tr_b16): 16 lanes read a 4-row x
 //     16-column patch and receive it transposed, which is how an operand
 //     whose contraction index runs along LDS rows is fetched.
+// LDS is always addressed through 32-bit byte addresses (lds_addr) and
+// address_space(3) accesses, so the compiler emits ds_* instructions with
+// immediate offsets instead of flat loads; the lane-dependent, swizzled part
+// of every fragment address is computed once per kernel (RowFragOffsets,
+// TrFragOffsets) and tile / block / stage bases are added as immediates.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -26,7 +31,10 @@ typedef bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_vs;
+typedef uint32_t lds_addr;
 
 #define CT_LDS __attribute__((address_space(3)))
 #define CT_DEVICE __device__ __forceinline__
@@ -57,7 +65,28 @@ CT_DEVICE float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 CT_DEVICE float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
 // ---------------------------------------------------------------------------
+// LDS access through 32-bit addresses
+// ---------------------------------------------------------------------------
+CT_DEVICE lds_addr lds_address_of(void* shared_ptr) {
+  return (lds_addr)(uintptr_t)(CT_LDS char*)shared_ptr;
+}
+template <class T>
+CT_DEVICE T lds_load(lds_addr a) {
+  return *(CT_LDS const T*)(uintptr_t)a;
+}
+template <class T>
+CT_DEVICE void lds_store(lds_addr a, T v) {
+  *(CT_LDS T*)(uintptr_t)a = v;
+}
+CT_DEVICE bf16x4_vs lds_load_tr(lds_addr a) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((CT_LDS bf16x4_vs*)(uintptr_t)a);
+}
+
+// ---------------------------------------------------------------------------
 // Swizzled LDS tiles. CPR = 16-byte chunks per row (row length / 8 elements).
+// The swizzle only depends on row bits 0..3, and only touches chunk bits
+// 0..3, so row offsets that are multiples of 16 rows and chunk offsets that
+// are multiples of 16 chunks are plain additive constants.
 // ---------------------------------------------------------------------------
 template <int CPR>
 CT_DEVICE int swizzle(int row) {
@@ -71,61 +100,68 @@ CT_DEVICE int swizzle(int row) {
   }
 }
 
-// Element offset of 16-byte chunk `chunk` of `row` inside a swizzled tile.
+// Byte offset of 16-byte chunk `chunk` of `row` inside a swizzled tile.
 template <int CPR>
-CT_DEVICE int tile_offset(int row, int chunk) {
-  return (row * CPR + (chunk ^ swizzle<CPR>(row))) * 8;
+CT_DEVICE int tile_byte_offset(int row, int chunk) {
+  return (row * CPR + (chunk ^ swizzle<CPR>(row))) * 16;
 }
 
+// Per-lane byte offsets of the k-contiguous MFMA fragments of a tile:
+// fragment (row block rb, k-step ks) of lane l is the 16 bytes at
+//   tile + rb * 32 * CPR * 16 + off[ks]
+// and holds row rb*32 + l%32, elements 16 ks + 8 (l/32) .. +7.
 template <int CPR>
-CT_DEVICE void tile_store_chunk(bf16* tile, int row, int chunk, uint4 value) {
-  *reinterpret_cast<uint4*>(tile + tile_offset<CPR>(row, chunk)) = value;
-}
+struct RowFragOffsets {
+  static constexpr int kSteps = CPR / 2;
+  int off[kSteps];
+  CT_DEVICE RowFragOffsets() {
+    const int l = lane_id(), row = l & 31, half = l >> 5;
+#pragma unroll
+    for (int ks = 0; ks < kSteps; ++ks) off[ks] = tile_byte_offset<CPR>(row, 2 * ks + half);
+  }
+  static constexpr int kRowBlockBytes = 32 * CPR * 16;
+};
 
-// k-contiguous operand: 8 consecutive elements of one row.
-template <int CPR>
-CT_DEVICE bf16x8 tile_read_row8(const bf16* tile, int row, int chunk) {
-  return *reinterpret_cast<const bf16x8*>(tile + tile_offset<CPR>(row, chunk));
-}
+// k-slot -> contraction index maps for transposed fragments.
+// "natural":  slot 8*half+e  <->  k0 + 8*half + e   (matches k-contiguous fragments)
+// "accum":    slot 8*half+e  <->  index held by accumulator registers 8t+e
+//             of a 32-row block, i.e. k0 + 4*half + e (e<4) and
+//             k0 + 8 + 4*half + (e-4) (e>=4), k0 = 16 t. This lets an MFMA
+//             result be fed back as an operand without cross-lane movement.
+enum class KSlots { kNatural, kAccum };
 
-// Transposed operand for mfma32: MFMA index i = lane % 32 runs along tile
-// columns col0 .. col0+31, and the 8 k-slots of this lane are tile rows
-// rowA .. rowA+3 then rowB .. rowB+3 (callers pass lane-half dependent
-// bases, see kslot_rows_*). Two ds_read_b64_tr_b16 per operand.
-template <int CPR>
-CT_DEVICE bf16x8 tile_read_tr8(const bf16* tile, int rowA, int rowB, int col0) {
-  const int l = lane_id();
-  const int p = l & 15;
-  const int col = col0 + (((l >> 4) & 1) << 4) + ((p & 3) << 2);
-  const int chunk = col >> 3;
-  const int sub = col & 4;
-  const int r0 = rowA + (p >> 2);
-  const int r1 = rowB + (p >> 2);
-  const bf16* a0 = tile + tile_offset<CPR>(r0, chunk) + sub;
-  const bf16* a1 = tile + tile_offset<CPR>(r1, chunk) + sub;
-  bf16x4_vs lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((CT_LDS bf16x4_vs*)(a0));
-  bf16x4_vs hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((CT_LDS bf16x4_vs*)(a1));
-  bf16x8 out;
-  out[0] = lo[0]; out[1] = lo[1]; out[2] = lo[2]; out[3] = lo[3];
-  out[4] = hi[0]; out[5] = hi[1]; out[6] = hi[2]; out[7] = hi[3];
-  return out;
-}
-
-// k-slot -> contraction index maps.
-// "natural":  slot 8*half+e  <->  k0 + 8*half + e        (matches tile_read_row8)
-// "accum":    slot 8*half+e  <->  index held by accumulator registers
-//             8t+e of a 32-row block, i.e. k0 + 4*half + e (e<4) and
-//             k0 + 8 + 4*half + (e-4) (e>=4), with k0 = 16*t.
-// This lets an MFMA result be fed back as the other operand of the next
-// MFMA without any cross-lane movement.
-CT_DEVICE void kslot_rows_natural(int k0, int half, int& rowA, int& rowB) {
-  rowA = k0 + 8 * half;
-  rowB = rowA + 4;
-}
-CT_DEVICE void kslot_rows_accum(int k0, int half, int& rowA, int& rowB) {
-  rowA = k0 + 4 * half;
-  rowB = rowA + 8;
-}
+// Per-lane byte offsets of transposed MFMA fragments: the MFMA row/column
+// index i = l % 32 runs along tile columns cb*32 .. cb*32+31 and the 8
+// k-slots of a lane are tile rows. Fragment (column block cb, k-step ks) is
+// two ds_read_b64_tr_b16 at
+//   tile + ks * 16 * CPR * 16 + (cb / 4) * 256 + off[second][cb % 4]
+template <int CPR, KSlots MAP>
+struct TrFragOffsets {
+  int off[2][4];
+  CT_DEVICE TrFragOffsets() {
+    const int l = lane_id(), p = l & 15, q16 = (l >> 4) & 1, half = l >> 5;
+#pragma unroll
+    for (int second = 0; second < 2; ++second) {
+      const int row = (MAP == KSlots::kNatural ? 8 * half + 4 * second : 4 * half + 8 * second) +
+                      (p >> 2);
+#pragma unroll
+      for (int cb = 0; cb < 4; ++cb) {
+        const int col = cb * 32 + 16 * q16 + 4 * (p & 3);
+        off[second][cb] = tile_byte_offset<CPR>(row, col >> 3) + (col & 4) * 2;
+      }
+    }
+  }
+  static constexpr int kStepBytes = 16 * CPR * 16;
+  CT_DEVICE bf16x8 load(lds_addr tile, int ks, int cb) const {
+    const lds_addr base = tile + ks * kStepBytes + (cb >> 2) * 256;
+    const bf16x4_vs lo = lds_load_tr(base + off[0][cb & 3]);
+    const bf16x4_vs hi = lds_load_tr(base + off[1][cb & 3]);
+    bf16x8 out;
+    out[0] = lo[0]; out[1] = lo[1]; out[2] = lo[2]; out[3] = lo[3];
+    out[4] = hi[0]; out[5] = hi[1]; out[6] = hi[2]; out[7] = hi[3];
+    return out;
+  }
+};
 
 // Pack accumulator registers 8t .. 8t+7 into a bf16 operand (round to nearest even).
 CT_DEVICE bf16x8 pack_acc8(const f32x16& c, int t) {
@@ -135,18 +171,11 @@ CT_DEVICE bf16x8 pack_acc8(const f32x16& c, int t) {
   return out;
 }
 
-CT_DEVICE uint4 load_global16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+CT_DEVICE u32x4 load_global16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+CT_DEVICE void store_global16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 
-CT_DEVICE bf16x8 as_bf16x8(uint4 v) {
-  union { uint4 u; bf16x8 b; } c;
-  c.u = v;
-  return c.b;
-}
-CT_DEVICE uint4 as_uint4(bf16x8 v) {
-  union { uint4 u; bf16x8 b; } c;
-  c.b = v;
-  return c.u;
-}
+CT_DEVICE bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+CT_DEVICE u32x4 as_u32x4(bf16x8 v) { return __builtin_bit_cast(u32x4, v); }
 
 // bf16 * bf16 rounded to bf16 (the product of two bf16 values is exact in f32).
 CT_DEVICE bf16x8 scale_bf16x8(bf16x8 v, float scale_as_bf16) {

@@ -95,7 +95,7 @@ CT_DEVICE void merge_stats(float& m, float& s, float m_o, float s_o) {
 
 __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* part, int chunks) {
   extern __shared__ __align__(16) char smem_raw[];
-  bf16* smem = reinterpret_cast<bf16*>(smem_raw);
+  const lds_addr smem = lds_address_of(smem_raw);
   __shared__ int unit_s;
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
@@ -271,8 +271,8 @@ __global__ __launch_bounds__(256) void cutce_zero_rows_kernel(const float* weigh
                                                               bf16* dhidden) {
   const int row = blockIdx.x;
   if (row >= N || weights[row] != 0.f) return;
-  uint4* dst = reinterpret_cast<uint4*>(dhidden + (size_t)row * d);
-  for (int c = threadIdx.x; c < d / 8; c += 256) dst[c] = make_uint4(0, 0, 0, 0);
+  u32x4* dst = reinterpret_cast<u32x4*>(dhidden + (size_t)row * d);
+  for (int c = threadIdx.x; c < d / 8; c += 256) dst[c] = u32x4{0u, 0u, 0u, 0u};
 }
 
 // G[slot, v - slab0] for one 256 x 256 tile.
@@ -280,7 +280,7 @@ __global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, const
                                                             const float* dy, int slab0,
                                                             int slab_tiles, bf16* G, int ldg) {
   extern __shared__ __align__(16) char smem_raw[];
-  bf16* smem = reinterpret_cast<bf16*>(smem_raw);
+  const lds_addr smem = lds_address_of(smem_raw);
   __shared__ float lse2_s[kGemmTile];
   __shared__ float fac_s[kGemmTile];
   __shared__ int tgt_s[kGemmTile];
@@ -354,7 +354,7 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
   // mode: 0 = single slab (store bf16), 1 = first slab (store f32), 2 = middle
   // slab (add f32), 3 = last slab (add, store bf16)
   extern __shared__ __align__(16) char smem_raw[];
-  bf16* smem = reinterpret_cast<bf16*>(smem_raw);
+  const lds_addr smem = lds_address_of(smem_raw);
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
   const int row_blocks = p.n_pad / kGemmTile, col_blocks = (p.d + kGemmTile - 1) / kGemmTile;
@@ -396,7 +396,7 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
 __global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const bf16* G, int ldg,
                                                           int slab0, int slab_tiles, bf16* dhead) {
   extern __shared__ __align__(16) char smem_raw[];
-  bf16* smem = reinterpret_cast<bf16*>(smem_raw);
+  const lds_addr smem = lds_address_of(smem_raw);
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
   const int m_blocks = (p.d + kGemmTile - 1) / kGemmTile;

@@ -18,21 +18,20 @@
 // element-wise loads.
 #pragma once
 
+#include <type_traits>
+
 #include "ct_common.cuh"
 
 namespace ct {
 
 constexpr int kGemmTile = 256;
 
-CT_DEVICE uint4 load_chunk_guarded(const bf16* p, int count, bool aligned) {
+CT_DEVICE u32x4 load_chunk_guarded(const bf16* p, int count, bool aligned) {
   if (count >= 8 && aligned) return load_global16(p);
-  union { uint4 u; unsigned short s[8]; } c;
-  c.u = make_uint4(0, 0, 0, 0);
-  const unsigned short* q = reinterpret_cast<const unsigned short*>(p);
+  bf16x8 v;
 #pragma unroll
-  for (int e = 0; e < 8; ++e)
-    if (e < count) c.s[e] = q[e];
-  return c.u;
+  for (int e = 0; e < 8; ++e) v[e] = e < count ? p[e] : (bf16)0.f;
+  return as_u32x4(v);
 }
 
 template <int BK>
@@ -42,7 +41,7 @@ struct KcLoader {
   static constexpr int kRowStep = 256 / CPR;  // rows between a thread's chunks
   static constexpr int kTileElems = kGemmTile * BK;
   const bf16* row_ptr[NCH];
-  uint4 regs[NCH];
+  u32x4 regs[NCH];
   int chunk, k_valid;
   bool aligned;
 
@@ -67,19 +66,20 @@ struct KcLoader {
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
       const int count = row_ptr[n] ? min(max(k_valid - k, 0), 8) : 0;
-      regs[n] = count ? load_chunk_guarded(row_ptr[n] + k, count, aligned) : make_uint4(0, 0, 0, 0);
+      regs[n] = count ? load_chunk_guarded(row_ptr[n] + k, count, aligned) : u32x4{0u, 0u, 0u, 0u};
     }
   }
-  CT_DEVICE void commit(bf16* tile) const {
+  CT_DEVICE void commit(lds_addr tile) const {
     const int tid = threadIdx.x;
 #pragma unroll
     for (int n = 0; n < NCH; ++n)
-      tile_store_chunk<CPR>(tile, tid / CPR + n * kRowStep, chunk, regs[n]);
+      lds_store<u32x4>(tile + tile_byte_offset<CPR>(tid / CPR + n * kRowStep, chunk), regs[n]);
   }
   // fragment for MFMA rows/cols first .. first+31, contraction steps 16*ks .. 16*ks+15
-  static CT_DEVICE bf16x8 frag(const bf16* tile, int ks, int first) {
-    const int l = lane_id();
-    return tile_read_row8<CPR>(tile, first + (l & 31), 2 * ks + (l >> 5));
+  typedef RowFragOffsets<CPR> FragOffsets;
+  // `wave_first` (multiple of 128) is the wavefront's first row, `i` its 32-row block.
+  static CT_DEVICE bf16x8 frag(lds_addr tile, const FragOffsets& fo, int ks, int wave_first, int i) {
+    return lds_load<bf16x8>(tile + (wave_first / 32 + i) * FragOffsets::kRowBlockBytes + fo.off[ks]);
   }
 };
 
@@ -91,7 +91,7 @@ struct McLoader {
   const bf16* base;
   const int* row_index;
   long ld;
-  uint4 regs[NCH];
+  u32x4 regs[NCH];
   int m0, cols_valid, k_valid;
   bool aligned;
 
@@ -117,26 +117,27 @@ struct McLoader {
         const long src = row_index ? row_index[k] : k;
         regs[n] = load_chunk_guarded(base + src * ld + m, count, aligned);
       } else {
-        regs[n] = make_uint4(0, 0, 0, 0);
+        regs[n] = u32x4{0u, 0u, 0u, 0u};
       }
     }
   }
-  CT_DEVICE void commit(bf16* tile) const {
+  CT_DEVICE void commit(lds_addr tile) const {
     const int tid = threadIdx.x;
 #pragma unroll
-    for (int n = 0; n < NCH; ++n) tile_store_chunk<CPR>(tile, tid / CPR + 8 * n, tid % CPR, regs[n]);
+    for (int n = 0; n < NCH; ++n)
+      lds_store<u32x4>(tile + tile_byte_offset<CPR>(tid / CPR + 8 * n, tid % CPR), regs[n]);
   }
-  static CT_DEVICE bf16x8 frag(const bf16* tile, int ks, int first) {
-    int rowA, rowB;
-    kslot_rows_natural(16 * ks, lane_id() >> 5, rowA, rowB);
-    return tile_read_tr8<CPR>(tile, rowA, rowB, first);
+  typedef TrFragOffsets<CPR, KSlots::kNatural> FragOffsets;
+  static CT_DEVICE bf16x8 frag(lds_addr tile, const FragOffsets& fo, int ks, int wave_first, int i) {
+    return fo.load(tile + (wave_first / 128) * 256, ks, i);
   }
 };
 
 template <int BK>
 struct GemmSmem {
-  static constexpr int kStageElems = 2 * kGemmTile * BK;
-  static constexpr size_t kBytes = 2 * kStageElems * sizeof(bf16);
+  static constexpr int kTileBytes = kGemmTile * BK * 2;
+  static constexpr int kStageBytes = 2 * kTileBytes;
+  static constexpr size_t kBytes = 2 * kStageBytes;
 };
 
 struct GemmAcc {
@@ -152,19 +153,22 @@ struct GemmAcc {
 // acc += A[m-tile, k_begin:k_end] * B[n-tile, k_begin:k_end]^T. Must be called by
 // all 256 threads; ends with the LDS tiles free for reuse.
 template <int BK, class ALoader, class BLoader>
-CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, bf16* smem, GemmAcc& acc) {
+CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, lds_addr smem,
+                         GemmAcc& acc) {
   const int w = threadIdx.x >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
-  bf16* a_tile[2] = {smem, smem + GemmSmem<BK>::kStageElems};
-  bf16* b_tile[2] = {smem + kGemmTile * BK, smem + GemmSmem<BK>::kStageElems + kGemmTile * BK};
+  constexpr int kTile = GemmSmem<BK>::kTileBytes, kStage = GemmSmem<BK>::kStageBytes;
   if (k_begin >= k_end) return;
+  const typename ALoader::FragOffsets afo;
+  const typename BLoader::FragOffsets bfo;
   A.fetch(k_begin);
   B.fetch(k_begin);
-  A.commit(a_tile[0]);
-  B.commit(b_tile[0]);
+  A.commit(smem);
+  B.commit(smem + kTile);
   __syncthreads();
-  int cur = 0;
+  lds_addr cur = smem, nxt = smem + kStage;
   for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+    const lds_addr a_tile = cur, b_tile = cur + kTile;
     const bool more = k0 + BK < k_end;
     if (more) {
       A.fetch(k0 + BK);
@@ -175,8 +179,8 @@ CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, bf16* s
       bf16x8 af[4], bfr[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        af[i] = ALoader::frag(a_tile[cur], ks, wm + 32 * i);
-        bfr[i] = BLoader::frag(b_tile[cur], ks, wn + 32 * i);
+        af[i] = ALoader::frag(a_tile, afo, ks, wm, i);
+        bfr[i] = BLoader::frag(b_tile, bfo, ks, wn, i);
       }
 #pragma unroll
       for (int i = 0; i < 4; ++i)
@@ -184,11 +188,13 @@ CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, bf16* s
         for (int jn = 0; jn < 4; ++jn) acc.c[i][jn] = mfma32(af[i], bfr[jn], acc.c[i][jn]);
     }
     if (more) {
-      A.commit(a_tile[cur ^ 1]);
-      B.commit(b_tile[cur ^ 1]);
+      A.commit(nxt);
+      B.commit(nxt + kTile);
     }
     __syncthreads();
-    cur ^= 1;
+    const lds_addr tmp = cur;
+    cur = nxt;
+    nxt = tmp;
   }
 }
 

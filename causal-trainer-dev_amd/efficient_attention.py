@@ -299,8 +299,18 @@ def prepare_attention_metadata(canonical_segment_ids, *, mesh, profile,
         q_block_segments=q_summary,
         kv_block_segments=kv_summary,
         attention_end=ends,
-        tile_bounds=bounds.view(batch, sequence // 32, _lib.ATTN_META_WIDTH),
+        tile_bounds=bounds,
     )
+
+
+def tile_bounds_table(metadata: AttentionMetadata) -> torch.Tensor:
+    """The ``[B, S/32, 12]`` per-row-block table at the head of ``metadata.tile_bounds``
+    (the work-sorted schedules follow it in the same buffer)."""
+
+    batch, sequence = metadata.query_segment_ids.shape
+    blocks = sequence // 32
+    return metadata.tile_bounds[: batch * blocks * _lib.ATTN_META_WIDTH].view(
+        batch, blocks, _lib.ATTN_META_WIDTH)
 
 
 def _validate_metadata(metadata, query_shape, profile) -> None:
@@ -322,9 +332,8 @@ def _validate_metadata(metadata, query_shape, profile) -> None:
             raise ValueError(f"metadata.{name} must have shape {shape}, got {tuple(value.shape)}")
         if value.dtype != torch.int32:
             raise TypeError(f"metadata.{name} must have dtype int32, got {value.dtype}")
-    if metadata.tile_bounds is None or tuple(metadata.tile_bounds.shape) != (
-        batch, sequence // 32, _lib.ATTN_META_WIDTH
-    ):
+    expected_bytes = _lib.load().ct_attn_meta_bytes(batch, sequence)
+    if metadata.tile_bounds is None or metadata.tile_bounds.numel() * 4 != expected_bytes:
         raise ValueError("metadata.tile_bounds is missing; build it with prepare_attention_metadata")
 
 
@@ -460,5 +469,6 @@ __all__ = [
     "efficient_attention",
     "prepare_attention_metadata",
     "resolve_attention_profile",
+    "tile_bounds_table",
     "validate_attention_profile",
 ]

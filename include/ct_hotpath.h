@@ -61,10 +61,11 @@ void ct_set_launch_hook(ct_launch_hook hook, void* user);
  * Attention
  * --------------------------------------------------------------------- */
 
-/* Number of int32 per 32-position block in the tile-bounds buffer. */
+/* Number of int32 per 32-position block in the per-block table that opens the
+ * tile-bounds buffer; the table is followed by work-sorted tile schedules. */
 #define CT_ATTN_META_WIDTH 12
 
-/* Bytes of the tile-bounds buffer for [batch, seq] segment ids. */
+/* Bytes of the tile-bounds buffer (table + schedules) for [batch, seq] segment ids. */
 size_t ct_attn_meta_bytes(int32_t batch, int32_t seq);
 
 /*

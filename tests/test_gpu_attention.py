@@ -232,7 +232,7 @@ def test_metadata_matches_oracle_bit_exact(ct, gpu):
         np.testing.assert_array_equal(metadata.q_block_segments.cpu().numpy(), q_summary)
         np.testing.assert_array_equal(metadata.kv_block_segments.cpu().numpy(), kv_summary)
         # tile bounds: every allowed pair lies inside the advertised visit ranges
-        bounds = metadata.tile_bounds.cpu().numpy()
+        bounds = ct.tile_bounds_table(metadata).cpu().numpy()
         allowed = ref.allowed_from_canonical(ids, ends)
         for b in range(2):
             for rb in range(1024 // 32):
@@ -246,6 +246,17 @@ def test_metadata_matches_oracle_bit_exact(ct, gpu):
                     assert bounds[b, rb, 7] <= queries[0] // 32 and queries[-1] // 32 <= bounds[b, rb, 8]
                 block = ids[b, rb * 32:(rb + 1) * 32]
                 assert bounds[b, rb, 2] == (block[0] if (block == block[0]).all() and block[0] != 0 else 0)
+        # schedules: permutations, ordered by non-increasing work
+        blocks = 1024 // 32
+        schedules = metadata.tile_bounds.cpu().numpy()[2 * blocks * 12:].reshape(2, 2 * blocks)
+        for b in range(2):
+            spans = np.where(bounds[b, :, 6] >= bounds[b, :, 5], bounds[b, :, 6] - bounds[b, :, 5] + 1, 0)
+            order = schedules[b, :blocks]
+            assert sorted(order.tolist()) == list(range(blocks))
+            assert (np.diff(spans[order]) <= 0).all()
+            for offset, count in ((blocks, blocks // 2), (blocks + blocks // 2, blocks // 4),
+                                  (blocks + blocks // 2 + blocks // 4, blocks // 4)):
+                assert sorted(schedules[b, offset:offset + count].tolist()) == list(range(count))
 
 
 def test_delta_pass_matches_torch(ct, gpu):

@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol(ct):
 
 def test_size_queries_need_no_gpu(ct):
     library = ct._lib.load()
-    assert library.ct_attn_meta_bytes(4, 4096) == 4 * (4096 // 32) * 12 * 4
+    assert library.ct_attn_meta_bytes(4, 4096) == 4 * (4096 // 32) * (12 + 2) * 4
     assert library.ct_attn_meta_bytes(0, 128) == 0
     shape = ct._lib.CutceShape(16384, 4096, 128256)
     fwd = library.ct_cutce_fwd_workspace_bytes(ctypes.byref(shape))
