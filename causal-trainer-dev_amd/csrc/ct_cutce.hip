@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
       tl[nb] = 0.f;
     }
     KcLoader<kBK> B;
-    B.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned);
+    B.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true);
 
     const int vt_end = min((chunk + 1) * kTilesPerChunk, vocab_tiles);
     for (int vt = chunk * kTilesPerChunk; vt < vt_end; ++vt) {
@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, const
     tgt_s[tid] = t;
   }
   KcLoader<kBK> A;
-  A.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned);
+  A.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true);
   McLoader<kBK> B;
   B.init(p.head, p.V, nullptr, v0, p.V, p.d, p.head_aligned);
   GemmAcc acc;
@@ -365,9 +365,9 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
   if (n0 >= n_act) return;
 
   KcLoader<kBK> A;
-  A.init(G, ldg, nullptr, n0, n_act, slab_width, true);
+  A.init(G, ldg, nullptr, n0, p.n_pad, slab_width, true, false);
   KcLoader<kBK> B;
-  B.init(p.head + slab0, p.V, nullptr, c0, p.d, min(slab_width, p.V - slab0), p.head_aligned);
+  B.init(p.head + slab0, p.V, nullptr, c0, p.d, min(slab_width, p.V - slab0), p.head_aligned, false);
   GemmAcc acc;
   acc.clear();
   gemm_tile<kBK>(A, B, 0, slab_width, smem, acc);

@@ -34,50 +34,69 @@ CT_DEVICE u32x4 load_chunk_guarded(const bf16* p, int count, bool aligned) {
   return as_u32x4(v);
 }
 
+// Both loaders have a straight-line fast path (every row / column / k of the
+// step in range and 16-byte aligned: unconditional 16-byte loads at
+// uniform-base + 32-bit lane offsets) and a guarded element-wise path that
+// zero fills; the choice is uniform over the workgroup.
 template <int BK>
 struct KcLoader {
   static constexpr int CPR = BK / 8;
   static constexpr int NCH = BK / 8;          // 16-byte chunks per thread per step
   static constexpr int kRowStep = 256 / CPR;  // rows between a thread's chunks
-  static constexpr int kTileElems = kGemmTile * BK;
-  const bf16* row_ptr[NCH];
+  const char* base;    // uniform
+  unsigned voff[NCH];  // byte offset of this thread's chunk n from base (k = 0)
   u32x4 regs[NCH];
-  int chunk, k_valid;
-  bool aligned;
+  int lds_off, k_valid, row_mask;
+  bool fast;
 
-  // rows m0 .. m0+255 of `base` (leading dimension ld), optionally gathered
-  // through row_index; rows >= rows_valid and k >= k_valid read as zero.
-  CT_DEVICE void init(const bf16* base, long ld, const int* row_index, int m0, int rows_valid,
-                      int k_valid_, bool aligned_) {
-    const int tid = threadIdx.x;
-    chunk = tid % CPR;
+  // rows m0 .. m0+255 of `base_` (leading dimension ld elements), optionally
+  // gathered through row_index. Rows >= rows_valid read as zero, or, with
+  // alias_invalid_rows, as a copy of the first row (for callers that discard
+  // those rows); k >= k_valid reads as zero.
+  CT_DEVICE void init(const bf16* base_, long ld, const int* row_index, int m0, int rows_valid,
+                      int k_valid_, bool aligned, bool alias_invalid_rows) {
+    const int tid = threadIdx.x, chunk = tid % CPR, row0 = tid / CPR;
     k_valid = k_valid_;
-    aligned = aligned_;
+    lds_off = tile_byte_offset<CPR>(row0, chunk);
+    const bool gathered = row_index != nullptr;
+    base = reinterpret_cast<const char*>(gathered ? base_ : base_ + (size_t)m0 * ld);
+    row_mask = 0;
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
-      const int gm = m0 + tid / CPR + n * kRowStep;
-      const bool ok = gm < rows_valid;
-      const long src = ok ? (row_index ? row_index[gm] : gm) : 0;
-      row_ptr[n] = ok ? base + src * ld : nullptr;
+      const int r = row0 + n * kRowStep;
+      const bool ok = m0 + r < rows_valid;
+      if (ok || alias_invalid_rows) row_mask |= 1 << n;
+      const long src = gathered ? row_index[ok ? m0 + r : 0] : (ok ? r : 0);
+      voff[n] = (unsigned)((src * ld + chunk * 8) * 2);
     }
+    fast = aligned && (alias_invalid_rows || m0 + kGemmTile <= rows_valid);
   }
   CT_DEVICE void fetch(int k0) {
-    const int k = k0 + chunk * 8;
+    if (fast && k0 + BK <= k_valid) {
+      const char* p = base + (size_t)k0 * 2;
 #pragma unroll
-    for (int n = 0; n < NCH; ++n) {
-      const int count = row_ptr[n] ? min(max(k_valid - k, 0), 8) : 0;
-      regs[n] = count ? load_chunk_guarded(row_ptr[n] + k, count, aligned) : u32x4{0u, 0u, 0u, 0u};
+      for (int n = 0; n < NCH; ++n) regs[n] = load_global16(p + voff[n]);
+    } else {
+      const int k = k0 + (threadIdx.x % CPR) * 8;
+      const int count = min(max(k_valid - k, 0), 8);
+#pragma unroll
+      for (int n = 0; n < NCH; ++n) {
+        const bool ok = (row_mask >> n) & 1;
+        regs[n] = (ok && count) ? load_chunk_guarded(reinterpret_cast<const bf16*>(
+                                                         base + (size_t)k0 * 2 + voff[n]),
+                                                     count, false)
+                                : u32x4{0u, 0u, 0u, 0u};
+      }
     }
   }
   CT_DEVICE void commit(lds_addr tile) const {
-    const int tid = threadIdx.x;
 #pragma unroll
     for (int n = 0; n < NCH; ++n)
-      lds_store<u32x4>(tile + tile_byte_offset<CPR>(tid / CPR + n * kRowStep, chunk), regs[n]);
+      lds_store<u32x4>(tile + lds_off + n * (kRowStep * CPR * 16), regs[n]);
   }
-  // fragment for MFMA rows/cols first .. first+31, contraction steps 16*ks .. 16*ks+15
+  // fragment for the wavefront's 32-row block i, contraction steps 16*ks .. 16*ks+15;
+  // `wave_first` (multiple of 128) is the wavefront's first row.
   typedef RowFragOffsets<CPR> FragOffsets;
-  // `wave_first` (multiple of 128) is the wavefront's first row, `i` its 32-row block.
   static CT_DEVICE bf16x8 frag(lds_addr tile, const FragOffsets& fo, int ks, int wave_first, int i) {
     return lds_load<bf16x8>(tile + (wave_first / 32 + i) * FragOffsets::kRowBlockBytes + fo.off[ks]);
   }
@@ -87,45 +106,62 @@ template <int BK>
 struct McLoader {
   static constexpr int CPR = kGemmTile / 8;  // 32
   static constexpr int NCH = BK / 8;
-  static constexpr int kTileElems = kGemmTile * BK;
-  const bf16* base;
+  const char* base;  // uniform: column m0 of row 0
   const int* row_index;
   long ld;
+  unsigned voff[NCH];
+  int lds_off[NCH];
   u32x4 regs[NCH];
-  int m0, cols_valid, k_valid;
-  bool aligned;
+  int count, k_valid;
+  bool fast;
 
-  // columns m0 .. m0+255 of `base`; contraction rows optionally gathered.
-  CT_DEVICE void init(const bf16* base_, long ld_, const int* row_index_, int m0_, int cols_valid_,
-                      int k_valid_, bool aligned_) {
-    base = base_;
-    ld = ld_;
+  // columns m0 .. m0+255 of `base_`; contraction rows optionally gathered.
+  // Columns >= cols_valid and rows >= k_valid read as zero.
+  CT_DEVICE void init(const bf16* base_, long ld_, const int* row_index_, int m0, int cols_valid,
+                      int k_valid_, bool aligned) {
+    const int tid = threadIdx.x, col = (tid % CPR) * 8, row0 = tid / CPR;
+    base = reinterpret_cast<const char*>(base_ + m0);
     row_index = row_index_;
-    m0 = m0_;
-    cols_valid = cols_valid_;
+    ld = ld_;
     k_valid = k_valid_;
-    aligned = aligned_;
-  }
-  CT_DEVICE void fetch(int k0) {
-    const int tid = threadIdx.x;
-    const int m = m0 + (tid % CPR) * 8;
-    const int count = min(max(cols_valid - m, 0), 8);
+    count = min(max(cols_valid - m0 - col, 0), 8);
+    fast = aligned && m0 + kGemmTile <= cols_valid;
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
-      const int k = k0 + tid / CPR + 8 * n;
-      if (k < k_valid && count) {
-        const long src = row_index ? row_index[k] : k;
-        regs[n] = load_chunk_guarded(base + src * ld + m, count, aligned);
+      const int r = row0 + 8 * n;
+      lds_off[n] = tile_byte_offset<CPR>(r, tid % CPR);
+      voff[n] = (unsigned)(((row_index ? 0 : (long)r * ld) + col) * 2);
+    }
+  }
+  CT_DEVICE void fetch(int k0) {
+    const int row0 = threadIdx.x / CPR;
+    if (fast && k0 + BK <= k_valid) {
+      if (row_index) {
+#pragma unroll
+        for (int n = 0; n < NCH; ++n)
+          regs[n] = load_global16(base + (size_t)row_index[k0 + row0 + 8 * n] * ld * 2 + voff[n]);
       } else {
-        regs[n] = u32x4{0u, 0u, 0u, 0u};
+        const char* p = base + (size_t)k0 * ld * 2;
+#pragma unroll
+        for (int n = 0; n < NCH; ++n) regs[n] = load_global16(p + voff[n]);
+      }
+    } else {
+#pragma unroll
+      for (int n = 0; n < NCH; ++n) {
+        const int k = k0 + row0 + 8 * n;
+        if (k < k_valid && count) {
+          const size_t src = row_index ? (size_t)row_index[k] : (size_t)k0;
+          const char* p = base + src * ld * 2 + voff[n];
+          regs[n] = load_chunk_guarded(reinterpret_cast<const bf16*>(p), count, false);
+        } else {
+          regs[n] = u32x4{0u, 0u, 0u, 0u};
+        }
       }
     }
   }
   CT_DEVICE void commit(lds_addr tile) const {
-    const int tid = threadIdx.x;
 #pragma unroll
-    for (int n = 0; n < NCH; ++n)
-      lds_store<u32x4>(tile + tile_byte_offset<CPR>(tid / CPR + 8 * n, tid % CPR), regs[n]);
+    for (int n = 0; n < NCH; ++n) lds_store<u32x4>(tile + lds_off[n], regs[n]);
   }
   typedef TrFragOffsets<CPR, KSlots::kNatural> FragOffsets;
   static CT_DEVICE bf16x8 frag(lds_addr tile, const FragOffsets& fo, int ks, int wave_first, int i) {
