@@ -21,7 +21,7 @@ namespace ct {
 // dQ
 // ---------------------------------------------------------------------------
 template <int D, int HS>
-__global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr lds0 = lds_address_of(smem_raw);
   constexpr int kStage = KvStage<D>::kBytes;
@@ -45,24 +45,23 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
 #pragma unroll
   for (int db = 0; db < D / 32; ++db) dqacc[db] = zero16();
 
+  const KvFetcher<D> fetch(ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride);
   int t = ctx.first;
   KeyTileBounds kb = {0, 0, 0};
   if (t <= ctx.last) {
-    KvRegs<D> regs;
-    kv_fetch<D>(regs, ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride, t);
+    fetch.issue(t, lds0);
     kb = key_tile_bounds(ctx.meta_b, t);
-    kv_commit<D>(regs, lds0);
   }
+  dma_wait_all();
   __syncthreads();
 
   auto step = [&](auto stage_tag) {
     constexpr int CUR = decltype(stage_tag)::value;
     const lds_addr stage = lds0 + CUR * kStage;
     const bool more = t + 1 <= ctx.last;
-    KvRegs<D> regs;
     KeyTileBounds nb = kb;
     if (more) {
-      kv_fetch<D>(regs, ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride, t + 1);
+      fetch.issue(t + 1, lds0 + (CUR ^ 1) * kStage);
       nb = key_tile_bounds(ctx.meta_b, t + 1);
     }
     if (ctx.wave_visits(kb, t)) {
@@ -82,7 +81,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(AttnParams p) {
         }
       accumulate_t<D>(stage + KvStage<D>::kK, to, s, dqacc);
     }
-    if (more) kv_commit<D>(regs, lds0 + (CUR ^ 1) * kStage);
+    dma_wait_all();
     __syncthreads();
     kb = nb;
     ++t;
@@ -116,29 +115,33 @@ struct QdoStage {
   static constexpr int kEnd = kSeg + kQueryTile * 4;
   static constexpr int kBytes = kEnd + kQueryTile * 4;
   static constexpr int kPatchBytes = 4 * 32 * D * 2;
-  static constexpr int kTotalBytes = (2 * kBytes > kPatchBytes) ? 2 * kBytes : kPatchBytes;
+  // resident V rows of the workgroup's 128 keys (32 per wavefront), after the two stages
+  static constexpr int kVResident = 2 * kBytes;
+  static constexpr int kTotalBytes = 2 * kBytes + kPatchBytes;
 };
 
+// Q goes through registers (it is rescaled on the way); dO is copied asynchronously.
 template <int D>
 struct QdoRegs {
   static constexpr int kChunks = kQueryTile * (D / 8) / 256;
   u32x4 q[kChunks];
-  u32x4 dout[kChunks];
   float lse2, delta;
   int seg, end;
 };
 
 template <int D>
-CT_DEVICE void qdo_fetch(QdoRegs<D>& r, const AttnParams& p, int b, int h, int qb) {
+CT_DEVICE void qdo_fetch(QdoRegs<D>& r, const TileDma<kQueryTile, D / 8>& dma, const AttnParams& p,
+                         int b, int h, int qb, lds_addr stage) {
   constexpr int CPR = D / 8;
   const int tid = threadIdx.x;
+  const size_t origin = (((size_t)b * p.S + qb * kQueryTile) * p.Hq + h) * D;
+  dma.issue(reinterpret_cast<const char*>(p.dout + origin), (size_t)p.Hq * D * 2,
+            stage + QdoStage<D>::kDo);
 #pragma unroll
   for (int n = 0; n < QdoRegs<D>::kChunks; ++n) {
     const int e = tid + 256 * n;
     const int row = e / CPR, c = e % CPR;
-    const size_t off = (((size_t)b * p.S + qb * kQueryTile + row) * p.Hq + h) * D + c * 8;
-    r.q[n] = load_global16(p.q + off);
-    r.dout[n] = load_global16(p.dout + off);
+    r.q[n] = load_global16(p.q + origin + (size_t)row * p.Hq * D + c * 8);
   }
   if (tid < kQueryTile) {
     const int pos = qb * kQueryTile + tid;
@@ -159,7 +162,6 @@ CT_DEVICE void qdo_commit(const QdoRegs<D>& r, lds_addr stage, float scale) {
     const int e = tid + 256 * n;
     const int off = tile_byte_offset<CPR>(e / CPR, e % CPR);
     lds_store<u32x4>(stage + QdoStage<D>::kQ + off, as_u32x4(scale_bf16x8(as_bf16x8(r.q[n]), scale)));
-    lds_store<u32x4>(stage + QdoStage<D>::kDo + off, r.dout[n]);
   }
   if (tid < kQueryTile) {
     lds_store<float>(stage + QdoStage<D>::kLse + tid * 4, r.lse2);
@@ -216,7 +218,7 @@ CT_DEVICE void store_rows(const f32x16* acc, lds_addr patch, bf16* gbase, size_t
 }
 
 template <int D>
-__global__ __launch_bounds__(256) void attn_dkv_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr lds0 = lds_address_of(smem_raw);
   constexpr int kStage = QdoStage<D>::kBytes;
@@ -251,11 +253,15 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(AttnParams p) {
   const size_t kv_row_stride = (size_t)p.Hkv * D;
   const size_t kv_off = (((size_t)b * p.S + key) * p.Hkv + kvh) * D;
 
-  bf16x8 kf[D / 16], vf[D / 16];
+  // K fragments stay in registers; V fragments are parked in LDS (this wavefront's
+  // private 32-row patch) and re-read per block, which keeps the kernel under 256
+  // registers so that two workgroups share a CU.
+  const lds_addr vpatch = lds0 + QdoStage<D>::kVResident + w * 32 * D * 2;
+  bf16x8 kf[D / 16];
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) {
     kf[ks] = as_bf16x8(load_global16(p.k + kv_off + 16 * ks + 8 * half));
-    vf[ks] = as_bf16x8(load_global16(p.v + kv_off + 16 * ks + 8 * half));
+    lds_store<u32x4>(vpatch + ro.off[ks], load_global16(p.v + kv_off + 16 * ks + 8 * half));
   }
   f32x16 dkacc[D / 32], dvacc[D / 32];
 #pragma unroll
@@ -268,11 +274,13 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(AttnParams p) {
   const int nq = (q_lo <= q_hi) ? (q_hi - q_lo + 1) : 0;
   const int items = nq * g;
   int it = 0, qb = q_lo, head = kvh * g;
+  const TileDma<kQueryTile, D / 8> dma;
   if (it < items) {
     QdoRegs<D> regs;
-    qdo_fetch<D>(regs, p, b, head, qb);
+    qdo_fetch<D>(regs, dma, p, b, head, qb, lds0);
     qdo_commit<D>(regs, lds0, p.scale);
   }
+  dma_wait_all();
   __syncthreads();
 
   auto step = [&](auto stage_tag) {
@@ -285,7 +293,7 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(AttnParams p) {
       ++head_next;
     }
     QdoRegs<D> regs;
-    if (more) qdo_fetch<D>(regs, p, b, head_next, qb_next);
+    if (more) qdo_fetch<D>(regs, dma, p, b, head_next, qb_next, lds0 + (CUR ^ 1) * kStage);
 
     const int* qm = meta_b + qb * kMetaW;
     const int q_min = uniform(qm[kMinNz]), q_max = uniform(qm[kMaxId]),
@@ -293,7 +301,11 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(AttnParams p) {
               q_uni = uniform(qm[kUniform]);
     if (blocks_interact(q_min, q_max, q_end_max, my_min, my_max, my_rb * 32)) {
       f32x16 s = rows_times_frags<D>(stage + QdoStage<D>::kQ, ro, kf);
-      f32x16 dp = rows_times_frags<D>(stage + QdoStage<D>::kDo, ro, vf);
+      f32x16 dp = zero16();
+#pragma unroll
+      for (int ks = 0; ks < D / 16; ++ks)
+        dp = mfma32(lds_load<bf16x8>(stage + QdoStage<D>::kDo + ro.off[ks]),
+                    lds_load<bf16x8>(vpatch + ro.off[ks]), dp);
       const bool interior = tile_is_interior(q_uni, q_end_min, my_uni, my_rb * 32 + 31);
       f32x16 prob;
 #pragma unroll
@@ -319,6 +331,7 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(AttnParams p) {
       accumulate_keys<D>(stage + QdoStage<D>::kQ, to, dp, dkacc);
     }
     if (more) qdo_commit<D>(regs, lds0 + (CUR ^ 1) * kStage, p.scale);
+    dma_wait_all();
     __syncthreads();
     ++it;
     qb = qb_next;
@@ -330,7 +343,7 @@ __global__ __launch_bounds__(256) void attn_dkv_kernel(AttnParams p) {
     step(std::integral_constant<int, 1>{});
   }
 
-  const lds_addr patch = lds0 + w * 32 * D * 2;
+  const lds_addr patch = vpatch;  // V fragments are no longer needed
   const size_t out_off = (((size_t)b * p.S + my_rb * 32) * p.Hkv + kvh) * D;
   store_rows<D>(dkacc, patch, p.dk + out_off, kv_row_stride);
   __builtin_amdgcn_wave_barrier();

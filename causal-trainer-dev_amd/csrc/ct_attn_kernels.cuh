@@ -64,43 +64,25 @@ struct KvStage {
   static constexpr int kBytes = 2 * kTileBytes + kKeyTile * 4;
 };
 
+// Asynchronous fetch of key tile `tile` (K rows, V rows, segment ids) into an LDS stage.
 template <int D>
-struct KvRegs {
-  static constexpr int kChunks = kKeyTile * (D / 8) / 256;
-  u32x4 k[kChunks];
-  u32x4 v[kChunks];
-  int seg;
+struct KvFetcher {
+  TileDma<kKeyTile, D / 8> dma;
+  const char* kbase;
+  const char* vbase;
+  const int* segb;
+  size_t row_stride_bytes;
+  CT_DEVICE KvFetcher(const bf16* k, const bf16* v, const int* seg, size_t row_stride_elems)
+      : kbase(reinterpret_cast<const char*>(k)), vbase(reinterpret_cast<const char*>(v)),
+        segb(seg), row_stride_bytes(row_stride_elems * 2) {}
+  CT_DEVICE void issue(int tile, lds_addr stage) const {
+    const size_t origin = (size_t)tile * kKeyTile * row_stride_bytes;
+    dma.issue(kbase + origin, row_stride_bytes, stage + KvStage<D>::kK);
+    dma.issue(vbase + origin, row_stride_bytes, stage + KvStage<D>::kV);
+    if (threadIdx.x < 16)  // 64 ids = 16 lanes x 16 bytes, linear layout
+      dma16(segb + tile * kKeyTile + threadIdx.x * 4, stage + KvStage<D>::kSeg);
+  }
 };
-
-template <int D>
-CT_DEVICE void kv_fetch(KvRegs<D>& r, const bf16* kbase, const bf16* vbase, const int* segb,
-                        size_t row_stride, int tile) {
-  constexpr int CPR = D / 8;
-  const int tid = threadIdx.x;
-#pragma unroll
-  for (int n = 0; n < KvRegs<D>::kChunks; ++n) {
-    const int e = tid + 256 * n;
-    const int row = e / CPR, c = e % CPR;
-    const size_t off = (size_t)(tile * kKeyTile + row) * row_stride + c * 8;
-    r.k[n] = load_global16(kbase + off);
-    r.v[n] = load_global16(vbase + off);
-  }
-  if (tid < kKeyTile) r.seg = segb[tile * kKeyTile + tid];
-}
-
-template <int D>
-CT_DEVICE void kv_commit(const KvRegs<D>& r, lds_addr stage) {
-  constexpr int CPR = D / 8;
-  const int tid = threadIdx.x;
-#pragma unroll
-  for (int n = 0; n < KvRegs<D>::kChunks; ++n) {
-    const int e = tid + 256 * n;
-    const int off = tile_byte_offset<CPR>(e / CPR, e % CPR);
-    lds_store<u32x4>(stage + KvStage<D>::kK + off, r.k[n]);
-    lds_store<u32x4>(stage + KvStage<D>::kV + off, r.v[n]);
-  }
-  if (tid < kKeyTile) lds_store<int>(stage + KvStage<D>::kSeg + tid * 4, r.seg);
-}
 
 // Decoded position of a workgroup / wavefront in the (batch, head, row block)
 // space. Hardware workgroup ids run over (rank, group): the group (batch,
@@ -261,7 +243,7 @@ struct QueryTileContext {
 // Forward
 // ---------------------------------------------------------------------------
 template <int D, int HS>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr lds0 = lds_address_of(smem_raw);
   constexpr int kStage = KvStage<D>::kBytes;
@@ -284,24 +266,23 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
   float m_run = kNegInf;  // running max, log2 domain
   float l_run = 0.f;      // this lane's share of the running sum
 
+  const KvFetcher<D> fetch(ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride);
   int t = ctx.first;
   KeyTileBounds kb = {0, 0, 0};
   if (t <= ctx.last) {
-    KvRegs<D> regs;
-    kv_fetch<D>(regs, ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride, t);
+    fetch.issue(t, lds0);
     kb = key_tile_bounds(ctx.meta_b, t);
-    kv_commit<D>(regs, lds0);
   }
+  dma_wait_all();
   __syncthreads();
 
   auto step = [&](auto stage_tag) {
     constexpr int CUR = decltype(stage_tag)::value;
     const lds_addr stage = lds0 + CUR * kStage;
     const bool more = t + 1 <= ctx.last;
-    KvRegs<D> regs;
     KeyTileBounds nb = kb;
     if (more) {
-      kv_fetch<D>(regs, ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride, t + 1);
+      fetch.issue(t + 1, lds0 + (CUR ^ 1) * kStage);
       nb = key_tile_bounds(ctx.meta_b, t + 1);
     }
     if (ctx.wave_visits(kb, t)) {
@@ -344,7 +325,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(AttnParams p) {
       l_run += psum;
       accumulate_t<D>(stage + KvStage<D>::kV, to, s, oacc);
     }
-    if (more) kv_commit<D>(regs, lds0 + (CUR ^ 1) * kStage);
+    dma_wait_all();
     __syncthreads();
     kb = nb;
     ++t;

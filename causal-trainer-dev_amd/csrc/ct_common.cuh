@@ -82,6 +82,17 @@ CT_DEVICE bf16x4_vs lds_load_tr(lds_addr a) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((CT_LDS bf16x4_vs*)(uintptr_t)a);
 }
 
+// Asynchronous global -> LDS copy of 16 bytes per lane (no registers): lane l
+// of the wavefront writes LDS bytes [dst + 16 l, dst + 16 l + 16). `dst` must
+// be wave-uniform. Completion is tracked by vmcnt: call dma_wait_all() and
+// then a barrier before other wavefronts read the data.
+CT_DEVICE void dma16(const void* src, lds_addr dst) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (CT_LDS void*)(uintptr_t)dst, 16, 0, 0);
+}
+// s_waitcnt vmcnt(0) only (expcnt / lgkmcnt fields left at "no wait")
+CT_DEVICE void dma_wait_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 // ---------------------------------------------------------------------------
 // Swizzled LDS tiles. CPR = 16-byte chunks per row (row length / 8 elements).
 // The swizzle only depends on row bits 0..3, and only touches chunk bits
@@ -105,6 +116,32 @@ template <int CPR>
 CT_DEVICE int tile_byte_offset(int row, int chunk) {
   return (row * CPR + (chunk ^ swizzle<CPR>(row))) * 16;
 }
+
+// Global -> LDS copy of a ROWS x (8 CPR) bf16 tile into its swizzled layout by
+// the 256 threads of a workgroup: thread t owns the 16-byte LDS slots t + 256 n;
+// the swizzle is undone on the global side (each lane fetches the chunk that
+// belongs in its slot). Requires 16 | 256 / CPR, so one lane constant describes
+// all of a thread's slots.
+template <int ROWS, int CPR>
+struct TileDma {
+  static constexpr int kRowsPerPass = 256 / CPR;
+  static constexpr int kPasses = ROWS / kRowsPerPass;
+  static_assert(kRowsPerPass % 16 == 0 && ROWS % kRowsPerPass == 0, "unsupported tile shape");
+  int row0, chunk;  // this thread's row in pass 0 and the logical chunk it fetches
+  CT_DEVICE TileDma() {
+    const int t = threadIdx.x;
+    row0 = t / CPR;
+    chunk = (t % CPR) ^ swizzle<CPR>(row0);
+  }
+  // tile row r lives at src + r * row_stride_bytes; src and tile are workgroup-uniform.
+  CT_DEVICE void issue(const char* src, size_t row_stride_bytes, lds_addr tile) const {
+    const int wave = uniform(threadIdx.x >> 6);
+    const char* p = src + (size_t)row0 * row_stride_bytes + chunk * 16;
+#pragma unroll
+    for (int n = 0; n < kPasses; ++n)
+      dma16(p + (size_t)n * kRowsPerPass * row_stride_bytes, tile + (n * 256 + wave * 64) * 16);
+  }
+};
 
 // Per-lane byte offsets of the k-contiguous MFMA fragments of a tile:
 // fragment (row block rb, k-step ks) of lane l is the 16 bytes at
