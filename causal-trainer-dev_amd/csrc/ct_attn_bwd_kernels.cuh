@@ -120,29 +120,21 @@ struct QdoStage {
   static constexpr int kTotalBytes = 2 * kBytes + kPatchBytes;
 };
 
-// Q goes through registers (it is rescaled on the way); dO is copied asynchronously.
-template <int D>
-struct QdoRegs {
-  static constexpr int kChunks = kQueryTile * (D / 8) / 256;
-  u32x4 q[kChunks];
+// Per-row statistics of a query block, carried in registers by lanes 0..31 of the workgroup.
+struct QueryRowRegs {
   float lse2, delta;
   int seg, end;
 };
 
+// Starts the asynchronous copy of Q and dO rows of query block qb into `stage`.
 template <int D>
-CT_DEVICE void qdo_fetch(QdoRegs<D>& r, const TileDma<kQueryTile, D / 8>& dma, const AttnParams& p,
+CT_DEVICE void qdo_fetch(QueryRowRegs& r, const TileDma<kQueryTile, D / 8>& dma, const AttnParams& p,
                          int b, int h, int qb, lds_addr stage) {
-  constexpr int CPR = D / 8;
   const int tid = threadIdx.x;
   const size_t origin = (((size_t)b * p.S + qb * kQueryTile) * p.Hq + h) * D;
+  dma.issue(reinterpret_cast<const char*>(p.q + origin), (size_t)p.Hq * D * 2, stage + QdoStage<D>::kQ);
   dma.issue(reinterpret_cast<const char*>(p.dout + origin), (size_t)p.Hq * D * 2,
             stage + QdoStage<D>::kDo);
-#pragma unroll
-  for (int n = 0; n < QdoRegs<D>::kChunks; ++n) {
-    const int e = tid + 256 * n;
-    const int row = e / CPR, c = e % CPR;
-    r.q[n] = load_global16(p.q + origin + (size_t)row * p.Hq * D + c * 8);
-  }
   if (tid < kQueryTile) {
     const int pos = qb * kQueryTile + tid;
     const size_t so = ((size_t)b * p.S + pos) * p.Hq + h;
@@ -153,15 +145,17 @@ CT_DEVICE void qdo_fetch(QdoRegs<D>& r, const TileDma<kQueryTile, D / 8>& dma, c
   }
 }
 
+// After this thread's copies have landed (dma_wait_all), fold the softmax scale
+// into its own Q slots in place (bf16 multiply, as the forward does) and publish
+// the row statistics. A barrier must follow.
 template <int D>
-CT_DEVICE void qdo_commit(const QdoRegs<D>& r, lds_addr stage, float scale) {
-  constexpr int CPR = D / 8;
+CT_DEVICE void qdo_commit(const QueryRowRegs& r, lds_addr stage, float scale) {
+  constexpr int kSlots = kQueryTile * (D / 8) / 256;
   const int tid = threadIdx.x;
 #pragma unroll
-  for (int n = 0; n < QdoRegs<D>::kChunks; ++n) {
-    const int e = tid + 256 * n;
-    const int off = tile_byte_offset<CPR>(e / CPR, e % CPR);
-    lds_store<u32x4>(stage + QdoStage<D>::kQ + off, as_u32x4(scale_bf16x8(as_bf16x8(r.q[n]), scale)));
+  for (int n = 0; n < kSlots; ++n) {
+    const lds_addr slot = stage + QdoStage<D>::kQ + (n * 256 + tid) * 16;
+    lds_store<u32x4>(slot, as_u32x4(scale_bf16x8(as_bf16x8(lds_load<u32x4>(slot)), scale)));
   }
   if (tid < kQueryTile) {
     lds_store<float>(stage + QdoStage<D>::kLse + tid * 4, r.lse2);
@@ -276,11 +270,11 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   int it = 0, qb = q_lo, head = kvh * g;
   const TileDma<kQueryTile, D / 8> dma;
   if (it < items) {
-    QdoRegs<D> regs;
+    QueryRowRegs regs;
     qdo_fetch<D>(regs, dma, p, b, head, qb, lds0);
+    dma_wait_all();
     qdo_commit<D>(regs, lds0, p.scale);
   }
-  dma_wait_all();
   __syncthreads();
 
   auto step = [&](auto stage_tag) {
@@ -292,7 +286,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
       qb_next = q_lo;
       ++head_next;
     }
-    QdoRegs<D> regs;
+    QueryRowRegs regs;
     if (more) qdo_fetch<D>(regs, dma, p, b, head_next, qb_next, lds0 + (CUR ^ 1) * kStage);
 
     const int* qm = meta_b + qb * kMetaW;
@@ -330,8 +324,8 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
       accumulate_keys<D>(stage + QdoStage<D>::kDo, to, prob, dvacc);
       accumulate_keys<D>(stage + QdoStage<D>::kQ, to, dp, dkacc);
     }
-    if (more) qdo_commit<D>(regs, lds0 + (CUR ^ 1) * kStage, p.scale);
     dma_wait_all();
+    if (more) qdo_commit<D>(regs, lds0 + (CUR ^ 1) * kStage, p.scale);
     __syncthreads();
     ++it;
     qb = qb_next;
