@@ -28,8 +28,8 @@ __global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
 
   const QueryTileContext<D, HS> ctx(p);
   const int l = lane_id(), half = l >> 5, w = threadIdx.x >> 6;
-  const RowFragOffsets<D / 8> ro;
-  const TrFragOffsets<D / 8, KSlots::kAccum> to;
+  const RowFragOffsets<D / 8> ro(lds0);
+  const TrFragOffsets<D / 8, KSlots::kAccum> to(lds0);
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
   const float lse2 = p.lse[ctx.stat_off] * kLog2e;
@@ -66,8 +66,8 @@ __global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
     }
     if (ctx.wave_visits(kb, t)) {
       f32x16 s[2], dp[2];
-      scores_t<D>(stage + KvStage<D>::kK, ro, qf, s);
-      scores_t<D>(stage + KvStage<D>::kV, ro, dof, dp);
+      scores_t<D>(CUR * kStage + KvStage<D>::kK, ro, qf, s);
+      scores_t<D>(CUR * kStage + KvStage<D>::kV, ro, dof, dp);
       unsigned allow[2] = {0xffffffffu, 0xffffffffu};
       if (!ctx.interior(kb, t))
         tile_mask(stage + KvStage<D>::kSeg, t, ctx.seg_q, ctx.end_q, ctx.row_valid, allow);
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
               ((allow[kbk] >> r) & 1u) ? exp2_fast(fmaf(s[kbk][r], kLog2e, -lse2)) : 0.f;
           s[kbk][r] = prob * (dp[kbk][r] - delta_q);
         }
-      accumulate_t<D>(stage + KvStage<D>::kK, to, s, dqacc);
+      accumulate_t<D>(CUR * kStage + KvStage<D>::kK, to, s, dqacc);
     }
     dma_wait_all();
     __syncthreads();
@@ -167,24 +167,24 @@ CT_DEVICE void qdo_commit(const QueryRowRegs& r, lds_addr stage, float scale) {
 
 // X (32 rows of an LDS tile) times register fragments: C[row, key] = sum_d X[row, d] F[key, d].
 template <int D>
-CT_DEVICE f32x16 rows_times_frags(lds_addr tile, const RowFragOffsets<D / 8>& ro,
+CT_DEVICE f32x16 rows_times_frags(int tile_off, const RowFragOffsets<D / 8>& ro,
                                   const bf16x8* frags) {
   f32x16 c = zero16();
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) c = mfma32(lds_load<bf16x8>(tile + ro.off[ks]), frags[ks], c);
+  for (int ks = 0; ks < D / 16; ++ks) c = mfma32(ro.load(tile_off, 0, ks), frags[ks], c);
   return c;
 }
 
 // acc (32 keys x D) += W^T X, W in accumulator layout (rows = the 32 tile rows,
 // cols = keys), X the 32-row LDS tile read transposed.
 template <int D>
-CT_DEVICE void accumulate_keys(lds_addr tile, const TrFragOffsets<D / 8, KSlots::kAccum>& to,
+CT_DEVICE void accumulate_keys(int tile_off, const TrFragOffsets<D / 8, KSlots::kAccum>& to,
                                const f32x16& wt, f32x16* acc) {
 #pragma unroll
   for (int step = 0; step < 2; ++step) {
     const bf16x8 aop = pack_acc8(wt, step);
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db) acc[db] = mfma32(aop, to.load(tile, step, db), acc[db]);
+    for (int db = 0; db < D / 32; ++db) acc[db] = mfma32(aop, to.load(tile_off, step, db), acc[db]);
   }
 }
 
@@ -227,8 +227,8 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
       uniform(p.sched[(size_t)b * schedule_ints(nrb) + key_schedule_offset(nrb) + rank]);
   const int g = p.Hq / p.Hkv;
   const int* meta_b = p.meta + (size_t)b * nrb * kMetaW;
-  const RowFragOffsets<D / 8> ro;
-  const TrFragOffsets<D / 8, KSlots::kAccum> to;
+  const RowFragOffsets<D / 8> ro(lds0);
+  const TrFragOffsets<D / 8, KSlots::kAccum> to(lds0);
 
   int q_lo = INT_MAX, q_hi = -1;
 #pragma unroll
@@ -250,12 +250,13 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   // K fragments stay in registers; V fragments are parked in LDS (this wavefront's
   // private 32-row patch) and re-read per block, which keeps the kernel under 256
   // registers so that two workgroups share a CU.
-  const lds_addr vpatch = lds0 + QdoStage<D>::kVResident + w * 32 * D * 2;
+  const int vpatch_off = QdoStage<D>::kVResident + w * 32 * D * 2;
+  const lds_addr vpatch = lds0 + vpatch_off;
   bf16x8 kf[D / 16];
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) {
     kf[ks] = as_bf16x8(load_global16(p.k + kv_off + 16 * ks + 8 * half));
-    lds_store<u32x4>(vpatch + ro.off[ks], load_global16(p.v + kv_off + 16 * ks + 8 * half));
+    lds_store<u32x4>(ro.ptr[ks] + vpatch_off, load_global16(p.v + kv_off + 16 * ks + 8 * half));
   }
   f32x16 dkacc[D / 32], dvacc[D / 32];
 #pragma unroll
@@ -294,12 +295,11 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
               q_end_max = uniform(qm[kEndMax]), q_end_min = uniform(qm[kEndMin]),
               q_uni = uniform(qm[kUniform]);
     if (blocks_interact(q_min, q_max, q_end_max, my_min, my_max, my_rb * 32)) {
-      f32x16 s = rows_times_frags<D>(stage + QdoStage<D>::kQ, ro, kf);
+      f32x16 s = rows_times_frags<D>(CUR * kStage + QdoStage<D>::kQ, ro, kf);
       f32x16 dp = zero16();
 #pragma unroll
       for (int ks = 0; ks < D / 16; ++ks)
-        dp = mfma32(lds_load<bf16x8>(stage + QdoStage<D>::kDo + ro.off[ks]),
-                    lds_load<bf16x8>(vpatch + ro.off[ks]), dp);
+        dp = mfma32(ro.load(CUR * kStage + QdoStage<D>::kDo, 0, ks), ro.load(vpatch_off, 0, ks), dp);
       const bool interior = tile_is_interior(q_uni, q_end_min, my_uni, my_rb * 32 + 31);
       f32x16 prob;
 #pragma unroll
@@ -321,8 +321,8 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
           dp[r] = pr * (dp[r] - del4[e]);
         }
       }
-      accumulate_keys<D>(stage + QdoStage<D>::kDo, to, prob, dvacc);
-      accumulate_keys<D>(stage + QdoStage<D>::kQ, to, dp, dkacc);
+      accumulate_keys<D>(CUR * kStage + QdoStage<D>::kDo, to, prob, dvacc);
+      accumulate_keys<D>(CUR * kStage + QdoStage<D>::kQ, to, dp, dkacc);
     }
     dma_wait_all();
     if (more) qdo_commit<D>(regs, lds0 + (CUR ^ 1) * kStage, p.scale);

@@ -113,19 +113,16 @@ struct QueryWork {
 };
 
 // S^T (two 32-key blocks) = K_tile Q^T for this wavefront's 32 queries.
+// `tile_off` is the tile's byte offset from the LDS base the offsets were built on.
 template <int D>
-CT_DEVICE void scores_t(lds_addr tile, const RowFragOffsets<D / 8>& ro, const bf16x8* qf,
+CT_DEVICE void scores_t(int tile_off, const RowFragOffsets<D / 8>& ro, const bf16x8* qf,
                         f32x16* s) {
   s[0] = zero16();
   s[1] = zero16();
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) {
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      const bf16x8 a =
-          lds_load<bf16x8>(tile + kb * RowFragOffsets<D / 8>::kRowBlockBytes + ro.off[ks]);
-      s[kb] = mfma32(a, qf[ks], s[kb]);
-    }
+    for (int kb = 0; kb < 2; ++kb) s[kb] = mfma32(ro.load(tile_off, kb, ks), qf[ks], s[kb]);
   }
 }
 
@@ -153,13 +150,13 @@ CT_DEVICE void tile_mask(lds_addr segk, int tile, int seg_q, int end_q, bool row
 // acc (D x 32 queries, transposed) += X^T W^T where X is a 64-row LDS tile read
 // transposed and W^T are the accumulator-layout weights wt[2].
 template <int D>
-CT_DEVICE void accumulate_t(lds_addr tile, const TrFragOffsets<D / 8, KSlots::kAccum>& to,
+CT_DEVICE void accumulate_t(int tile_off, const TrFragOffsets<D / 8, KSlots::kAccum>& to,
                             const f32x16* wt, f32x16* acc) {
 #pragma unroll
   for (int step = 0; step < 4; ++step) {
     const bf16x8 bop = pack_acc8(wt[step >> 1], step & 1);
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db) acc[db] = mfma32(to.load(tile, step, db), bop, acc[db]);
+    for (int db = 0; db < D / 32; ++db) acc[db] = mfma32(to.load(tile_off, step, db), bop, acc[db]);
   }
 }
 
@@ -250,8 +247,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 
   const QueryTileContext<D, HS> ctx(p);
   const int l = lane_id(), half = l >> 5, w = threadIdx.x >> 6;
-  const RowFragOffsets<D / 8> ro;
-  const TrFragOffsets<D / 8, KSlots::kAccum> to;
+  const RowFragOffsets<D / 8> ro(lds0);
+  const TrFragOffsets<D / 8, KSlots::kAccum> to(lds0);
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
 
@@ -287,7 +284,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
     }
     if (ctx.wave_visits(kb, t)) {
       f32x16 s[2];
-      scores_t<D>(stage + KvStage<D>::kK, ro, qf, s);
+      scores_t<D>(CUR * kStage + KvStage<D>::kK, ro, qf, s);
       float mx = kNegInf;
       if (!ctx.interior(kb, t)) {
         unsigned allow[2];
@@ -323,7 +320,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
         m_run = m_new;
       }
       l_run += psum;
-      accumulate_t<D>(stage + KvStage<D>::kV, to, s, oacc);
+      accumulate_t<D>(CUR * kStage + KvStage<D>::kV, to, s, oacc);
     }
     dma_wait_all();
     __syncthreads();

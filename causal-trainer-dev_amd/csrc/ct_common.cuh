@@ -34,9 +34,11 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_vs;
-typedef uint32_t lds_addr;
-
+// A byte address in LDS. Kept as an address_space(3) pointer so that "pointer + constant"
+// folds into the 16-bit offset field of ds_* instructions.
 #define CT_LDS __attribute__((address_space(3)))
+typedef CT_LDS char* lds_addr;
+
 #define CT_DEVICE __device__ __forceinline__
 
 constexpr float kLog2e = 1.4426950408889634f;
@@ -67,19 +69,17 @@ CT_DEVICE float xor32(float v) { return __shfl_xor(v, 32, 64); }
 // ---------------------------------------------------------------------------
 // LDS access through 32-bit addresses
 // ---------------------------------------------------------------------------
-CT_DEVICE lds_addr lds_address_of(void* shared_ptr) {
-  return (lds_addr)(uintptr_t)(CT_LDS char*)shared_ptr;
-}
+CT_DEVICE lds_addr lds_address_of(void* shared_ptr) { return (lds_addr)shared_ptr; }
 template <class T>
 CT_DEVICE T lds_load(lds_addr a) {
-  return *(CT_LDS const T*)(uintptr_t)a;
+  return *(CT_LDS const T*)a;
 }
 template <class T>
 CT_DEVICE void lds_store(lds_addr a, T v) {
-  *(CT_LDS T*)(uintptr_t)a = v;
+  *(CT_LDS T*)a = v;
 }
 CT_DEVICE bf16x4_vs lds_load_tr(lds_addr a) {
-  return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((CT_LDS bf16x4_vs*)(uintptr_t)a);
+  return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((CT_LDS bf16x4_vs*)a);
 }
 
 // Asynchronous global -> LDS copy of 16 bytes per lane (no registers): lane l
@@ -88,7 +88,7 @@ CT_DEVICE bf16x4_vs lds_load_tr(lds_addr a) {
 // then a barrier before other wavefronts read the data.
 CT_DEVICE void dma16(const void* src, lds_addr dst) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                   (CT_LDS void*)(uintptr_t)dst, 16, 0, 0);
+                                   (CT_LDS void*)dst, 16, 0, 0);
 }
 // s_waitcnt vmcnt(0) only (expcnt / lgkmcnt fields left at "no wait")
 CT_DEVICE void dma_wait_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
@@ -143,20 +143,26 @@ struct TileDma {
   }
 };
 
-// Per-lane byte offsets of the k-contiguous MFMA fragments of a tile:
-// fragment (row block rb, k-step ks) of lane l is the 16 bytes at
-//   tile + rb * 32 * CPR * 16 + off[ks]
-// and holds row rb*32 + l%32, elements 16 ks + 8 (l/32) .. +7.
+// Per-lane LDS addresses of the k-contiguous MFMA fragments of tiles placed at
+// constant offsets from `base`: fragment (row block rb, k-step ks) of the tile
+// at base + tile_off is the 16 bytes at
+//   ptr[ks] + tile_off + rb * kRowBlockBytes
+// and holds row rb*32 + l%32, elements 16 ks + 8 (l/32) .. +7. Keeping the
+// lane-dependent part in registers as pointers lets every other term fold into
+// the instruction's immediate offset.
 template <int CPR>
 struct RowFragOffsets {
   static constexpr int kSteps = CPR / 2;
-  int off[kSteps];
-  CT_DEVICE RowFragOffsets() {
+  static constexpr int kRowBlockBytes = 32 * CPR * 16;
+  lds_addr ptr[kSteps];
+  CT_DEVICE explicit RowFragOffsets(lds_addr base) {
     const int l = lane_id(), row = l & 31, half = l >> 5;
 #pragma unroll
-    for (int ks = 0; ks < kSteps; ++ks) off[ks] = tile_byte_offset<CPR>(row, 2 * ks + half);
+    for (int ks = 0; ks < kSteps; ++ks) ptr[ks] = base + tile_byte_offset<CPR>(row, 2 * ks + half);
   }
-  static constexpr int kRowBlockBytes = 32 * CPR * 16;
+  CT_DEVICE bf16x8 load(int tile_off, int rb, int ks) const {
+    return lds_load<bf16x8>(ptr[ks] + (tile_off + rb * kRowBlockBytes));
+  }
 };
 
 // k-slot -> contraction index maps for transposed fragments.
@@ -167,15 +173,16 @@ struct RowFragOffsets {
 //             result be fed back as an operand without cross-lane movement.
 enum class KSlots { kNatural, kAccum };
 
-// Per-lane byte offsets of transposed MFMA fragments: the MFMA row/column
+// Per-lane LDS addresses of transposed MFMA fragments: the MFMA row/column
 // index i = l % 32 runs along tile columns cb*32 .. cb*32+31 and the 8
-// k-slots of a lane are tile rows. Fragment (column block cb, k-step ks) is
-// two ds_read_b64_tr_b16 at
-//   tile + ks * 16 * CPR * 16 + (cb / 4) * 256 + off[second][cb % 4]
+// k-slots of a lane are tile rows. Fragment (column block cb, k-step ks) of
+// the tile at base + tile_off is two ds_read_b64_tr_b16 at
+//   ptr[second][cb % 4] + tile_off + ks * kStepBytes + (cb / 4) * 256
 template <int CPR, KSlots MAP>
 struct TrFragOffsets {
-  int off[2][4];
-  CT_DEVICE TrFragOffsets() {
+  static constexpr int kStepBytes = 16 * CPR * 16;
+  lds_addr ptr[2][4];
+  CT_DEVICE explicit TrFragOffsets(lds_addr base) {
     const int l = lane_id(), p = l & 15, q16 = (l >> 4) & 1, half = l >> 5;
 #pragma unroll
     for (int second = 0; second < 2; ++second) {
@@ -184,15 +191,14 @@ struct TrFragOffsets {
 #pragma unroll
       for (int cb = 0; cb < 4; ++cb) {
         const int col = cb * 32 + 16 * q16 + 4 * (p & 3);
-        off[second][cb] = tile_byte_offset<CPR>(row, col >> 3) + (col & 4) * 2;
+        ptr[second][cb] = base + (tile_byte_offset<CPR>(row, col >> 3) + (col & 4) * 2);
       }
     }
   }
-  static constexpr int kStepBytes = 16 * CPR * 16;
-  CT_DEVICE bf16x8 load(lds_addr tile, int ks, int cb) const {
-    const lds_addr base = tile + ks * kStepBytes + (cb >> 2) * 256;
-    const bf16x4_vs lo = lds_load_tr(base + off[0][cb & 3]);
-    const bf16x4_vs hi = lds_load_tr(base + off[1][cb & 3]);
+  CT_DEVICE bf16x8 load(int tile_off, int ks, int cb) const {
+    const int off = tile_off + ks * kStepBytes + (cb >> 2) * 256;
+    const bf16x4_vs lo = lds_load_tr(ptr[0][cb & 3] + off);
+    const bf16x4_vs hi = lds_load_tr(ptr[1][cb & 3] + off);
     bf16x8 out;
     out[0] = lo[0]; out[1] = lo[1]; out[2] = lo[2]; out[3] = lo[3];
     out[4] = hi[0]; out[5] = hi[1]; out[6] = hi[2]; out[7] = hi[3];

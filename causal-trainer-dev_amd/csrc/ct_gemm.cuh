@@ -97,8 +97,8 @@ struct KcLoader {
   // fragment for the wavefront's 32-row block i, contraction steps 16*ks .. 16*ks+15;
   // `wave_first` (multiple of 128) is the wavefront's first row.
   typedef RowFragOffsets<CPR> FragOffsets;
-  static CT_DEVICE bf16x8 frag(lds_addr tile, const FragOffsets& fo, int ks, int wave_first, int i) {
-    return lds_load<bf16x8>(tile + (wave_first / 32 + i) * FragOffsets::kRowBlockBytes + fo.off[ks]);
+  static CT_DEVICE bf16x8 frag(int tile_off, const FragOffsets& fo, int ks, int wave_first, int i) {
+    return fo.load(tile_off + (wave_first / 32) * FragOffsets::kRowBlockBytes, i, ks);
   }
 };
 
@@ -164,8 +164,8 @@ struct McLoader {
     for (int n = 0; n < NCH; ++n) lds_store<u32x4>(tile + lds_off[n], regs[n]);
   }
   typedef TrFragOffsets<CPR, KSlots::kNatural> FragOffsets;
-  static CT_DEVICE bf16x8 frag(lds_addr tile, const FragOffsets& fo, int ks, int wave_first, int i) {
-    return fo.load(tile + (wave_first / 128) * 256, ks, i);
+  static CT_DEVICE bf16x8 frag(int tile_off, const FragOffsets& fo, int ks, int wave_first, int i) {
+    return fo.load(tile_off + (wave_first / 128) * 256, ks, i);
   }
 };
 
@@ -195,16 +195,16 @@ CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, lds_add
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
   constexpr int kTile = GemmSmem<BK>::kTileBytes, kStage = GemmSmem<BK>::kStageBytes;
   if (k_begin >= k_end) return;
-  const typename ALoader::FragOffsets afo;
-  const typename BLoader::FragOffsets bfo;
+  const typename ALoader::FragOffsets afo(smem);
+  const typename BLoader::FragOffsets bfo(smem);
   A.fetch(k_begin);
   B.fetch(k_begin);
   A.commit(smem);
   B.commit(smem + kTile);
   __syncthreads();
-  lds_addr cur = smem, nxt = smem + kStage;
+  int cur = 0, nxt = kStage;
   for (int k0 = k_begin; k0 < k_end; k0 += BK) {
-    const lds_addr a_tile = cur, b_tile = cur + kTile;
+    const int a_tile = cur, b_tile = cur + kTile;
     const bool more = k0 + BK < k_end;
     if (more) {
       A.fetch(k0 + BK);
@@ -224,11 +224,11 @@ CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, lds_add
         for (int jn = 0; jn < 4; ++jn) acc.c[i][jn] = mfma32(af[i], bfr[jn], acc.c[i][jn]);
     }
     if (more) {
-      A.commit(nxt);
-      B.commit(nxt + kTile);
+      A.commit(smem + nxt);
+      B.commit(smem + nxt + kTile);
     }
     __syncthreads();
-    const lds_addr tmp = cur;
+    const int tmp = cur;
     cur = nxt;
     nxt = tmp;
   }
