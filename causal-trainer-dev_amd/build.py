@@ -29,6 +29,7 @@ HIP_FLAGS = (
     "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-value",
+    "-Wno-inline-asm",
 )
 
 

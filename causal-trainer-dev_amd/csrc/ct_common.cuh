@@ -84,11 +84,17 @@ CT_DEVICE bf16x4_vs lds_load_tr(lds_addr a) {
 
 // Asynchronous global -> LDS copy of 16 bytes per lane (no registers): lane l
 // of the wavefront writes LDS bytes [dst + 16 l, dst + 16 l + 16). `dst` must
-// be wave-uniform. Completion is tracked by vmcnt: call dma_wait_all() and
-// then a barrier before other wavefronts read the data.
+// be wave-uniform. Completion is tracked by vmcnt: call dma_wait_all() (or a
+// partial vmcnt wait) and then a barrier before other wavefronts read the data.
+// Issued through inline assembly on purpose: with the compiler builtin every
+// later LDS read is preceded by a full vmcnt(0) wait (the compiler cannot tell
+// that the reads touch another stage), which serialises copy and compute.
 CT_DEVICE void dma16(const void* src, lds_addr dst) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                   (CT_LDS void*)dst, 16, 0, 0);
+  const unsigned m0_value = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)dst);
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(src), "s"(m0_value)
+               : "memory", "m0");
 }
 // s_waitcnt vmcnt(0) only (expcnt / lgkmcnt fields left at "no wait")
 CT_DEVICE void dma_wait_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }

@@ -22,7 +22,7 @@
 
 namespace ct {
 
-constexpr int kBK = 64;
+constexpr int kBK = kGemmBK;
 constexpr int kTilesPerChunk = 4;  // vocab tiles per stats work unit
 constexpr float kNegInfF = -__builtin_inff();
 
@@ -76,7 +76,9 @@ __global__ __launch_bounds__(1024) void cutce_index_kernel(const float* weights,
     carry += all;
     __syncthreads();
   }
-  for (int i = carry + tid; i < n_pad; i += blockDim.x) idx[i] = 0;
+  __syncthreads();
+  const int filler = carry > 0 ? idx[0] : 0;  // keeps gathers past the end on a live row
+  for (int i = carry + tid; i < n_pad; i += blockDim.x) idx[i] = filler;
   if (tid == 0) {
     header->n_act = carry;
     header->counter = 0;
@@ -128,17 +130,17 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
       sum[nb] = 0.f;
       tl[nb] = 0.f;
     }
-    KcLoader<kBK> B;
+    KcLoader B;
     B.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true);
 
     const int vt_end = min((chunk + 1) * kTilesPerChunk, vocab_tiles);
     for (int vt = chunk * kTilesPerChunk; vt < vt_end; ++vt) {
       const int v0 = vt * kGemmTile;
-      McLoader<kBK> A;
+      McLoader A;
       A.init(p.head, p.V, nullptr, v0, p.V, p.d, p.head_aligned);
       GemmAcc acc;
       acc.clear();
-      gemm_tile<kBK>(A, B, 0, p.d, smem, acc);
+      gemm_tile(A, B, 0, p.d, smem, acc);
 
       const int vbase = v0 + wm + 4 * half;  // vocab id of (i, r) = vbase + 32 i + 8 (r/4) + r%4
       const bool ragged = v0 + kGemmTile > p.V;
@@ -311,13 +313,13 @@ __global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, const
     lse2_s[tid] = l2;
     tgt_s[tid] = t;
   }
-  KcLoader<kBK> A;
+  KcLoader A;
   A.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true);
-  McLoader<kBK> B;
+  McLoader B;
   B.init(p.head, p.V, nullptr, v0, p.V, p.d, p.head_aligned);
   GemmAcc acc;
   acc.clear();
-  gemm_tile<kBK>(A, B, 0, p.d, smem, acc);  // barriers inside also publish the row arrays
+  gemm_tile(A, B, 0, p.d, smem, acc);  // barriers inside also publish the row arrays
 
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -364,13 +366,13 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
   const int n_act = p.header->n_act;
   if (n0 >= n_act) return;
 
-  KcLoader<kBK> A;
+  KcLoader A;
   A.init(G, ldg, nullptr, n0, p.n_pad, slab_width, true, false);
-  KcLoader<kBK> B;
+  KcLoader B;
   B.init(p.head + slab0, p.V, nullptr, c0, p.d, min(slab_width, p.V - slab0), p.head_aligned, false);
   GemmAcc acc;
   acc.clear();
-  gemm_tile<kBK>(A, B, 0, slab_width, smem, acc);
+  gemm_tile(A, B, 0, slab_width, smem, acc);
 
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -406,13 +408,15 @@ __global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const b
   const int n_act = p.header->n_act;
   const int k_end = min(p.n_pad, (n_act + kBK - 1) / kBK * kBK);
 
-  McLoader<kBK> A;
-  A.init(p.hidden, p.d, p.idx, m0, p.d, n_act, p.hidden_aligned);
-  McLoader<kBK> B;
-  B.init(G, ldg, nullptr, v0, ldg, n_act, true);
+  McLoader A;
+  // Rows n_act .. k_end-1 are valid memory: G holds zeros there (written by the
+  // dlogits kernel for the whole 256-row block) and idx repeats the first active row.
+  A.init(p.hidden, p.d, p.idx, m0, p.d, k_end, p.hidden_aligned);
+  McLoader B;
+  B.init(G, ldg, nullptr, v0, ldg, k_end, true);
   GemmAcc acc;
   acc.clear();
-  gemm_tile<kBK>(A, B, 0, k_end, smem, acc);
+  gemm_tile(A, B, 0, k_end, smem, acc);
 
 #pragma unroll
   for (int i = 0; i < 4; ++i)
@@ -579,7 +583,7 @@ extern "C" int32_t ct_cutce_fwd(void* stream_, const ct_cutce_fwd_args* a) {
                      a->sparse_compaction ? 1 : 0, p.idx, p.header);
   if ((rc = scope1.done())) return rc;
 
-  const size_t smem = GemmSmem<kBK>::kBytes;
+  const size_t smem = GemmSmem::kBytes;
   if ((rc = set_smem(cutce_stats_kernel, smem, "ct_cutce_fwd"))) return rc;
   const int persistent = min(device_cu_count(), chunks * row_blocks);
   LaunchScope scope2("cutce_stats_kernel", stream);
@@ -618,7 +622,7 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
   bf16* dhead = reinterpret_cast<bf16*>(a->dhead);
   const int row_blocks = p.n_pad / kGemmTile;
   const int ldg = L.slab_cols;
-  const size_t smem = GemmSmem<kBK>::kBytes;
+  const size_t smem = GemmSmem::kBytes;
   if ((rc = set_smem(cutce_dlogits_kernel, smem, "ct_cutce_bwd"))) return rc;
   if ((rc = set_smem(cutce_dhidden_kernel, smem, "ct_cutce_bwd"))) return rc;
   if ((rc = set_smem(cutce_dhead_kernel, smem, "ct_cutce_bwd"))) return rc;

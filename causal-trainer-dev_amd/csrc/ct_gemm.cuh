@@ -2,9 +2,8 @@
 // cross-entropy kernels.
 //
 // 4 wavefronts in a 2 x 2 arrangement, 128 x 128 outputs per wavefront held
-// as 4 x 4 mfma32 accumulator blocks (256 f32 registers per lane). Operand
-// tiles of BK contraction steps are staged global -> registers -> swizzled
-// LDS, double buffered with one barrier per step.
+// as 4 x 4 mfma32 accumulator blocks (256 f32 registers per lane). The
+// contraction runs in steps of BK = 32.
 //
 // An operand comes in one of two memory layouts:
 //   KcLoader  "k-contiguous": matrix rows are the M (or N) index, the
@@ -13,40 +12,52 @@
 //   McLoader  "m-contiguous": matrix rows are the contraction index, the M
 //             (or N) index is contiguous. LDS tile [BK][256], fragments read
 //             with transposed LDS reads.
-// Rows can be addressed through an index list (gather), everything out of
-// range is zero filled, and unaligned leading dimensions fall back to
-// element-wise loads.
+// Rows can be addressed through an index list (gather).
+//
+// Two main loops share the loaders:
+//   pipelined  every row / column / k of the tile is in range and 16-byte
+//              aligned: tiles are copied global -> LDS asynchronously, three
+//              steps ahead, into a ring of 4 LDS stages; MFMA fragments are
+//              double buffered in registers so that LDS reads of the next
+//              half step overlap the 16 MFMAs of the current one; one
+//              barrier per step.
+//   guarded    anything ragged or unaligned: element-wise guarded loads that
+//              zero fill, staged through registers, 2 LDS stages.
+// The choice is uniform over the workgroup.
 #pragma once
-
-#include <type_traits>
 
 #include "ct_common.cuh"
 
 namespace ct {
 
 constexpr int kGemmTile = 256;
+constexpr int kGemmBK = 32;
 
-CT_DEVICE u32x4 load_chunk_guarded(const bf16* p, int count, bool aligned) {
-  if (count >= 8 && aligned) return load_global16(p);
+CT_DEVICE u32x4 load_chunk_guarded(const bf16* p, int count) {
   bf16x8 v;
 #pragma unroll
   for (int e = 0; e < 8; ++e) v[e] = e < count ? p[e] : (bf16)0.f;
   return as_u32x4(v);
 }
 
-// Both loaders have a straight-line fast path (every row / column / k of the
-// step in range and 16-byte aligned: unconditional 16-byte loads at
-// uniform-base + 32-bit lane offsets) and a guarded element-wise path that
-// zero fills; the choice is uniform over the workgroup.
-template <int BK>
+struct GemmSmem {
+  static constexpr int kTileBytes = kGemmTile * kGemmBK * 2;  // 16 KB
+  static constexpr int kStageBytes = 2 * kTileBytes;          // A tile then B tile
+  static constexpr int kStages = 4;
+  static constexpr size_t kBytes = (size_t)kStages * kStageBytes;  // 128 KB
+};
+
+// In both loaders thread t owns the 16-byte LDS slots t + 256 n of the tile
+// (n < 4): slot P holds physical chunk P % CPR of row P / CPR, i.e. logical
+// chunk (P % CPR) ^ swizzle(row); voff[n] is the byte offset of that chunk
+// from `base` at k = 0.
 struct KcLoader {
-  static constexpr int CPR = BK / 8;
-  static constexpr int NCH = BK / 8;          // 16-byte chunks per thread per step
-  static constexpr int kRowStep = 256 / CPR;  // rows between a thread's chunks
+  static constexpr int CPR = kGemmBK / 8;  // 4
+  static constexpr int NCH = 4;
   const char* base;    // uniform
-  unsigned voff[NCH];  // byte offset of this thread's chunk n from base (k = 0)
+  unsigned voff[NCH];
   u32x4 regs[NCH];
-  int lds_off, k_valid, row_mask;
+  int chunk, k_valid, row_mask;
   bool fast;
 
   // rows m0 .. m0+255 of `base_` (leading dimension ld elements), optionally
@@ -55,44 +66,44 @@ struct KcLoader {
   // those rows); k >= k_valid reads as zero.
   CT_DEVICE void init(const bf16* base_, long ld, const int* row_index, int m0, int rows_valid,
                       int k_valid_, bool aligned, bool alias_invalid_rows) {
-    const int tid = threadIdx.x, chunk = tid % CPR, row0 = tid / CPR;
+    const int t = threadIdx.x;
     k_valid = k_valid_;
-    lds_off = tile_byte_offset<CPR>(row0, chunk);
     const bool gathered = row_index != nullptr;
     base = reinterpret_cast<const char*>(gathered ? base_ : base_ + (size_t)m0 * ld);
     row_mask = 0;
+    const int r0 = t / CPR;
+    chunk = (t % CPR) ^ swizzle<CPR>(r0);  // rows r0 + 64 n share the swizzle
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
-      const int r = row0 + n * kRowStep;
+      const int r = r0 + 64 * n;
       const bool ok = m0 + r < rows_valid;
       if (ok || alias_invalid_rows) row_mask |= 1 << n;
       const long src = gathered ? row_index[ok ? m0 + r : 0] : (ok ? r : 0);
       voff[n] = (unsigned)((src * ld + chunk * 8) * 2);
     }
-    fast = aligned && (alias_invalid_rows || m0 + kGemmTile <= rows_valid);
+    fast = aligned && (alias_invalid_rows || m0 + kGemmTile <= rows_valid) && k_valid % kGemmBK == 0;
+  }
+  CT_DEVICE void dma(int k0, lds_addr tile) const {
+    const int wave = uniform(threadIdx.x >> 6);
+    const char* p = base + (size_t)k0 * 2;
+#pragma unroll
+    for (int n = 0; n < NCH; ++n) dma16(p + voff[n], tile + (n * 256 + wave * 64) * 16);
   }
   CT_DEVICE void fetch(int k0) {
-    if (fast && k0 + BK <= k_valid) {
-      const char* p = base + (size_t)k0 * 2;
+    const int k = k0 + chunk * 8;
+    const int count = min(max(k_valid - k, 0), 8);
 #pragma unroll
-      for (int n = 0; n < NCH; ++n) regs[n] = load_global16(p + voff[n]);
-    } else {
-      const int k = k0 + (threadIdx.x % CPR) * 8;
-      const int count = min(max(k_valid - k, 0), 8);
-#pragma unroll
-      for (int n = 0; n < NCH; ++n) {
-        const bool ok = (row_mask >> n) & 1;
-        regs[n] = (ok && count) ? load_chunk_guarded(reinterpret_cast<const bf16*>(
-                                                         base + (size_t)k0 * 2 + voff[n]),
-                                                     count, false)
-                                : u32x4{0u, 0u, 0u, 0u};
-      }
+    for (int n = 0; n < NCH; ++n) {
+      const bool ok = (row_mask >> n) & 1;
+      regs[n] = (ok && count) ? load_chunk_guarded(reinterpret_cast<const bf16*>(
+                                                       base + (size_t)k0 * 2 + voff[n]),
+                                                   count)
+                              : u32x4{0u, 0u, 0u, 0u};
     }
   }
   CT_DEVICE void commit(lds_addr tile) const {
 #pragma unroll
-    for (int n = 0; n < NCH; ++n)
-      lds_store<u32x4>(tile + lds_off + n * (kRowStep * CPR * 16), regs[n]);
+    for (int n = 0; n < NCH; ++n) lds_store<u32x4>(tile + (n * 256 + (int)threadIdx.x) * 16, regs[n]);
   }
   // fragment for the wavefront's 32-row block i, contraction steps 16*ks .. 16*ks+15;
   // `wave_first` (multiple of 128) is the wavefront's first row.
@@ -102,78 +113,86 @@ struct KcLoader {
   }
 };
 
-template <int BK>
 struct McLoader {
   static constexpr int CPR = kGemmTile / 8;  // 32
-  static constexpr int NCH = BK / 8;
+  static constexpr int NCH = 4;
   const char* base;  // uniform: column m0 of row 0
   const int* row_index;
   long ld;
   unsigned voff[NCH];
-  int lds_off[NCH];
   u32x4 regs[NCH];
-  int count, k_valid;
+  int col[2];  // first column of the chunk fetched in even / odd passes
+  int cols_left, k_valid;
   bool fast;
 
   // columns m0 .. m0+255 of `base_`; contraction rows optionally gathered.
   // Columns >= cols_valid and rows >= k_valid read as zero.
   CT_DEVICE void init(const bf16* base_, long ld_, const int* row_index_, int m0, int cols_valid,
                       int k_valid_, bool aligned) {
-    const int tid = threadIdx.x, col = (tid % CPR) * 8, row0 = tid / CPR;
+    const int t = threadIdx.x;
     base = reinterpret_cast<const char*>(base_ + m0);
     row_index = row_index_;
     ld = ld_;
     k_valid = k_valid_;
-    count = min(max(cols_valid - m0 - col, 0), 8);
-    fast = aligned && m0 + kGemmTile <= cols_valid;
+    cols_left = cols_valid - m0;
+    fast = aligned && m0 + kGemmTile <= cols_valid && k_valid % kGemmBK == 0;
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
-      const int r = row0 + 8 * n;
-      lds_off[n] = tile_byte_offset<CPR>(r, tid % CPR);
-      voff[n] = (unsigned)(((row_index ? 0 : (long)r * ld) + col) * 2);
+      const int r = t / CPR + 8 * n;
+      const int c = ((t % CPR) ^ swizzle<CPR>(r)) * 8;
+      col[n & 1] = c;
+      voff[n] = (unsigned)(((row_index ? 0 : (long)r * ld) + c) * 2);
+    }
+  }
+  CT_DEVICE void dma(int k0, lds_addr tile) const {
+    const int wave = uniform(threadIdx.x >> 6);
+    if (row_index) {
+      // A wavefront covers rows k0 + 2 wave + {0, 1} + 8 n: read the two row indices
+      // with scalar loads (tracked by lgkmcnt, so they do not force the copies
+      // still in flight to drain the way a vector load would).
+      typedef int i32x2 __attribute__((ext_vector_type(2)));
+      const int* ip = row_index + k0 + 2 * wave;
+      i32x2 pair[NCH];
+      asm volatile(
+          "s_load_dwordx2 %0, %4, 0x0\n\ts_load_dwordx2 %1, %4, 0x20\n\t"
+          "s_load_dwordx2 %2, %4, 0x40\n\ts_load_dwordx2 %3, %4, 0x60\n\ts_waitcnt lgkmcnt(0)"
+          : "=&s"(pair[0]), "=&s"(pair[1]), "=&s"(pair[2]), "=&s"(pair[3])
+          : "s"(ip)
+          : "memory");
+      const bool upper = lane_id() >= 32;
+#pragma unroll
+      for (int n = 0; n < NCH; ++n)
+        dma16(base + (size_t)(upper ? pair[n][1] : pair[n][0]) * ld * 2 + voff[n],
+              tile + (n * 256 + wave * 64) * 16);
+    } else {
+      const char* p = base + (size_t)k0 * ld * 2;
+#pragma unroll
+      for (int n = 0; n < NCH; ++n) dma16(p + voff[n], tile + (n * 256 + wave * 64) * 16);
     }
   }
   CT_DEVICE void fetch(int k0) {
-    const int row0 = threadIdx.x / CPR;
-    if (fast && k0 + BK <= k_valid) {
-      if (row_index) {
+    const int r0 = (int)threadIdx.x / CPR;
 #pragma unroll
-        for (int n = 0; n < NCH; ++n)
-          regs[n] = load_global16(base + (size_t)row_index[k0 + row0 + 8 * n] * ld * 2 + voff[n]);
+    for (int n = 0; n < NCH; ++n) {
+      const int k = k0 + r0 + 8 * n;
+      const int count = min(max(cols_left - col[n & 1], 0), 8);
+      if (k < k_valid && count) {
+        const size_t src = row_index ? (size_t)row_index[k] : (size_t)k0;
+        regs[n] = load_chunk_guarded(reinterpret_cast<const bf16*>(base + src * ld * 2 + voff[n]),
+                                     count);
       } else {
-        const char* p = base + (size_t)k0 * ld * 2;
-#pragma unroll
-        for (int n = 0; n < NCH; ++n) regs[n] = load_global16(p + voff[n]);
-      }
-    } else {
-#pragma unroll
-      for (int n = 0; n < NCH; ++n) {
-        const int k = k0 + row0 + 8 * n;
-        if (k < k_valid && count) {
-          const size_t src = row_index ? (size_t)row_index[k] : (size_t)k0;
-          const char* p = base + src * ld * 2 + voff[n];
-          regs[n] = load_chunk_guarded(reinterpret_cast<const bf16*>(p), count, false);
-        } else {
-          regs[n] = u32x4{0u, 0u, 0u, 0u};
-        }
+        regs[n] = u32x4{0u, 0u, 0u, 0u};
       }
     }
   }
   CT_DEVICE void commit(lds_addr tile) const {
 #pragma unroll
-    for (int n = 0; n < NCH; ++n) lds_store<u32x4>(tile + lds_off[n], regs[n]);
+    for (int n = 0; n < NCH; ++n) lds_store<u32x4>(tile + (n * 256 + (int)threadIdx.x) * 16, regs[n]);
   }
   typedef TrFragOffsets<CPR, KSlots::kNatural> FragOffsets;
   static CT_DEVICE bf16x8 frag(int tile_off, const FragOffsets& fo, int ks, int wave_first, int i) {
     return fo.load(tile_off + (wave_first / 128) * 256, ks, i);
   }
-};
-
-template <int BK>
-struct GemmSmem {
-  static constexpr int kTileBytes = kGemmTile * BK * 2;
-  static constexpr int kStageBytes = 2 * kTileBytes;
-  static constexpr size_t kBytes = 2 * kStageBytes;
 };
 
 struct GemmAcc {
@@ -186,17 +205,89 @@ struct GemmAcc {
   }
 };
 
+struct GemmFrags {
+  bf16x8 a[4], b[4];
+};
+
+template <class ALoader, class BLoader>
+CT_DEVICE void load_frags(GemmFrags& f, int stage_off, const typename ALoader::FragOffsets& afo,
+                          const typename BLoader::FragOffsets& bfo, int ks, int wm, int wn) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f.a[i] = ALoader::frag(stage_off, afo, ks, wm, i);
+    f.b[i] = BLoader::frag(stage_off + GemmSmem::kTileBytes, bfo, ks, wn, i);
+  }
+}
+
+CT_DEVICE void mfma_block(const GemmFrags& f, GemmAcc& acc) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int jn = 0; jn < 4; ++jn) acc.c[i][jn] = mfma32(f.a[i], f.b[jn], acc.c[i][jn]);
+}
+
+// s_waitcnt vmcnt(N) for N in {0, 8, 16} (expcnt / lgkmcnt left at "no wait").
+CT_DEVICE void wait_vmcnt(int outstanding) {
+  if (outstanding >= 16)
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (1 << 14));  // vmcnt = 16
+  else if (outstanding >= 8)
+    __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+  else
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+}
+CT_DEVICE void wait_lds() { __builtin_amdgcn_s_waitcnt(0xC07F); }  // lgkmcnt(0) only
+// Execution barrier without the memory fence of __syncthreads() (which would wait for
+// every copy in flight); callers order their own LDS traffic with the waits above.
+CT_DEVICE void workgroup_barrier() { __builtin_amdgcn_s_barrier(); }
+
 // acc += A[m-tile, k_begin:k_end] * B[n-tile, k_begin:k_end]^T. Must be called by
 // all 256 threads; ends with the LDS tiles free for reuse.
-template <int BK, class ALoader, class BLoader>
+template <class ALoader, class BLoader>
 CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, lds_addr smem,
                          GemmAcc& acc) {
+  constexpr int BK = kGemmBK, kTile = GemmSmem::kTileBytes, kStage = GemmSmem::kStageBytes;
+  constexpr int kRing = GemmSmem::kStages * kStage;
+  constexpr int kLoadsPerStep = ALoader::NCH + BLoader::NCH;  // 8 per thread
+  static_assert(kLoadsPerStep == 8, "wait_vmcnt assumes 8 copies per thread per step");
   const int w = threadIdx.x >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
-  constexpr int kTile = GemmSmem<BK>::kTileBytes, kStage = GemmSmem<BK>::kStageBytes;
   if (k_begin >= k_end) return;
   const typename ALoader::FragOffsets afo(smem);
   const typename BLoader::FragOffsets bfo(smem);
+  const int steps = (k_end - k_begin + BK - 1) / BK;
+
+  if (A.fast && B.fast) {
+    dma_wait_all();  // nothing of ours may still be in flight when counting copies below
+    for (int i = 0; i < 3 && i < steps; ++i) {
+      A.dma(k_begin + i * BK, smem + i * kStage);
+      B.dma(k_begin + i * BK, smem + i * kStage + kTile);
+    }
+    wait_vmcnt((min(steps, 3) - 1) * kLoadsPerStep);
+    workgroup_barrier();
+    GemmFrags f0, f1;
+    load_frags<ALoader, BLoader>(f0, 0, afo, bfo, 0, wm, wn);
+    int stage = 0;
+    for (int k = 0; k < steps; ++k) {
+      if (k + 3 < steps) {
+        const int dst = (stage + 3 * kStage) & (kRing - 1);
+        A.dma(k_begin + (k + 3) * BK, smem + dst);
+        B.dma(k_begin + (k + 3) * BK, smem + dst + kTile);
+      }
+      load_frags<ALoader, BLoader>(f1, stage, afo, bfo, 1, wm, wn);
+      mfma_block(f0, acc);
+      // step k+1 must have landed: at most the copies of steps k+2, k+3 may be in flight
+      wait_vmcnt(min(max(steps - k - 2, 0), 2) * kLoadsPerStep);
+      wait_lds();  // our reads of this stage are done before anyone recycles it
+      workgroup_barrier();
+      stage = (stage + kStage) & (kRing - 1);
+      if (k + 1 < steps) load_frags<ALoader, BLoader>(f0, stage, afo, bfo, 0, wm, wn);
+      mfma_block(f1, acc);
+    }
+    wait_lds();
+    __syncthreads();
+    return;
+  }
+
   A.fetch(k_begin);
   B.fetch(k_begin);
   A.commit(smem);
@@ -204,7 +295,6 @@ CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, lds_add
   __syncthreads();
   int cur = 0, nxt = kStage;
   for (int k0 = k_begin; k0 < k_end; k0 += BK) {
-    const int a_tile = cur, b_tile = cur + kTile;
     const bool more = k0 + BK < k_end;
     if (more) {
       A.fetch(k0 + BK);
@@ -212,16 +302,9 @@ CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, lds_add
     }
 #pragma unroll
     for (int ks = 0; ks < BK / 16; ++ks) {
-      bf16x8 af[4], bfr[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        af[i] = ALoader::frag(a_tile, afo, ks, wm, i);
-        bfr[i] = BLoader::frag(b_tile, bfo, ks, wn, i);
-      }
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int jn = 0; jn < 4; ++jn) acc.c[i][jn] = mfma32(af[i], bfr[jn], acc.c[i][jn]);
+      GemmFrags f;
+      load_frags<ALoader, BLoader>(f, cur, afo, bfo, ks, wm, wn);
+      mfma_block(f, acc);
     }
     if (more) {
       A.commit(smem + nxt);
