@@ -48,6 +48,7 @@ class AttnBwdArgs(Structure):
         ("segment_ids", c_void_p), ("attention_end", c_void_p), ("tile_meta", c_void_p),
         ("out", c_void_p), ("lse", c_void_p), ("dout", c_void_p),
         ("dq", c_void_p), ("dk", c_void_p), ("dv", c_void_p), ("delta", c_void_p),
+        ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("batch", c_int32), ("seq", c_int32), ("q_heads", c_int32), ("kv_heads", c_int32),
         ("head_dim", c_int32), ("scale", c_float),
     ]
@@ -83,6 +84,7 @@ SYMBOLS = {
     "ct_last_error": (ctypes.c_char_p, []),
     "ct_abi_version": (c_int32, []),
     "ct_attn_meta_bytes": (c_size_t, [c_int32, c_int32]),
+    "ct_attn_bwd_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
     "ct_attn_prepare": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "ct_attn_block_summary": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
                                         c_void_p]),

@@ -5,6 +5,8 @@
 
 #include <string.h>
 
+#include <initializer_list>
+
 namespace ct {
 
 // ---------------------------------------------------------------------------
@@ -185,6 +187,13 @@ static int validate_shape(const char* fn, int B, int S, int Hq, int Hkv, int D) 
   return CT_OK;
 }
 
+// Tiles move by 16-byte asynchronous copies, so every tensor base must be 16-byte aligned.
+static bool aligned16(std::initializer_list<const void*> ptrs) {
+  for (const void* p : ptrs)
+    if (reinterpret_cast<uintptr_t>(p) & 15u) return false;
+  return true;
+}
+
 // Query heads of one KV head handled by a single workgroup.
 static int heads_per_group(int Hq, int Hkv) {
   const int g = Hq / Hkv;
@@ -238,7 +247,13 @@ static int launch_dkv(hipStream_t stream, const AttnParams& p) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
   }
-  const int grid = (p.S / 128) * p.Hkv * p.B;  // rank-major, see attn_dkv_kernel
+  LaunchScope scope7("attn_dkv_schedule_kernel", stream);
+  hipLaunchKernelGGL(attn_dkv_schedule_kernel, dim3(1), dim3(1024), 0, stream, p.meta, p.B, p.S,
+                     p.Hkv, p.Hq / p.Hkv, p.dkv_max_entries, p.dkv_max_partials, p.dkv_header,
+                     p.dkv_counters, p.dkv_entries);
+  int rc = scope7.done();
+  if (rc) return rc;
+  const int grid = p.dkv_max_entries * p.Hkv;  // entries beyond the list's length exit at once
   LaunchScope scope3("attn_dkv_kernel", stream);
   hipLaunchKernelGGL((attn_dkv_kernel<D>), dim3(grid), dim3(256), smem, stream, p);
   return scope3.done();
@@ -274,6 +289,12 @@ using namespace ct;
 extern "C" size_t ct_attn_meta_bytes(int32_t batch, int32_t seq) {
   if (batch <= 0 || seq <= 0) return 0;
   return (size_t)batch * (size_t)(seq / 32) * (kMetaW + 2) * sizeof(int32_t);
+}
+
+extern "C" size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t kv_heads,
+                                             int32_t head_dim) {
+  if (batch <= 0 || seq <= 0 || kv_heads <= 0 || head_dim <= 0 || seq % kDkvKeys != 0) return 0;
+  return dkv_layout(batch, seq, kv_heads, head_dim).total;
 }
 
 extern "C" int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
@@ -319,6 +340,8 @@ extern "C" int32_t ct_attn_fwd(void* stream, const ct_attn_fwd_args* a) {
   int rc = validate_shape("ct_attn_fwd", a->batch, a->seq, a->q_heads, a->kv_heads, a->head_dim);
   if (rc) return rc;
   CT_REQUIRE(a->scale == a->scale && a->scale - a->scale == 0.f, "ct_attn_fwd: scale must be finite");
+  CT_REQUIRE(aligned16({a->q, a->k, a->v, a->segment_ids, a->attention_end, a->tile_meta, a->out, a->lse}),
+             "ct_attn_fwd: every device pointer must be 16-byte aligned");
   AttnParams p = {};
   p.q = reinterpret_cast<const bf16*>(a->q);
   p.k = reinterpret_cast<const bf16*>(a->k);
@@ -342,6 +365,7 @@ extern "C" int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16
                                  float* delta, int64_t rows, int32_t head_dim) {
   CT_REQUIRE(out && dout && delta, "ct_attn_delta: null pointer");
   CT_REQUIRE(rows > 0, "ct_attn_delta: rows must be positive");
+  CT_REQUIRE(aligned16({out, dout, delta}), "ct_attn_delta: every device pointer must be 16-byte aligned");
   if (head_dim != 64 && head_dim != 128)
     return fail(CT_UNSUPPORTED, "ct_attn_delta: head_dim must be 64 or 128, got %d", head_dim);
   const bf16* o = reinterpret_cast<const bf16*>(out);
@@ -353,11 +377,14 @@ extern "C" int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16
 extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   CT_REQUIRE(a, "ct_attn_bwd: null args");
   CT_REQUIRE(a->q && a->k && a->v && a->segment_ids && a->tile_meta && a->out && a->lse &&
-                 a->dout && a->dq && a->dk && a->dv && a->delta,
+                 a->dout && a->dq && a->dk && a->dv && a->delta && a->workspace,
              "ct_attn_bwd: null pointer");
   int rc = validate_shape("ct_attn_bwd", a->batch, a->seq, a->q_heads, a->kv_heads, a->head_dim);
   if (rc) return rc;
   CT_REQUIRE(a->scale == a->scale && a->scale - a->scale == 0.f, "ct_attn_bwd: scale must be finite");
+  CT_REQUIRE(aligned16({a->q, a->k, a->v, a->segment_ids, a->attention_end, a->tile_meta, a->out, a->lse,
+                        a->dout, a->dq, a->dk, a->dv, a->delta, a->workspace}),
+             "ct_attn_bwd: every device pointer must be 16-byte aligned");
   AttnParams p = {};
   p.q = reinterpret_cast<const bf16*>(a->q);
   p.k = reinterpret_cast<const bf16*>(a->k);
@@ -378,6 +405,17 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   p.Hq = a->q_heads;
   p.Hkv = a->kv_heads;
   p.scale = round_to_bf16(a->scale);
+  const DkvLayout L = dkv_layout(a->batch, a->seq, a->kv_heads, a->head_dim);
+  if (a->workspace_bytes < L.total)
+    return fail(CT_WORKSPACE_TOO_SMALL, "ct_attn_bwd: workspace %zu < %zu bytes", a->workspace_bytes,
+                L.total);
+  char* ws = static_cast<char*>(a->workspace);
+  p.dkv_header = reinterpret_cast<int*>(ws + L.header);
+  p.dkv_counters = reinterpret_cast<int*>(ws + L.counters);
+  p.dkv_entries = reinterpret_cast<int2*>(ws + L.entries);
+  p.dkv_partials = reinterpret_cast<float*>(ws + L.partials);
+  p.dkv_max_entries = L.max_entries;
+  p.dkv_max_partials = L.max_partials;
   return a->head_dim == 128 ? dispatch_bwd<128>((hipStream_t)stream, p)
                             : dispatch_bwd<64>((hipStream_t)stream, p);
 }

@@ -117,7 +117,9 @@ struct QdoStage {
   static constexpr int kPatchBytes = 4 * 32 * D * 2;
   // resident V rows of the workgroup's 128 keys (32 per wavefront), after the two stages
   static constexpr int kVResident = 2 * kBytes;
-  static constexpr int kTotalBytes = 2 * kBytes + kPatchBytes;
+  // one flag word after the patch: "this workgroup is the last chunk of its tile to finish"
+  static constexpr int kLastFlag = 2 * kBytes + kPatchBytes;
+  static constexpr int kTotalBytes = kLastFlag + 16;
 };
 
 // Per-row statistics of a query block, carried in registers by lanes 0..31 of the workgroup.
@@ -211,6 +213,143 @@ CT_DEVICE void store_rows(const f32x16* acc, lds_addr patch, bf16* gbase, size_t
   }
 }
 
+
+// Number of (head, query block) items of 128-key tile `tile` (= batch row * tiles per row + kt).
+CT_DEVICE int dkv_tile_items(const int* meta, int nrb, int tile, int g, int* q_lo_out = nullptr) {
+  const int nt = nrb / 4;
+  const int* m = meta + ((size_t)(tile / nt) * nrb + (size_t)(tile % nt) * 4) * kMetaW;
+  int q_lo = INT_MAX, q_hi = -1;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    q_lo = min(q_lo, m[i * kMetaW + kQFirst]);
+    q_hi = max(q_hi, m[i * kMetaW + kQLast]);
+  }
+  if (q_lo_out) *q_lo_out = q_lo;
+  return q_lo <= q_hi ? (q_hi - q_lo + 1) * g : 0;
+}
+
+CT_DEVICE int dkv_split_count(int items, int target) {
+  return items <= target ? 1 : min(kDkvMaxSplit, (items + target - 1) / target);
+}
+
+// Builds the dK/dV work list (one workgroup of 1024 threads): chunk target from
+// the total amount of work, chunk count per tile, entries bucketed by
+// decreasing work, arrival counters cleared.
+__global__ __launch_bounds__(1024) void attn_dkv_schedule_kernel(const int* meta, int B, int S,
+                                                                 int Hkv, int g, int max_entries,
+                                                                 int max_partials, int* header,
+                                                                 int* counters, int2* entries) {
+  __shared__ long long red[1024];
+  __shared__ int hist[256];
+  __shared__ int fill[256];
+  __shared__ int carry;
+  const int tid = threadIdx.x;
+  const int nrb = S / 32, ntiles = B * (nrb / 4);
+  for (int i = tid; i < ntiles * Hkv; i += 1024) counters[i] = 0;
+
+  auto block_sum = [&](long long v) {
+    red[tid] = v;
+    __syncthreads();
+    for (int s = 512; s > 0; s >>= 1) {
+      if (tid < s) red[tid] += red[tid + s];
+      __syncthreads();
+    }
+    const long long out = red[0];
+    __syncthreads();
+    return out;
+  };
+
+  long long local = 0;
+  for (int t = tid; t < ntiles; t += 1024) local += dkv_tile_items(meta, nrb, t, g);
+  const long long total = block_sum(local);
+  long long want = (total * Hkv + 2 * kDkvSlots - 1) / (2 * kDkvSlots);
+  int target = (int)min((long long)INT_MAX / 2, max((long long)kDkvMinChunk, want));
+
+  // Entry and partial-slot counts for this target; coarsen the target if they overflow the
+  // space the host reserved (cannot happen for target >= want, kept as a guard).
+  int max_work = 1;
+  for (;;) {
+    long long counts = 0;  // entries in the high half, partial slots in the low half
+    int local_max = 1;
+    for (int t = tid; t < ntiles; t += 1024) {
+      const int items = dkv_tile_items(meta, nrb, t, g);
+      const int ns = dkv_split_count(items, target);
+      counts += ((long long)ns << 32) + (ns > 1 ? ns : 0);
+      local_max = max(local_max, (items + ns - 1) / ns);
+    }
+    const long long both = block_sum(counts);
+    red[tid] = local_max;
+    __syncthreads();
+    for (int s = 512; s > 0; s >>= 1) {
+      if (tid < s) red[tid] = max(red[tid], red[tid + s]);
+      __syncthreads();
+    }
+    max_work = (int)red[0];
+    __syncthreads();
+    if ((both >> 32) <= max_entries && (both & 0xffffffffll) <= max_partials) break;
+    target = target >= INT_MAX / 4 ? INT_MAX / 2 : target * 2;
+  }
+
+  // Histogram of entries over 256 buckets of decreasing work.
+  if (tid < 256) {
+    hist[tid] = 0;
+    fill[tid] = 0;
+  }
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  auto bucket_of = [&](int work) { return 255 - (int)((long long)work * 255 / max_work); };
+  for (int t = tid; t < ntiles; t += 1024) {
+    const int items = dkv_tile_items(meta, nrb, t, g);
+    const int ns = dkv_split_count(items, target);
+    const int per = (items + ns - 1) / ns;
+    for (int c = 0; c < ns; ++c) atomicAdd(&hist[bucket_of(max(0, min(per, items - c * per)))], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int i = 0; i < 256; ++i) {
+      const int n = hist[i];
+      hist[i] = run;
+      run += n;
+    }
+    header[0] = run;
+    header[1] = target;
+  }
+  __syncthreads();
+
+  // Partial-slot offsets by a running scan over tiles, then scatter.
+  for (int base = 0; base < ntiles; base += 1024) {
+    const int t = base + tid;
+    int items = 0, ns = 1;
+    if (t < ntiles) {
+      items = dkv_tile_items(meta, nrb, t, g);
+      ns = dkv_split_count(items, target);
+    }
+    const int mine = (t < ntiles && ns > 1) ? ns : 0;
+    red[tid] = mine;
+    __syncthreads();
+    for (int s = 1; s < 1024; s <<= 1) {
+      const long long add = tid >= s ? red[tid - s] : 0;
+      __syncthreads();
+      red[tid] += add;
+      __syncthreads();
+    }
+    const int slot0 = carry + (int)red[tid] - mine;
+    const int chunk_total = (int)red[1023];
+    __syncthreads();
+    if (tid == 0) carry += chunk_total;
+    if (t < ntiles) {
+      const int per = (items + ns - 1) / ns;
+      for (int c = 0; c < ns; ++c) {
+        const int bk = bucket_of(max(0, min(per, items - c * per)));
+        const int pos = hist[bk] + atomicAdd(&fill[bk], 1);
+        entries[pos] = make_int2(t, c | (ns << 8) | (slot0 << 16));
+      }
+    }
+    __syncthreads();
+  }
+}
+
 template <int D>
 __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   extern __shared__ __align__(16) char smem_raw[];
@@ -219,12 +358,12 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
 
   const int l = lane_id(), j = l & 31, half = l >> 5, w = threadIdx.x >> 6;
   const int nrb = p.S / 32;
-  const int groups = p.B * p.Hkv;
-  const int group = blockIdx.x % groups, rank = blockIdx.x / groups;
-  const int kvh = group % p.Hkv;
-  const int b = group / p.Hkv;
-  const int kt =
-      uniform(p.sched[(size_t)b * schedule_ints(nrb) + key_schedule_offset(nrb) + rank]);
+  const int kvh = blockIdx.x % p.Hkv, entry = blockIdx.x / p.Hkv;
+  if (entry >= uniform(p.dkv_header[0])) return;
+  const int2 work_entry = p.dkv_entries[entry];
+  const int tile = uniform(work_entry.x), packed = uniform(work_entry.y);
+  const int chunk = packed & 255, nsplit = (packed >> 8) & 255, slot0 = (unsigned)packed >> 16;
+  const int b = tile / (nrb / 4), kt = tile % (nrb / 4);
   const int g = p.Hq / p.Hkv;
   const int* meta_b = p.meta + (size_t)b * nrb * kMetaW;
   const RowFragOffsets<D / 8> ro(lds0);
@@ -267,8 +406,14 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
 
   // Work items: (head of the group, query block) pairs, flattened; query block fastest.
   const int nq = (q_lo <= q_hi) ? (q_hi - q_lo + 1) : 0;
-  const int items = nq * g;
-  int it = 0, qb = q_lo, head = kvh * g;
+  const int per_chunk = (nq * g + nsplit - 1) / nsplit;
+  int it = chunk * per_chunk;
+  const int items = min(nq * g, it + per_chunk);  // end of this chunk's item range
+  int qb = q_lo, head = kvh * g;
+  if (it < items) {
+    head += it / nq;
+    qb += it % nq;
+  }
   const TileDma<kQueryTile, D / 8> dma;
   if (it < items) {
     QueryRowRegs regs;
@@ -335,6 +480,44 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
     step(std::integral_constant<int, 0>{});
     if (it >= items) break;
     step(std::integral_constant<int, 1>{});
+  }
+
+  if (nsplit > 1) {
+    // Leave this chunk's sums as f32, laid out [dK | dV][wavefront][d block][register][lane].
+    constexpr int kPerWave = (D / 32) * 16 * 64;
+    constexpr size_t kPerChunk = 2 * 4 * kPerWave;
+    float* mine = p.dkv_partials + ((size_t)(slot0 + chunk) * p.Hkv + kvh) * kPerChunk + w * kPerWave + l;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        mine[(db * 16 + r) * 64] = dkacc[db][r];
+        mine[4 * kPerWave + (db * 16 + r) * 64] = dvacc[db][r];
+      }
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0)
+      lds_store<int>(lds0 + QdoStage<D>::kLastFlag,
+                     atomicAdd(&p.dkv_counters[tile * p.Hkv + kvh], 1) == nsplit - 1);
+    __syncthreads();
+    if (!uniform(lds_load<int>(lds0 + QdoStage<D>::kLastFlag))) return;
+    __threadfence();
+    // Last chunk to arrive: add all chunks in chunk order.
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) {
+      dkacc[db] = zero16();
+      dvacc[db] = zero16();
+    }
+    for (int c = 0; c < nsplit; ++c) {
+      const float* src = p.dkv_partials + ((size_t)(slot0 + c) * p.Hkv + kvh) * kPerChunk + w * kPerWave + l;
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          dkacc[db][r] += src[(db * 16 + r) * 64];
+          dvacc[db][r] += src[4 * kPerWave + (db * 16 + r) * 64];
+        }
+    }
   }
 
   const lds_addr patch = vpatch;  // V fragments are no longer needed

@@ -53,6 +53,46 @@ __host__ __device__ inline int query_schedule_offset(int nrb, int pb) {
 }
 __host__ __device__ inline int key_schedule_offset(int nrb) { return nrb + nrb / 2 + nrb / 4; }
 
+// ---------------------------------------------------------------------------
+// dK/dV work list (backward workspace).
+//
+// A 128-key tile's work is the list of (query head of the group, visiting
+// 32-row query block) items. Tiles at the start of a long segment carry many
+// times the mean, so the list of a heavy tile is cut into up to kDkvMaxSplit
+// chunks of about half a compute slot's fair share; every chunk is one
+// workgroup, chunks are dispatched heaviest first, and the chunks of a split
+// tile leave f32 partial sums that the last one to finish adds up in chunk
+// order (fixed order: results do not depend on timing).
+// Workspace: header (entry count, chunk target), one arrival counter per
+// (tile, KV head), the sorted entries, the partial sums.
+// ---------------------------------------------------------------------------
+constexpr int kDkvSlots = 512;     // workgroups resident at once on the device (2 per CU)
+constexpr int kDkvMinChunk = 16;   // items
+constexpr int kDkvMaxSplit = 32;
+constexpr int kDkvKeys = 128;      // keys per dK/dV tile
+
+struct DkvLayout {
+  int max_entries, max_partials;
+  size_t header, counters, entries, partials, total;
+};
+
+// Sum over tiles of the chunk count is at most tiles + total_items / target and the
+// target is at least total_items * kv_heads / (2 * kDkvSlots).
+__host__ inline DkvLayout dkv_layout(int B, int S, int Hkv, int D) {
+  DkvLayout L;
+  const int tiles = B * (S / kDkvKeys);
+  const int extra = (2 * kDkvSlots + Hkv - 1) / Hkv + 1;
+  L.max_entries = tiles + extra;
+  L.max_partials = min(2 * extra, L.max_entries);
+  auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+  L.header = 0;
+  L.counters = 256;
+  L.entries = L.counters + up((size_t)tiles * Hkv * sizeof(int));
+  L.partials = L.entries + up((size_t)L.max_entries * 2 * sizeof(int));
+  L.total = L.partials + (size_t)L.max_partials * Hkv * 2 * kDkvKeys * D * sizeof(float);
+  return L;
+}
+
 struct KeyTileBounds {
   int min_nz;
   int max_id;

@@ -78,7 +78,8 @@ ffi::Error AttnBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> q, ffi::Buffer<ffi
                    ffi::Buffer<ffi::BF16> out, ffi::Buffer<ffi::F32> lse,
                    ffi::Buffer<ffi::BF16> dout, ffi::ResultBuffer<ffi::BF16> dq,
                    ffi::ResultBuffer<ffi::BF16> dk, ffi::ResultBuffer<ffi::BF16> dv,
-                   ffi::ResultBuffer<ffi::F32> delta_scratch, float scale, bool has_end) {
+                   ffi::ResultBuffer<ffi::F32> delta_scratch, ffi::ResultBuffer<ffi::U8> workspace,
+                   float scale, bool has_end) {
   const auto qd = q.dimensions();
   const auto kd = k.dimensions();
   if (qd.size() != 4 || kd.size() != 4)
@@ -97,6 +98,8 @@ ffi::Error AttnBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> q, ffi::Buffer<ffi
   a.dk = bits_out(dk);
   a.dv = bits_out(dv);
   a.delta = delta_scratch->typed_data();
+  a.workspace = workspace->untyped_data();
+  a.workspace_bytes = workspace->size_bytes();
   a.batch = (int32_t)qd[0];
   a.seq = (int32_t)qd[1];
   a.q_heads = (int32_t)qd[2];
@@ -199,6 +202,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_attn_bwd, AttnBwd,
                                   .Ret<ffi::Buffer<ffi::BF16>>()
                                   .Ret<ffi::Buffer<ffi::BF16>>()
                                   .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
                                   .Attr<float>("scale")
                                   .Attr<bool>("has_end"));
 

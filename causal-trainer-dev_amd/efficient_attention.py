@@ -361,6 +361,8 @@ def _attn_backward(query, key, value, metadata, out, lse, dout, scale):
     dk = torch.empty_like(key)
     dv = torch.empty_like(value)
     delta = torch.empty_like(lse)
+    workspace_bytes = int(_lib.load().ct_attn_bwd_workspace_bytes(batch, sequence, key.shape[2], head_dim))
+    workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=query.device)
     args = _lib.AttnBwdArgs(
         q=query.data_ptr(), k=key.data_ptr(), v=value.data_ptr(),
         segment_ids=metadata.query_segment_ids.data_ptr(),
@@ -368,6 +370,7 @@ def _attn_backward(query, key, value, metadata, out, lse, dout, scale):
         tile_meta=metadata.tile_bounds.data_ptr(),
         out=out.data_ptr(), lse=lse.data_ptr(), dout=dout.data_ptr(),
         dq=dq.data_ptr(), dk=dk.data_ptr(), dv=dv.data_ptr(), delta=delta.data_ptr(),
+        workspace=workspace.data_ptr(), workspace_bytes=workspace_bytes,
         batch=batch, seq=sequence, q_heads=q_heads, kv_heads=key.shape[2], head_dim=head_dim,
         scale=scale,
     )

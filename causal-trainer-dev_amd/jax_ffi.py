@@ -42,7 +42,8 @@ def _workspace_bytes(kind: str, rows: int, hidden: int, vocab: int) -> int:
 
 
 def tile_bounds(segment_ids, attention_end=None):
-    """int32 [B, S/32, 12] per-tile bounds; call once per forward, next to prepare_attention_metadata."""
+    """Flat int32 tile table + schedules (ct_attn_meta_bytes); call once per forward, next to
+    prepare_attention_metadata, and reuse for every layer."""
 
     import jax
     import jax.numpy as jnp
@@ -50,7 +51,10 @@ def tile_bounds(segment_ids, attention_end=None):
     register()
     batch, seq = segment_ids.shape
     has_end = attention_end is not None
-    out = jax.ShapeDtypeStruct((batch, seq // 32, 12), jnp.int32)
+    from . import _lib
+
+    words = int(_lib.load().ct_attn_meta_bytes(batch, seq)) // 4
+    out = jax.ShapeDtypeStruct((words,), jnp.int32)
     return jax.ffi.ffi_call("ct_ffi_attn_prepare", out)(
         segment_ids, attention_end if has_end else segment_ids, has_end=has_end)
 
@@ -81,9 +85,13 @@ def make_efficient_attention():
     def attention_bwd(scale, residual, dout):
         q, k, v, segment_ids, attention_end, bounds, out, lse = residual
         has_end = attention_end is not None
+        from . import _lib
+
+        scratch = int(_lib.load().ct_attn_bwd_workspace_bytes(q.shape[0], q.shape[1], k.shape[2], q.shape[3]))
         shapes = (jax.ShapeDtypeStruct(q.shape, q.dtype), jax.ShapeDtypeStruct(k.shape, k.dtype),
-                  jax.ShapeDtypeStruct(v.shape, v.dtype), jax.ShapeDtypeStruct(lse.shape, jnp.float32))
-        dq, dk, dv, _ = jax.ffi.ffi_call("ct_ffi_attn_bwd", shapes)(
+                  jax.ShapeDtypeStruct(v.shape, v.dtype), jax.ShapeDtypeStruct(lse.shape, jnp.float32),
+                  jax.ShapeDtypeStruct((scratch,), jnp.uint8))
+        dq, dk, dv, _, _ = jax.ffi.ffi_call("ct_ffi_attn_bwd", shapes)(
             q, k, v, segment_ids, attention_end if has_end else segment_ids, bounds, out, lse,
             dout.astype(jnp.bfloat16), scale=jnp.float32(scale), has_end=has_end)
         return dq, dk, dv, None, None, None

@@ -141,14 +141,24 @@ typedef struct ct_attn_bwd_args {
   uint16_t* dk;                 /* bf16 [batch, seq, kv_heads, head_dim] */
   uint16_t* dv;                 /* bf16 [batch, seq, kv_heads, head_dim] */
   float* delta;                 /* f32 scratch [batch, seq, q_heads] */
+  void* workspace;              /* scratch, ct_attn_bwd_workspace_bytes(); contents need not be kept */
+  size_t workspace_bytes;
   int32_t batch, seq, q_heads, kv_heads, head_dim;
   float scale;
 } ct_attn_bwd_args;
 
+/* Bytes of scratch ct_attn_bwd needs: the dK/dV work list (key tiles whose
+ * list of visiting query blocks is long are cut into chunks that run as
+ * separate workgroups) and the f32 partial sums of such chunks. 0 for an
+ * unsupported shape. No reference counterpart (the reference's dK/dV kernel
+ * accumulates in its f32 output window, src/kernels/efficient_attention.py:1545-1549). */
+size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t kv_heads, int32_t head_dim);
+
 /*
- * dq, dk, dv from the saved (q, k, v, out, lse) and dout. Three launches:
- * delta = rowsum(out * dout); dq per query tile; dk/dv per key tile (single
- * owner, no atomics, deterministic).
+ * dq, dk, dv from the saved (q, k, v, out, lse) and dout. Four launches:
+ * delta = rowsum(out * dout); dq per query tile; the dK/dV work list; dk/dv
+ * per key tile (chunks of a split tile are summed in a fixed order, so the
+ * result is deterministic).
  * Replaces: delta at src/kernels/efficient_attention.py:1735-1738,
  * _local_attention_dq (:985-1267), _local_attention_dkv (:1270-1602) and the
  * f32 -> bf16 cast at :1774.

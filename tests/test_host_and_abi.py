@@ -26,6 +26,8 @@ def test_size_queries_need_no_gpu(ct):
     library = ct._lib.load()
     assert library.ct_attn_meta_bytes(4, 4096) == 4 * (4096 // 32) * (12 + 2) * 4
     assert library.ct_attn_meta_bytes(0, 128) == 0
+    assert 0 < library.ct_attn_bwd_workspace_bytes(4, 4096, 8, 128) < 1 << 30
+    assert library.ct_attn_bwd_workspace_bytes(4, 4000, 8, 128) == 0
     shape = ct._lib.CutceShape(16384, 4096, 128256)
     fwd = library.ct_cutce_fwd_workspace_bytes(ctypes.byref(shape))
     full = library.ct_cutce_bwd_workspace_bytes(ctypes.byref(shape))
@@ -49,6 +51,9 @@ def test_argument_validation_happens_before_any_launch(ct):
     assert b"divisible by the KV head count" in library.ct_last_error()
     args.q_heads, args.head_dim = 4, 96
     assert library.ct_attn_fwd(None, ctypes.byref(args)) == ct._lib.CT_UNSUPPORTED
+    args.head_dim, args.k = 128, 4096 + 8
+    assert library.ct_attn_fwd(None, ctypes.byref(args)) == ct._lib.CT_INVALID_ARGUMENT
+    assert b"16-byte aligned" in library.ct_last_error()
     shape = ct._lib.CutceShape(10, 100, 50)
     cargs = ct._lib.CutceFwdArgs(shape=shape)
     for field in ("hidden", "head", "targets", "weights", "nll_sum", "weight_sum", "lse", "workspace"):
