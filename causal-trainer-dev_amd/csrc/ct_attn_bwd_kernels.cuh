@@ -372,14 +372,14 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   int q_lo = INT_MAX, q_hi = -1;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int* m = meta_b + (kt * 4 + i) * kMetaW;
+    const MetaPtr m = meta_const(meta_b + (kt * 4 + i) * kMetaW);
     q_lo = min(q_lo, uniform(m[kQFirst]));
     q_hi = max(q_hi, uniform(m[kQLast]));
   }
   const int my_rb = kt * 4 + w;
-  const int my_min = uniform(meta_b[my_rb * kMetaW + kMinNz]);
-  const int my_max = uniform(meta_b[my_rb * kMetaW + kMaxId]);
-  const int my_uni = uniform(meta_b[my_rb * kMetaW + kUniform]);
+  const int my_min = uniform(meta_const(meta_b)[my_rb * kMetaW + kMinNz]);
+  const int my_max = uniform(meta_const(meta_b)[my_rb * kMetaW + kMaxId]);
+  const int my_uni = uniform(meta_const(meta_b)[my_rb * kMetaW + kUniform]);
 
   const int key = my_rb * 32 + j;
   const int seg_k = p.seg[(size_t)b * p.S + key];
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
     QueryRowRegs regs;
     if (more) qdo_fetch<D>(regs, dma, p, b, head_next, qb_next, lds0 + (CUR ^ 1) * kStage);
 
-    const int* qm = meta_b + qb * kMetaW;
+    const MetaPtr qm = meta_const(meta_b + qb * kMetaW);
     const int q_min = uniform(qm[kMinNz]), q_max = uniform(qm[kMaxId]),
               q_end_max = uniform(qm[kEndMax]), q_end_min = uniform(qm[kEndMin]),
               q_uni = uniform(qm[kUniform]);

@@ -217,7 +217,7 @@ struct QueryTileContext {
     last = -1;
 #pragma unroll
     for (int i = 0; i < PB; ++i) {
-      const int* m = meta_b + (work.qt * PB + i) * kMetaW;
+      const MetaPtr m = meta_const(meta_b + (work.qt * PB + i) * kMetaW);
       first = min(first, uniform(m[kKvFirst]));
       last = max(last, uniform(m[kKvLast]));
     }

@@ -99,10 +99,17 @@ struct KeyTileBounds {
   int uniform;
 };
 
+// The table is written by an earlier kernel and only read here. Reading it through the
+// constant address space makes wave-uniform accesses scalar loads: they are counted by
+// lgkmcnt, so waiting for them does not also wait for the asynchronous tile copies in
+// flight (a vector load would, vmcnt completes in order).
+typedef __attribute__((address_space(4))) const int* MetaPtr;
+CT_DEVICE MetaPtr meta_const(const int* p) { return (MetaPtr)p; }
+
 // Bounds of the 64-key tile `t` = row blocks 2t and 2t+1 (wave-uniform).
 CT_DEVICE KeyTileBounds key_tile_bounds(const int* meta_b, int t) {
-  const int* a = meta_b + (2 * t) * kMetaW;
-  const int* c = a + kMetaW;
+  const MetaPtr a = meta_const(meta_b + (2 * t) * kMetaW);
+  const MetaPtr c = a + kMetaW;
   const int a_min = a[kMinNz], c_min = c[kMinNz];
   KeyTileBounds out;
   out.min_nz = a_min == 0 ? c_min : (c_min == 0 ? a_min : min(a_min, c_min));
@@ -116,7 +123,7 @@ struct QueryBlockBounds {
 };
 
 CT_DEVICE QueryBlockBounds query_block_bounds(const int* meta_b, int rb) {
-  const int* m = meta_b + rb * kMetaW;
+  const MetaPtr m = meta_const(meta_b + rb * kMetaW);
   QueryBlockBounds q;
   q.min_nz = uniform(m[kMinNz]);
   q.max_id = uniform(m[kMaxId]);
