@@ -15,7 +15,7 @@ namespace ct {
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, const int* end, int S,
                                                             int* meta, int* sched_all) {
-  extern __shared__ int lds_meta[];  // [nrb][3]: min_nz, max_id, end_max
+  extern __shared__ int lds_meta[];  // [nrb][3]: min_nz, max_id, end_max; later schedule_ints(nrb) work counts
   const int b = blockIdx.x;
   const int nrb = S / 32, nt = S / kKeyTile;
   const int* segb = seg + (size_t)b * S;
@@ -122,12 +122,22 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, cons
     }
     work[offk + i] = last >= first ? last - first + 1 : 0;
   }
+  const int off8 = 2 * nrb, n8 = (nrb + 7) / 8;
+  for (int i = threadIdx.x; i < n8; i += blockDim.x) {
+    int first = INT_MAX, last = -1;
+    for (int k = 0; k < 8 && i * 8 + k < nrb; ++k) {
+      const int* m = mb + (i * 8 + k) * kMetaW;
+      first = min(first, m[kKvFirst]);
+      last = max(last, m[kKvLast]);
+    }
+    work[off8 + i] = last >= first ? last - first + 1 : 0;
+  }
   __syncthreads();
 
   // Phase 4: rank sort (descending work, ties by index) -> schedules.
-  const int counts[4] = {nrb, nrb / 2, nrb / 4, nrb / 4};
-  const int offsets[4] = {0, off2, off4, offk};
-  for (int sidx = 0; sidx < 4; ++sidx) {
+  const int counts[5] = {nrb, nrb / 2, nrb / 4, nrb / 4, n8};
+  const int offsets[5] = {0, off2, off4, offk, off8};
+  for (int sidx = 0; sidx < 5; ++sidx) {
     const int n = counts[sidx];
     const int* wk = work + offsets[sidx];
     int* out = sched + offsets[sidx];
@@ -202,16 +212,16 @@ static int heads_per_group(int Hq, int Hkv) {
 
 template <int D, int HS>
 static int launch_fwd(hipStream_t stream, const AttnParams& p) {
-  constexpr int PB = 4 / HS;
-  const size_t smem = 2 * KvStage<D>::kBytes;
+  constexpr int PB = kFwdWaves / HS;
+  const size_t smem = VkStage<D>::kTotalBytes;
   {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, HS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_fwd: %s", hipGetErrorString(e));
   }
-  const int grid = (p.S / (32 * PB)) * (p.Hq / HS) * p.B;
+  const int grid = ((p.S / 32 + PB - 1) / PB) * (p.Hq / HS) * p.B;
   LaunchScope scope1("attn_fwd_kernel", stream);
-  hipLaunchKernelGGL((attn_fwd_kernel<D, HS>), dim3(grid), dim3(256), smem, stream, p);
+  hipLaunchKernelGGL((attn_fwd_kernel<D, HS>), dim3(grid), dim3(kFwdWaves * 64), smem, stream, p);
   return scope1.done();
 }
 
@@ -288,7 +298,8 @@ using namespace ct;
 
 extern "C" size_t ct_attn_meta_bytes(int32_t batch, int32_t seq) {
   if (batch <= 0 || seq <= 0) return 0;
-  return (size_t)batch * (size_t)(seq / 32) * (kMetaW + 2) * sizeof(int32_t);
+  const size_t nrb = (size_t)(seq / 32);
+  return (size_t)batch * (nrb * kMetaW + schedule_ints((int)nrb)) * sizeof(int32_t);
 }
 
 extern "C" size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t kv_heads,

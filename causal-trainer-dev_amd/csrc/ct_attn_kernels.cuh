@@ -96,9 +96,9 @@ struct KvFetcher {
 // XCD (ids are dealt round robin to the 8 XCDs) and keeps its K/V in that L2;
 // the rank is the position in the batch row's work-sorted schedule, longest
 // tiles first.
-template <int HS>
+template <int HS, int NW = 4>
 struct QueryWork {
-  static constexpr int PB = 4 / HS;  // row blocks per workgroup
+  static constexpr int PB = NW / HS;  // row blocks per workgroup
   int b, h, kvh, qt, rb;
   CT_DEVICE QueryWork(const AttnParams& p) {
     const int nrb = p.S / 32;
@@ -196,15 +196,16 @@ CT_DEVICE void store_rows_t(const f32x16* acc, float row_scale, lds_addr patch, 
 }
 
 // Shared prologue of the forward and dQ kernels.
-template <int D, int HS>
+template <int D, int HS, int NW = 4>
 struct QueryTileContext {
-  static constexpr int PB = 4 / HS;
-  QueryWork<HS> work;
+  static constexpr int PB = NW / HS;
+  QueryWork<HS, NW> work;
   const int* meta_b;
   QueryBlockBounds mine;
   int first, last;
   int pos, seg_q, end_q;
   bool row_valid;
+  bool active;  // false for the row blocks past the end of a partial last tile
   size_t q_off, stat_off;
   const bf16* kbase;
   const bf16* vbase;
@@ -212,11 +213,15 @@ struct QueryTileContext {
   CT_DEVICE explicit QueryTileContext(const AttnParams& p) : work(p) {
     const int nrb = p.S / 32;
     meta_b = p.meta + (size_t)work.b * nrb * kMetaW;
+    active = work.rb < nrb;
+    if (!active) work.rb = nrb - 1;  // keeps every address below in range
     mine = query_block_bounds(meta_b, work.rb);
+    if (!active) mine.min_nz = 0;    // interacts with nothing
     first = INT_MAX;
     last = -1;
 #pragma unroll
     for (int i = 0; i < PB; ++i) {
+      if (work.qt * PB + i >= nrb) break;
       const MetaPtr m = meta_const(meta_b + (work.qt * PB + i) * kMetaW);
       first = min(first, uniform(m[kKvFirst]));
       last = max(last, uniform(m[kKvLast]));
@@ -244,15 +249,80 @@ struct QueryTileContext {
 
 // ---------------------------------------------------------------------------
 // Forward
+//
+// One workgroup of 8 wavefronts per compute unit: wavefronts w and w + 4 share
+// a SIMD. Per key tile a wavefront alternates between a VALU phase (softmax of
+// the tile's scores) and an MFMA phase (O += V^T P of this tile, then the
+// scores of the next tile). Wavefronts 4..7 (the "late" group) run half a step
+// behind wavefronts 0..3 (they pass one extra barrier before the loop, the
+// others one after it), and a workgroup barrier closes every phase, so on each
+// SIMD one wavefront is in its VALU phase while the other one is in its MFMA
+// phase and the two pipes overlap.
+//
+// Global phase numbering: the early group runs VALU phase t in phase 2t and
+// MFMA phase t in phase 2t + 1; the late group one phase later. LDS holds 2
+// stages; stage s = V rows of tile s and K rows of tile s + 1, exactly the
+// operands of MFMA phase s, read in phases 2s + 1 and 2s + 2. The copies for
+// stage t + 1 replace stage t - 1 and are issued at the start of phase 2t + 1
+// (early group: on entering MFMA phase t; late group: on entering VALU phase
+// t) and awaited at the end of phase 2t + 2, one barrier before the first read.
+// Segment ids of the key tiles go through a ring of 4 slots (tile t in slot
+// t % 4, copied together with stage t - 1, read in phases 2t and 2t + 1).
 // ---------------------------------------------------------------------------
+constexpr int kFwdWaves = 8;
+constexpr float kRescaleSlack = 8.f;
+
+template <int D>
+struct VkStage {
+  static constexpr int kTileBytes = kKeyTile * D * 2;
+  static constexpr int kV = 0;
+  static constexpr int kK = kTileBytes;
+  static constexpr int kBytes = 2 * kTileBytes;
+  static constexpr int kSegRing = 2 * kBytes;  // after both stages
+  static constexpr int kSegSlotBytes = kKeyTile * 4;
+  static constexpr int kTotalBytes = kSegRing + 4 * kSegSlotBytes;
+  // offset of the slot that holds the ids of key tile t
+  static CT_DEVICE int seg_slot(int t) { return kSegRing + (t & 3) * kSegSlotBytes; }
+};
+
+template <int D>
+struct VkFetcher {
+  TileDma<kKeyTile, D / 8, kFwdWaves * 64> dma;
+  const char* kbase;
+  const char* vbase;
+  const int* segb;
+  size_t row_stride_bytes;
+  CT_DEVICE VkFetcher(const bf16* k, const bf16* v, const int* seg, size_t row_stride_elems)
+      : kbase(reinterpret_cast<const char*>(k)), vbase(reinterpret_cast<const char*>(v)),
+        segb(seg), row_stride_bytes(row_stride_elems * 2) {}
+  CT_DEVICE void issue_v(int tile, lds_addr stage) const {
+    dma.issue(vbase + (size_t)tile * kKeyTile * row_stride_bytes, row_stride_bytes,
+              stage + VkStage<D>::kV);
+  }
+  // K rows of `tile` into `stage`, its segment ids into the ring (lds0 = start of LDS)
+  CT_DEVICE void issue_k(int tile, lds_addr stage, lds_addr lds0) const {
+    dma.issue(kbase + (size_t)tile * kKeyTile * row_stride_bytes, row_stride_bytes,
+              stage + VkStage<D>::kK);
+    if (threadIdx.x < 16)  // 64 ids = 16 lanes x 16 bytes, linear layout
+      dma16(segb + tile * kKeyTile + threadIdx.x * 4, lds0 + VkStage<D>::seg_slot(tile));
+  }
+  // stage s: V(s), K(s + 1); tiles past `last` are skipped
+  CT_DEVICE void issue_stage(int s, int last, lds_addr stage, lds_addr lds0) const {
+    if (s <= last) issue_v(s, stage);
+    if (s + 1 <= last) issue_k(s + 1, stage, lds0);
+  }
+};
+
 template <int D, int HS>
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
+__global__ __launch_bounds__(kFwdWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
+attn_fwd_kernel(AttnParams p) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr lds0 = lds_address_of(smem_raw);
-  constexpr int kStage = KvStage<D>::kBytes;
+  constexpr int kStage = VkStage<D>::kBytes;
 
-  const QueryTileContext<D, HS> ctx(p);
+  const QueryTileContext<D, HS, kFwdWaves> ctx(p);
   const int l = lane_id(), half = l >> 5, w = threadIdx.x >> 6;
+  const bool late = uniform(w) >= kFwdWaves / 2;
   const RowFragOffsets<D / 8> ro(lds0);
   const TrFragOffsets<D / 8, KSlots::kAccum> to(lds0);
   const size_t q_row_stride = (size_t)p.Hq * D;
@@ -266,35 +336,40 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
   f32x16 oacc[D / 32];
 #pragma unroll
   for (int db = 0; db < D / 32; ++db) oacc[db] = zero16();
-  float m_run = kNegInf;  // running max, log2 domain
-  float l_run = 0.f;      // this lane's share of the running sum
+  float m_run = kNegInf;  // softmax reference (a recent running max), log2 domain
+  float l_run = 0.f;      // this lane's share of the running sum (f32: the LSE is held to 1e-3)
 
-  const KvFetcher<D> fetch(ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride);
+  const VkFetcher<D> fetch(ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride);
   int t = ctx.first;
+  const int last = ctx.last;
   KeyTileBounds kb = {0, 0, 0};
-  if (t <= ctx.last) {
-    fetch.issue(t, lds0);
+  f32x16 s[2];
+  bool visit = false;
+  if (t <= last) {
+    fetch.issue_k(t, lds0 + kStage, lds0);  // stage first - 1 (buffer 1): only its K half
+    fetch.issue_stage(t, last, lds0, lds0);  // stage first -> buffer 0
     kb = key_tile_bounds(ctx.meta_b, t);
+    visit = ctx.wave_visits(kb, t);
   }
   dma_wait_all();
   __syncthreads();
+  if (visit) scores_t<D>(kStage + VkStage<D>::kK, ro, qf, s);
+  if (late) __builtin_amdgcn_s_barrier();
 
+  // One step = VALU phase + MFMA phase of tile t; CUR is the buffer of stage t.
   auto step = [&](auto stage_tag) {
     constexpr int CUR = decltype(stage_tag)::value;
-    const lds_addr stage = lds0 + CUR * kStage;
-    const bool more = t + 1 <= ctx.last;
+    const lds_addr next_stage = lds0 + (CUR ^ 1) * kStage;
+    // ---- VALU phase ----
+    if (late) fetch.issue_stage(t + 1, last, next_stage, lds0);
     KeyTileBounds nb = kb;
-    if (more) {
-      fetch.issue(t + 1, lds0 + (CUR ^ 1) * kStage);
-      nb = key_tile_bounds(ctx.meta_b, t + 1);
-    }
-    if (ctx.wave_visits(kb, t)) {
-      f32x16 s[2];
-      scores_t<D>(CUR * kStage + KvStage<D>::kK, ro, qf, s);
+    if (t + 1 <= last) nb = key_tile_bounds(ctx.meta_b, t + 1);
+    bf16x8 pf[4];
+    if (visit) {
       float mx = kNegInf;
       if (!ctx.interior(kb, t)) {
         unsigned allow[2];
-        tile_mask(stage + KvStage<D>::kSeg, t, ctx.seg_q, ctx.end_q, ctx.row_valid, allow);
+        tile_mask(lds0 + VkStage<D>::seg_slot(t), t, ctx.seg_q, ctx.end_q, ctx.row_valid, allow);
 #pragma unroll
         for (int kbk = 0; kbk < 2; ++kbk)
 #pragma unroll
@@ -306,8 +381,22 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kbk][r]);
       mx = fmaxf(mx, xor32(mx)) * kLog2e;
-      const float m_new = fmaxf(m_run, mx);
-      const float m_use = (m_new == kNegInf) ? 0.f : m_new;
+      // The running reference m_run only follows the true maximum when that has grown by
+      // more than kRescaleSlack (log2 units): probabilities are then at most 2^slack, well
+      // inside bf16 / f32 range, the normalisation by the row sum is unchanged, and the
+      // accumulator is rescaled on few tiles instead of most.
+      if (__any(mx > m_run + kRescaleSlack)) {
+        const float m_new = fmaxf(m_run, mx);
+        const float m_use = (m_new == kNegInf) ? 0.f : m_new;
+        const float alpha = exp2_fast(m_run - m_use);  // m_run = -inf -> 0
+        l_run *= alpha;
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+        m_run = m_new;
+      }
+      const float m_use = (m_run == kNegInf) ? 0.f : m_run;
       float psum = 0.f;
 #pragma unroll
       for (int kbk = 0; kbk < 2; ++kbk)
@@ -316,32 +405,59 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(AttnParams p) {
           s[kbk][r] = exp2_fast(fmaf(s[kbk][r], kLog2e, -m_use));
           psum += s[kbk][r];
         }
-      if (__any(m_new != m_run)) {
-        const float alpha = exp2_fast(m_run - m_use);
-        l_run *= alpha;
+      l_run += psum;
+#pragma unroll
+      for (int step4 = 0; step4 < 4; ++step4) pf[step4] = pack_acc8(s[step4 >> 1], step4 & 1);
+    }
+    if (!late) dma_wait_all();  // stage t, issued one step ago
+    __builtin_amdgcn_s_barrier();
+    // ---- MFMA phase ----
+    if (!late) fetch.issue_stage(t + 1, last, next_stage, lds0);
+    if (visit) {
+#pragma unroll
+      for (int step4 = 0; step4 < 4; ++step4)
 #pragma unroll
         for (int db = 0; db < D / 32; ++db)
+          oacc[db] = mfma32(to.load(CUR * kStage + VkStage<D>::kV, step4, db), pf[step4], oacc[db]);
+      // LDS fragment reads run kAhead fragments ahead of the MFMA that consumes them.
+      constexpr int kMfma = 4 * (D / 32), kAhead = 4;
+      __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
 #pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
-        m_run = m_new;
+      for (int i = 0; i < kMfma; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i + kAhead < kMfma) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
       }
-      l_run += psum;
-      accumulate_t<D>(CUR * kStage + KvStage<D>::kV, to, s, oacc);
     }
-    dma_wait_all();
-    __syncthreads();
+    const bool visit_next = (t + 1 <= last) && ctx.wave_visits(nb, t + 1);
+    if (visit_next) {
+      scores_t<D>(CUR * kStage + VkStage<D>::kK, ro, qf, s);
+      constexpr int kMfma = 2 * (D / 16), kAhead = 6;
+      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+      for (int i = 0; i < kMfma; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        if (i + kAhead < kMfma) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+    }
+    if (late) dma_wait_all();  // stage t + 1, issued at the start of this step
+    __builtin_amdgcn_s_barrier();
+    visit = visit_next;
     kb = nb;
     ++t;
   };
-  while (t <= ctx.last) {
+  while (t <= last) {
     step(std::integral_constant<int, 0>{});
-    if (t > ctx.last) break;
+    if (t > last) break;
     step(std::integral_constant<int, 1>{});
   }
+  if (!late) __builtin_amdgcn_s_barrier();
+  dma_wait_all();
+  __syncthreads();  // every wavefront is done with the stages before they become store patches
 
   const float l_tot = l_run + xor32(l_run);
   const bool has = l_tot > 0.f;
   const float inv = has ? 1.f / l_tot : 0.f;
+  if (!ctx.active) return;
   if (half == 0) p.lse[ctx.stat_off] = has ? (__logf(l_tot) + m_run * kLn2) : 0.f;
   const lds_addr patch = lds0 + w * 32 * D * 2;
   bf16* obase = p.out + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;

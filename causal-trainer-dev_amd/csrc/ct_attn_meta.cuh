@@ -23,7 +23,8 @@
 // work, so that the hardware's in-order workgroup dispatch places the longest
 // tiles first:
 //   query tiles of 1, 2 and 4 row blocks (by number of key tiles to visit),
-//   128-key tiles (by number of query blocks to visit).
+//   128-key tiles (by number of query blocks to visit),
+//   query tiles of 8 row blocks (the last one may be partial).
 #pragma once
 
 #include <limits.h>
@@ -45,11 +46,12 @@ enum MetaSlot {
   kQLast = 8,
 };
 
-// ints of schedule data per batch row (nrb + nrb/2 + nrb/4 + nrb/4)
-__host__ __device__ inline int schedule_ints(int nrb) { return 2 * nrb; }
-// offset of the schedule for query tiles of pb row blocks (pb = 1, 2, 4) inside a row's schedules
+// ints of schedule data per batch row (nrb + nrb/2 + nrb/4 + nrb/4, then ceil(nrb/8) <= nrb/4)
+__host__ __device__ inline int schedule_ints(int nrb) { return 2 * nrb + nrb / 4; }
+// offset of the schedule for query tiles of pb row blocks (pb = 1, 2, 4, 8) inside a row's
+// schedules; a row has ceil(nrb / pb) tiles of pb blocks
 __host__ __device__ inline int query_schedule_offset(int nrb, int pb) {
-  return pb == 1 ? 0 : (pb == 2 ? nrb : nrb + nrb / 2);
+  return pb == 1 ? 0 : (pb == 2 ? nrb : (pb == 4 ? nrb + nrb / 2 : 2 * nrb));
 }
 __host__ __device__ inline int key_schedule_offset(int nrb) { return nrb + nrb / 2 + nrb / 4; }
 

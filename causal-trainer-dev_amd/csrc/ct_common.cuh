@@ -124,13 +124,13 @@ CT_DEVICE int tile_byte_offset(int row, int chunk) {
 }
 
 // Global -> LDS copy of a ROWS x (8 CPR) bf16 tile into its swizzled layout by
-// the 256 threads of a workgroup: thread t owns the 16-byte LDS slots t + 256 n;
-// the swizzle is undone on the global side (each lane fetches the chunk that
-// belongs in its slot). Requires 16 | 256 / CPR, so one lane constant describes
-// all of a thread's slots.
-template <int ROWS, int CPR>
+// the THREADS threads of a workgroup: thread t owns the 16-byte LDS slots
+// t + THREADS n; the swizzle is undone on the global side (each lane fetches the
+// chunk that belongs in its slot). Requires 16 | THREADS / CPR, so one lane
+// constant describes all of a thread's slots.
+template <int ROWS, int CPR, int THREADS = 256>
 struct TileDma {
-  static constexpr int kRowsPerPass = 256 / CPR;
+  static constexpr int kRowsPerPass = THREADS / CPR;
   static constexpr int kPasses = ROWS / kRowsPerPass;
   static_assert(kRowsPerPass % 16 == 0 && ROWS % kRowsPerPass == 0, "unsupported tile shape");
   int row0, chunk;  // this thread's row in pass 0 and the logical chunk it fetches
@@ -145,7 +145,7 @@ struct TileDma {
     const char* p = src + (size_t)row0 * row_stride_bytes + chunk * 16;
 #pragma unroll
     for (int n = 0; n < kPasses; ++n)
-      dma16(p + (size_t)n * kRowsPerPass * row_stride_bytes, tile + (n * 256 + wave * 64) * 16);
+      dma16(p + (size_t)n * kRowsPerPass * row_stride_bytes, tile + (n * THREADS + wave * 64) * 16);
   }
 };
 

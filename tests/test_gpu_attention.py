@@ -248,14 +248,16 @@ def test_metadata_matches_oracle_bit_exact(ct, gpu):
                 assert bounds[b, rb, 2] == (block[0] if (block == block[0]).all() and block[0] != 0 else 0)
         # schedules: permutations, ordered by non-increasing work
         blocks = 1024 // 32
-        schedules = metadata.tile_bounds.cpu().numpy()[2 * blocks * 12:].reshape(2, 2 * blocks)
+        per_row = 2 * blocks + blocks // 4
+        schedules = metadata.tile_bounds.cpu().numpy()[2 * blocks * 12:].reshape(2, per_row)
         for b in range(2):
             spans = np.where(bounds[b, :, 6] >= bounds[b, :, 5], bounds[b, :, 6] - bounds[b, :, 5] + 1, 0)
             order = schedules[b, :blocks]
             assert sorted(order.tolist()) == list(range(blocks))
             assert (np.diff(spans[order]) <= 0).all()
             for offset, count in ((blocks, blocks // 2), (blocks + blocks // 2, blocks // 4),
-                                  (blocks + blocks // 2 + blocks // 4, blocks // 4)):
+                                  (blocks + blocks // 2 + blocks // 4, blocks // 4),
+                                  (2 * blocks, (blocks + 7) // 8)):
                 assert sorted(schedules[b, offset:offset + count].tolist()) == list(range(count))
 
 
