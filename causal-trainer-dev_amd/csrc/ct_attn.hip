@@ -153,6 +153,83 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, cons
   }
 }
 
+// Packs the query tiles of the whole batch into kBins bins of near equal work
+// (longest processing time first). One workgroup per tile size (2, 4, 8 row blocks);
+// the greedy pass runs on one wavefront, lane j keeping the load of bin j.
+__global__ __launch_bounds__(1024) void attn_bins_kernel(int* meta, int B, int S) {
+  extern __shared__ int lds_bins[];  // work[n], order[n], bin_of[n]
+  __shared__ int counts[kBins];
+  const int nrb = S / 32;
+  const int pb = 2 << blockIdx.x;
+  const int tpr = bin_tiles_per_row(nrb, pb), n = B * tpr;
+  int* work = lds_bins;
+  int* order = lds_bins + n;
+  int* bin_of = lds_bins + 2 * n;
+  int* region = meta + bin_region_offset(B, nrb, pb);
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int b = i / tpr, qt = i % tpr;
+    const int* mb = meta + (size_t)b * nrb * kMetaW;
+    int first = INT_MAX, last = -1;
+    for (int k = 0; k < pb && qt * pb + k < nrb; ++k) {
+      first = min(first, mb[(qt * pb + k) * kMetaW + kKvFirst]);
+      last = max(last, mb[(qt * pb + k) * kMetaW + kKvLast]);
+    }
+    // a tile without keys still costs a launch of the prologue; +3 ~ prologue and store
+    work[i] = (last >= first ? last - first + 1 : 0) + 3;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int wi = work[i];
+    int rank = 0;
+    for (int k = 0; k < n; ++k) {
+      const int wv = work[k];
+      rank += (wv > wi) || (wv == wi && k < i);
+    }
+    order[rank] = i;
+  }
+  __syncthreads();
+  if (threadIdx.x < 64) {
+    const int lane = threadIdx.x;
+    int load = lane < kBins ? 0 : INT_MAX;
+    for (int r = 0; r < n; ++r) {
+      // argmin over lanes (ties to the lowest bin): reduce (load, lane) keys
+      long long key = ((long long)load << 8) | lane;
+      for (int off = 32; off > 0; off >>= 1) {
+        const long long other = __shfl_xor(key, off, 64);
+        key = other < key ? other : key;
+      }
+      const int target = (int)(key & 0xff);
+      const int item = order[r];
+      if (lane == target) {
+        load += work[item];
+        bin_of[r] = target;
+      }
+    }
+  }
+  __syncthreads();
+  // offsets by counting, then a stable scatter in rank order (heaviest first inside a bin)
+  if (threadIdx.x < kBins) {
+    int count = 0;
+    for (int r = 0; r < n; ++r) count += bin_of[r] == (int)threadIdx.x;
+    counts[threadIdx.x] = count;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int run = 0;
+    for (int j = 0; j < kBins; ++j) {
+      region[j] = run;
+      run += counts[j];
+    }
+    region[kBins] = run;
+  }
+  __syncthreads();
+  if (threadIdx.x < kBins) {
+    int pos = region[threadIdx.x];
+    for (int r = 0; r < n; ++r)
+      if (bin_of[r] == (int)threadIdx.x) region[kBins + 1 + pos++] = order[r];
+  }
+}
+
 __global__ void attn_block_summary_kernel(const int* seg, const int* end, int S, int block,
                                           int nblocks, int width, int* out) {
   const int gid = blockIdx.x * blockDim.x + threadIdx.x;
@@ -219,7 +296,8 @@ static int launch_fwd(hipStream_t stream, const AttnParams& p) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_fwd: %s", hipGetErrorString(e));
   }
-  const int grid = ((p.S / 32 + PB - 1) / PB) * (p.Hq / HS) * p.B;
+  (void)PB;
+  const int grid = (p.Hq / HS) * kBins;  // (head slice, KV head) groups x work bins
   LaunchScope scope1("attn_fwd_kernel", stream);
   hipLaunchKernelGGL((attn_fwd_kernel<D, HS>), dim3(grid), dim3(kFwdWaves * 64), smem, stream, p);
   return scope1.done();
@@ -298,8 +376,7 @@ using namespace ct;
 
 extern "C" size_t ct_attn_meta_bytes(int32_t batch, int32_t seq) {
   if (batch <= 0 || seq <= 0) return 0;
-  const size_t nrb = (size_t)(seq / 32);
-  return (size_t)batch * (nrb * kMetaW + schedule_ints((int)nrb)) * sizeof(int32_t);
+  return meta_total_ints(batch, seq / 32) * sizeof(int32_t);
 }
 
 extern "C" size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t kv_heads,
@@ -326,7 +403,21 @@ extern "C" int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
   hipLaunchKernelGGL(attn_prepare_kernel, dim3(batch), dim3(threads), smem, (hipStream_t)stream,
                      segment_ids, attention_end, seq, tile_meta,
                      tile_meta + (size_t)batch * nrb * kMetaW);
-  return scope5.done();
+  rc = scope5.done();
+  if (rc) return rc;
+  const size_t bins_smem = (size_t)3 * batch * bin_tiles_per_row(nrb, 2) * sizeof(int);
+  CT_REQUIRE(bins_smem <= 160 * 1024 - 1024,
+             "ct_attn_prepare: batch %d x sequence %d has too many query tiles for the work bins",
+             batch, seq);
+  {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bins_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 1024);
+    if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_prepare: %s", hipGetErrorString(e));
+  }
+  LaunchScope scope8("attn_bins_kernel", (hipStream_t)stream);
+  hipLaunchKernelGGL(attn_bins_kernel, dim3(3), dim3(1024), bins_smem, (hipStream_t)stream, tile_meta,
+                     batch, seq);
+  return scope8.done();
 }
 
 extern "C" int32_t ct_attn_block_summary(void* stream, const int32_t* segment_ids,

@@ -134,9 +134,8 @@ CT_DEVICE void qdo_fetch(QueryRowRegs& r, const TileDma<kQueryTile, D / 8>& dma,
                          int b, int h, int qb, lds_addr stage) {
   const int tid = threadIdx.x;
   const size_t origin = (((size_t)b * p.S + qb * kQueryTile) * p.Hq + h) * D;
-  dma.issue(reinterpret_cast<const char*>(p.q + origin), (size_t)p.Hq * D * 2, stage + QdoStage<D>::kQ);
-  dma.issue(reinterpret_cast<const char*>(p.dout + origin), (size_t)p.Hq * D * 2,
-            stage + QdoStage<D>::kDo);
+  dma.issue(reinterpret_cast<const char*>(p.q + origin), stage + QdoStage<D>::kQ);
+  dma.issue(reinterpret_cast<const char*>(p.dout + origin), stage + QdoStage<D>::kDo);
   if (tid < kQueryTile) {
     const int pos = qb * kQueryTile + tid;
     const size_t so = ((size_t)b * p.S + pos) * p.Hq + h;
@@ -414,7 +413,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
     head += it / nq;
     qb += it % nq;
   }
-  const TileDma<kQueryTile, D / 8> dma;
+  const TileDma<kQueryTile, D / 8> dma((size_t)p.Hq * D * 2);
   if (it < items) {
     QueryRowRegs regs;
     qdo_fetch<D>(regs, dma, p, b, head, qb, lds0);

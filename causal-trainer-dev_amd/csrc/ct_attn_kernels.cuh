@@ -79,14 +79,14 @@ struct KvFetcher {
   const int* segb;
   size_t row_stride_bytes;
   CT_DEVICE KvFetcher(const bf16* k, const bf16* v, const int* seg, size_t row_stride_elems)
-      : kbase(reinterpret_cast<const char*>(k)), vbase(reinterpret_cast<const char*>(v)),
-        segb(seg), row_stride_bytes(row_stride_elems * 2) {}
+      : dma(row_stride_elems * 2), kbase(reinterpret_cast<const char*>(k)),
+        vbase(reinterpret_cast<const char*>(v)), segb(seg), row_stride_bytes(row_stride_elems * 2) {}
   CT_DEVICE void issue(int tile, lds_addr stage) const {
     const size_t origin = (size_t)tile * kKeyTile * row_stride_bytes;
-    dma.issue(kbase + origin, row_stride_bytes, stage + KvStage<D>::kK);
-    dma.issue(vbase + origin, row_stride_bytes, stage + KvStage<D>::kV);
+    dma.issue(kbase + origin, stage + KvStage<D>::kK);
+    dma.issue(vbase + origin, stage + KvStage<D>::kV);
     if (threadIdx.x < 16)  // 64 ids = 16 lanes x 16 bytes, linear layout
-      dma16(segb + tile * kKeyTile + threadIdx.x * 4, stage + KvStage<D>::kSeg);
+      dma16_s(segb + tile * kKeyTile, threadIdx.x * 16, stage + KvStage<D>::kSeg);
   }
 };
 
@@ -114,6 +114,13 @@ struct QueryWork {
     qt = uniform(sched[rank]);
     const int w = threadIdx.x >> 6;
     h = kvh * g + slice * HS + (w % HS);
+    rb = qt * PB + (w / HS);
+  }
+  // explicit coordinates: batch row, KV head, head slice of the group, query tile
+  CT_DEVICE QueryWork(const AttnParams& p, int b_, int kvh_, int slice, int qt_)
+      : b(b_), kvh(kvh_), qt(qt_) {
+    const int w = threadIdx.x >> 6;
+    h = kvh * (p.Hq / p.Hkv) + slice * HS + (w % HS);
     rb = qt * PB + (w / HS);
   }
 };
@@ -210,7 +217,12 @@ struct QueryTileContext {
   const bf16* kbase;
   const bf16* vbase;
   const int* segb;
-  CT_DEVICE explicit QueryTileContext(const AttnParams& p) : work(p) {
+  CT_DEVICE explicit QueryTileContext(const AttnParams& p) : work(p) { init(p); }
+  CT_DEVICE QueryTileContext(const AttnParams& p, int b, int kvh, int slice, int qt)
+      : work(p, b, kvh, slice, qt) {
+    init(p);
+  }
+  CT_DEVICE void init(const AttnParams& p) {
     const int nrb = p.S / 32;
     meta_b = p.meta + (size_t)work.b * nrb * kMetaW;
     active = work.rb < nrb;
@@ -293,18 +305,16 @@ struct VkFetcher {
   const int* segb;
   size_t row_stride_bytes;
   CT_DEVICE VkFetcher(const bf16* k, const bf16* v, const int* seg, size_t row_stride_elems)
-      : kbase(reinterpret_cast<const char*>(k)), vbase(reinterpret_cast<const char*>(v)),
-        segb(seg), row_stride_bytes(row_stride_elems * 2) {}
+      : dma(row_stride_elems * 2), kbase(reinterpret_cast<const char*>(k)),
+        vbase(reinterpret_cast<const char*>(v)), segb(seg), row_stride_bytes(row_stride_elems * 2) {}
   CT_DEVICE void issue_v(int tile, lds_addr stage) const {
-    dma.issue(vbase + (size_t)tile * kKeyTile * row_stride_bytes, row_stride_bytes,
-              stage + VkStage<D>::kV);
+    dma.issue(vbase + (size_t)tile * kKeyTile * row_stride_bytes, stage + VkStage<D>::kV);
   }
   // K rows of `tile` into `stage`, its segment ids into the ring (lds0 = start of LDS)
   CT_DEVICE void issue_k(int tile, lds_addr stage, lds_addr lds0) const {
-    dma.issue(kbase + (size_t)tile * kKeyTile * row_stride_bytes, row_stride_bytes,
-              stage + VkStage<D>::kK);
+    dma.issue(kbase + (size_t)tile * kKeyTile * row_stride_bytes, stage + VkStage<D>::kK);
     if (threadIdx.x < 16)  // 64 ids = 16 lanes x 16 bytes, linear layout
-      dma16(segb + tile * kKeyTile + threadIdx.x * 4, lds0 + VkStage<D>::seg_slot(tile));
+      dma16_s(segb + tile * kKeyTile, threadIdx.x * 16, lds0 + VkStage<D>::seg_slot(tile));
   }
   // stage s: V(s), K(s + 1); tiles past `last` are skipped
   CT_DEVICE void issue_stage(int s, int last, lds_addr stage, lds_addr lds0) const {
@@ -313,18 +323,15 @@ struct VkFetcher {
   }
 };
 
+// One query tile (kFwdWaves / HS row blocks x HS heads of one KV head), start to finish.
 template <int D, int HS>
-__global__ __launch_bounds__(kFwdWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
-attn_fwd_kernel(AttnParams p) {
-  extern __shared__ __align__(16) char smem_raw[];
-  const lds_addr lds0 = lds_address_of(smem_raw);
+CT_DEVICE void attn_fwd_item(const AttnParams& p, int b, int kvh, int slice, int qt,
+                             const lds_addr lds0, const RowFragOffsets<D / 8>& ro,
+                             const TrFragOffsets<D / 8, KSlots::kAccum>& to) {
   constexpr int kStage = VkStage<D>::kBytes;
-
-  const QueryTileContext<D, HS, kFwdWaves> ctx(p);
+  const QueryTileContext<D, HS, kFwdWaves> ctx(p, b, kvh, slice, qt);
   const int l = lane_id(), half = l >> 5, w = threadIdx.x >> 6;
   const bool late = uniform(w) >= kFwdWaves / 2;
-  const RowFragOffsets<D / 8> ro(lds0);
-  const TrFragOffsets<D / 8, KSlots::kAccum> to(lds0);
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
 
@@ -342,13 +349,14 @@ attn_fwd_kernel(AttnParams p) {
   const VkFetcher<D> fetch(ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride);
   int t = ctx.first;
   const int last = ctx.last;
-  KeyTileBounds kb = {0, 0, 0};
+  KeyTileBounds kb = {0, 0, 0}, nb = {0, 0, 0};  // bounds of tiles t and t + 1
   f32x16 s[2];
   bool visit = false;
   if (t <= last) {
     fetch.issue_k(t, lds0 + kStage, lds0);  // stage first - 1 (buffer 1): only its K half
     fetch.issue_stage(t, last, lds0, lds0);  // stage first -> buffer 0
     kb = key_tile_bounds(ctx.meta_b, t);
+    if (t + 1 <= last) nb = key_tile_bounds(ctx.meta_b, t + 1);
     visit = ctx.wave_visits(kb, t);
   }
   dma_wait_all();
@@ -362,8 +370,9 @@ attn_fwd_kernel(AttnParams p) {
     const lds_addr next_stage = lds0 + (CUR ^ 1) * kStage;
     // ---- VALU phase ----
     if (late) fetch.issue_stage(t + 1, last, next_stage, lds0);
-    KeyTileBounds nb = kb;
-    if (t + 1 <= last) nb = key_tile_bounds(ctx.meta_b, t + 1);
+    // bounds of tile t + 2: requested now, first needed one step from now
+    KeyTileBounds nnb = nb;
+    if (t + 2 <= last) nnb = key_tile_bounds(ctx.meta_b, t + 2);
     bf16x8 pf[4];
     if (visit) {
       float mx = kNegInf;
@@ -380,7 +389,7 @@ attn_fwd_kernel(AttnParams p) {
       for (int kbk = 0; kbk < 2; ++kbk)
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kbk][r]);
-      mx = fmaxf(mx, xor32(mx)) * kLog2e;
+      mx = pair_max(mx) * kLog2e;
       // The running reference m_run only follows the true maximum when that has grown by
       // more than kRescaleSlack (log2 units): probabilities are then at most 2^slack, well
       // inside bf16 / f32 range, the normalisation by the row sum is unchanged, and the
@@ -443,6 +452,7 @@ attn_fwd_kernel(AttnParams p) {
     __builtin_amdgcn_s_barrier();
     visit = visit_next;
     kb = nb;
+    nb = nnb;
     ++t;
   };
   while (t <= last) {
@@ -454,14 +464,42 @@ attn_fwd_kernel(AttnParams p) {
   dma_wait_all();
   __syncthreads();  // every wavefront is done with the stages before they become store patches
 
-  const float l_tot = l_run + xor32(l_run);
+  const float l_tot = pair_sum(l_run);
   const bool has = l_tot > 0.f;
   const float inv = has ? 1.f / l_tot : 0.f;
-  if (!ctx.active) return;
-  if (half == 0) p.lse[ctx.stat_off] = has ? (__logf(l_tot) + m_run * kLn2) : 0.f;
-  const lds_addr patch = lds0 + w * 32 * D * 2;
-  bf16* obase = p.out + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
-  store_rows_t<D>(oacc, inv, patch, obase, q_row_stride);
+  if (ctx.active) {
+    if (half == 0) p.lse[ctx.stat_off] = has ? (__logf(l_tot) + m_run * kLn2) : 0.f;
+    const lds_addr patch = lds0 + w * 32 * D * 2;
+    bf16* obase = p.out + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
+    store_rows_t<D>(oacc, inv, patch, obase, q_row_stride);
+  }
+  __syncthreads();  // the store patches overlap the stages of the next item
+}
+
+// Workgroup (group, bin): walks the query tiles of one work bin for one
+// (head slice, KV head) group. The group is the fast index, so with 8 groups a
+// group stays on one XCD (workgroup ids are dealt round robin to the 8 XCDs)
+// and its K/V rows stay in that XCD's L2.
+template <int D, int HS>
+__global__ __launch_bounds__(kFwdWaves * 64) __attribute__((amdgpu_waves_per_eu(2, 2))) void
+attn_fwd_kernel(AttnParams p) {
+  extern __shared__ __align__(16) char smem_raw[];
+  const lds_addr lds0 = lds_address_of(smem_raw);
+  constexpr int PB = kFwdWaves / HS;
+  const RowFragOffsets<D / 8> ro(lds0);
+  const TrFragOffsets<D / 8, KSlots::kAccum> to(lds0);
+  const int nrb = p.S / 32;
+  const int slices = (p.Hq / p.Hkv) / HS;
+  const int groups = slices * p.Hkv;
+  const int group = blockIdx.x % groups, bin = blockIdx.x / groups;
+  const int kvh = group % p.Hkv, slice = group / p.Hkv;
+  const MetaPtr region = meta_const(p.meta + bin_region_offset(p.B, nrb, PB));
+  const int tpr = bin_tiles_per_row(nrb, PB);
+  const int it_end = uniform(region[bin + 1]);
+  for (int it = uniform(region[bin]); it < it_end; ++it) {
+    const int item = uniform(region[kBins + 1 + it]);
+    attn_fwd_item<D, HS>(p, item / tpr, kvh, slice, item % tpr, lds0, ro, to);
+  }
 }
 
 // ---------------------------------------------------------------------------

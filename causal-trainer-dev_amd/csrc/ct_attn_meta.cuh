@@ -56,6 +56,37 @@ __host__ __device__ inline int query_schedule_offset(int nrb, int pb) {
 __host__ __device__ inline int key_schedule_offset(int nrb) { return nrb + nrb / 2 + nrb / 4; }
 
 // ---------------------------------------------------------------------------
+// Static work bins (after the schedules of the last batch row).
+//
+// A kernel that keeps one workgroup per compute unit cannot rely on the
+// hardware dispatcher for balance: workgroups are dealt to the 8 XCDs round
+// robin and in order, so one full XCD stalls the launch of every later
+// workgroup. Instead the query tiles of the whole batch (items (batch row,
+// tile), for tiles of 2, 4 and 8 row blocks) are packed once, by decreasing
+// work onto the least loaded bin, into kBins bins of near equal work; a
+// workgroup walks one bin for one (head slice, KV head) group. With 8 groups
+// per 8 XCDs that is exactly one workgroup per compute unit, no atomics and a
+// fixed assignment.
+// Layout per tile size: kBins + 1 offsets, then the items (batch row * tiles
+// per row + tile) bin after bin, heaviest first inside a bin.
+// ---------------------------------------------------------------------------
+constexpr int kBins = 32;
+__host__ __device__ inline int bin_tiles_per_row(int nrb, int pb) { return (nrb + pb - 1) / pb; }
+__host__ __device__ inline int bin_region_ints(int B, int nrb, int pb) {
+  return kBins + 1 + B * bin_tiles_per_row(nrb, pb);
+}
+// offset (ints) of the bins for tiles of pb row blocks (pb = 2, 4, 8) from the start of the table
+__host__ __device__ inline size_t bin_region_offset(int B, int nrb, int pb) {
+  size_t off = (size_t)B * ((size_t)nrb * 12 + schedule_ints(nrb));
+  if (pb >= 4) off += bin_region_ints(B, nrb, 2);
+  if (pb >= 8) off += bin_region_ints(B, nrb, 4);
+  return off;
+}
+__host__ __device__ inline size_t meta_total_ints(int B, int nrb) {
+  return bin_region_offset(B, nrb, 8) + bin_region_ints(B, nrb, 8);
+}
+
+// ---------------------------------------------------------------------------
 // dK/dV work list (backward workspace).
 //
 // A 128-key tile's work is the list of (query head of the group, visiting

@@ -66,6 +66,26 @@ CT_DEVICE float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
 CT_DEVICE float xor32(float v) { return __shfl_xor(v, 32, 64); }
 
+// Reductions over the lane pair (l, l ^ 32) without an LDS round trip:
+// v_permlane32_swap exchanges the upper half of its first operand with the
+// lower half of its second, so two copies of v become {lo, lo} and {hi, hi}.
+// Both lanes of a pair get the same bits.
+CT_DEVICE void halves_of(float v, float& lo, float& hi) {
+  lo = v;
+  hi = v;
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(lo), "+v"(hi));
+}
+CT_DEVICE float pair_max(float v) {
+  float lo, hi;
+  halves_of(v, lo, hi);
+  return fmaxf(lo, hi);
+}
+CT_DEVICE float pair_sum(float v) {
+  float lo, hi;
+  halves_of(v, lo, hi);
+  return lo + hi;
+}
+
 // ---------------------------------------------------------------------------
 // LDS access through 32-bit addresses
 // ---------------------------------------------------------------------------
@@ -94,6 +114,22 @@ CT_DEVICE void dma16(const void* src, lds_addr dst) {
   asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                :
                : "v"(src), "s"(m0_value)
+               : "memory", "m0");
+}
+// Same copy with the address split into a wave-uniform base (scalar registers) and a 32-bit
+// per-lane byte offset. With loop-invariant lane offsets a copy costs no vector ALU work and
+// no vector register is rewritten between copies (rewriting the address registers of a
+// queued copy stalls the wavefront until the copy has left the queue).
+CT_DEVICE void dma16_s(const void* uniform_base, unsigned lane_offset, lds_addr dst) {
+  const unsigned m0_value = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)dst);
+  const unsigned long long b = (unsigned long long)(uintptr_t)uniform_base;
+  // (the builtin returns a signed int: go through unsigned so that the low half is not sign extended)
+  const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
+  const unsigned long long base = ((unsigned long long)hi << 32) | (unsigned long long)lo;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(lane_offset), "s"(base), "s"(m0_value)
                : "memory", "m0");
 }
 // s_waitcnt vmcnt(0) only (expcnt / lgkmcnt fields left at "no wait")
@@ -133,19 +169,21 @@ struct TileDma {
   static constexpr int kRowsPerPass = THREADS / CPR;
   static constexpr int kPasses = ROWS / kRowsPerPass;
   static_assert(kRowsPerPass % 16 == 0 && ROWS % kRowsPerPass == 0, "unsupported tile shape");
-  int row0, chunk;  // this thread's row in pass 0 and the logical chunk it fetches
-  CT_DEVICE TileDma() {
+  unsigned lane_off[kPasses];  // byte offset of this thread's chunk in pass n from the tile origin
+  // tile row r lives at origin + r * row_stride_bytes (ROWS * row_stride_bytes < 4 GiB)
+  CT_DEVICE explicit TileDma(size_t row_stride_bytes) {
     const int t = threadIdx.x;
-    row0 = t / CPR;
-    chunk = (t % CPR) ^ swizzle<CPR>(row0);
-  }
-  // tile row r lives at src + r * row_stride_bytes; src and tile are workgroup-uniform.
-  CT_DEVICE void issue(const char* src, size_t row_stride_bytes, lds_addr tile) const {
-    const int wave = uniform(threadIdx.x >> 6);
-    const char* p = src + (size_t)row0 * row_stride_bytes + chunk * 16;
+    const int row0 = t / CPR;
+    const int chunk = (t % CPR) ^ swizzle<CPR>(row0);
 #pragma unroll
     for (int n = 0; n < kPasses; ++n)
-      dma16(p + (size_t)n * kRowsPerPass * row_stride_bytes, tile + (n * THREADS + wave * 64) * 16);
+      lane_off[n] = (unsigned)((size_t)(row0 + n * kRowsPerPass) * row_stride_bytes + chunk * 16);
+  }
+  // origin and tile are workgroup-uniform
+  CT_DEVICE void issue(const char* origin, lds_addr tile) const {
+    const int wave = uniform(threadIdx.x >> 6);
+#pragma unroll
+    for (int n = 0; n < kPasses; ++n) dma16_s(origin, lane_off[n], tile + (n * THREADS + wave * 64) * 16);
   }
 };
 

@@ -87,7 +87,7 @@ struct KcLoader {
     const int wave = uniform(threadIdx.x >> 6);
     const char* p = base + (size_t)k0 * 2;
 #pragma unroll
-    for (int n = 0; n < NCH; ++n) dma16(p + voff[n], tile + (n * 256 + wave * 64) * 16);
+    for (int n = 0; n < NCH; ++n) dma16_s(p, voff[n], tile + (n * 256 + wave * 64) * 16);
   }
   CT_DEVICE void fetch(int k0) {
     const int k = k0 + chunk * 8;
@@ -167,7 +167,7 @@ struct McLoader {
     } else {
       const char* p = base + (size_t)k0 * ld * 2;
 #pragma unroll
-      for (int n = 0; n < NCH; ++n) dma16(p + voff[n], tile + (n * 256 + wave * 64) * 16);
+      for (int n = 0; n < NCH; ++n) dma16_s(p, voff[n], tile + (n * 256 + wave * 64) * 16);
     }
   }
   CT_DEVICE void fetch(int k0) {

@@ -249,7 +249,8 @@ def test_metadata_matches_oracle_bit_exact(ct, gpu):
         # schedules: permutations, ordered by non-increasing work
         blocks = 1024 // 32
         per_row = 2 * blocks + blocks // 4
-        schedules = metadata.tile_bounds.cpu().numpy()[2 * blocks * 12:].reshape(2, per_row)
+        flat = metadata.tile_bounds.cpu().numpy()
+        schedules = flat[2 * blocks * 12:2 * blocks * 12 + 2 * per_row].reshape(2, per_row)
         for b in range(2):
             spans = np.where(bounds[b, :, 6] >= bounds[b, :, 5], bounds[b, :, 6] - bounds[b, :, 5] + 1, 0)
             order = schedules[b, :blocks]
@@ -259,6 +260,26 @@ def test_metadata_matches_oracle_bit_exact(ct, gpu):
                                   (blocks + blocks // 2 + blocks // 4, blocks // 4),
                                   (2 * blocks, (blocks + 7) // 8)):
                 assert sorted(schedules[b, offset:offset + count].tolist()) == list(range(count))
+        # work bins: every (batch row, query tile) item appears in exactly one of the 32 bins,
+        # and the bins are balanced to within the heaviest item (longest-first packing)
+        cursor = 2 * blocks * 12 + 2 * per_row
+        for tile_blocks in (2, 4, 8):
+            tiles_per_row = (blocks + tile_blocks - 1) // tile_blocks
+            items = 2 * tiles_per_row
+            offsets = flat[cursor:cursor + 33]
+            listed = flat[cursor + 33:cursor + 33 + items]
+            assert offsets[0] == 0 and offsets[32] == items and (np.diff(offsets) >= 0).all()
+            assert sorted(listed.tolist()) == list(range(items))
+            work = np.zeros(items, dtype=np.int64)
+            for item in range(items):
+                b, tile = divmod(item, tiles_per_row)
+                rows = bounds[b, tile * tile_blocks:(tile + 1) * tile_blocks]
+                first, last = rows[:, 5].min(), rows[:, 6].max()
+                work[item] = (last - first + 1 if last >= first else 0) + 3
+            loads = np.array([work[listed[offsets[j]:offsets[j + 1]]].sum() for j in range(32)])
+            assert loads.max() - loads.min() <= work.max()
+            cursor += 33 + items
+        assert cursor == flat.size
 
 
 def test_delta_pass_matches_torch(ct, gpu):

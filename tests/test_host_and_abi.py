@@ -25,7 +25,8 @@ def test_library_exports_every_declared_symbol(ct):
 def test_size_queries_need_no_gpu(ct):
     library = ct._lib.load()
     nrb = 4096 // 32
-    assert library.ct_attn_meta_bytes(4, 4096) == 4 * (nrb * 12 + 2 * nrb + nrb // 4) * 4
+    bins = sum(33 + 4 * ((nrb + pb - 1) // pb) for pb in (2, 4, 8))
+    assert library.ct_attn_meta_bytes(4, 4096) == (4 * (nrb * 12 + 2 * nrb + nrb // 4) + bins) * 4
     assert library.ct_attn_meta_bytes(0, 128) == 0
     assert 0 < library.ct_attn_bwd_workspace_bytes(4, 4096, 8, 128) < 1 << 30
     assert library.ct_attn_bwd_workspace_bytes(4, 4000, 8, 128) == 0
