@@ -24,6 +24,7 @@
 
 #include <type_traits>
 
+#include "ct_attn_asm.inc"
 #include "ct_attn_meta.cuh"
 #include "ct_common.cuh"
 
@@ -160,6 +161,34 @@ CT_DEVICE void tile_mask(lds_addr segk, int tile, int seg_q, int end_q, bool row
   }
 }
 
+// Sets the scores of disallowed (query, key) pairs of a transposed score tile to -inf.
+// The pair rule is seg_k == seg_q != 0 and key <= end_q (src/modeling/attention.py:67-97);
+// each half is only evaluated where the tile's summaries do not already prove it:
+//   SEG     the key tile or the query block mixes segment ids
+//   CAUSAL  the tile's last key lies beyond the smallest visible end of the block
+// `seg_q_or_never` is the query's id, or -1 for a padding query (ids are >= 0, so -1 never
+// matches); `last_rel` is end_q - first key of the tile - 4 * (lane / 32), which makes the
+// key offset of accumulator register r of block kb the lane-independent constant
+// 32 kb + 8 (r / 4) + r % 4.
+template <bool SEG, bool CAUSAL>
+CT_DEVICE void mask_scores_t(lds_addr segk, int seg_q_or_never, int last_rel, f32x16* s) {
+  const int half = lane_id() >> 5;
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      i32x4 sk = {0, 0, 0, 0};
+      if constexpr (SEG) sk = lds_load<i32x4>(segk + (kb * 32 + 8 * qd + 4 * half) * 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        bool ok = true;
+        if constexpr (SEG) ok = sk[e] == seg_q_or_never;
+        if constexpr (CAUSAL) ok = ok && (kb * 32 + 8 * qd + e <= last_rel);
+        s[kb][4 * qd + e] = ok ? s[kb][4 * qd + e] : kNegInf;
+      }
+    }
+}
+
 // acc (D x 32 queries, transposed) += X^T W^T where X is a 64-row LDS tile read
 // transposed and W^T are the accumulator-layout weights wt[2].
 template <int D>
@@ -258,6 +287,28 @@ struct QueryTileContext {
                             t * kKeyTile + kKeyTile - 1);
   }
 };
+
+// Hand-scheduled MFMA sequences for D = 128 (see gen_attn_asm.py). TILE_OFF is the byte
+// offset of the operand tile from the LDS base the fragment pointers were built on.
+template <int TILE_OFF>
+CT_DEVICE void pv_sequence_128(const TrFragOffsets<16, KSlots::kAccum>& to, const bf16x8* pf,
+                               f32x16* oacc) {
+  asm volatile(CT_ATTN_PV_SEQUENCE
+               : "+v"(oacc[0]), "+v"(oacc[1]), "+v"(oacc[2]), "+v"(oacc[3])
+               : "v"(to.ptr[0][0]), "v"(to.ptr[0][1]), "v"(to.ptr[0][2]), "v"(to.ptr[0][3]),
+                 "v"(to.ptr[1][0]), "v"(to.ptr[1][1]), "v"(to.ptr[1][2]), "v"(to.ptr[1][3]),
+                 "v"(pf[0]), "v"(pf[1]), "v"(pf[2]), "v"(pf[3]), "i"(TILE_OFF)
+               : "memory", CT_ATTN_ASM_SCRATCH);
+}
+template <int TILE_OFF>
+CT_DEVICE void qk_sequence_128(const RowFragOffsets<16>& ro, const bf16x8* qf, f32x16* s) {
+  asm volatile(CT_ATTN_QK_SEQUENCE
+               : "=&v"(s[0]), "=&v"(s[1])
+               : "v"(ro.ptr[0]), "v"(ro.ptr[1]), "v"(ro.ptr[2]), "v"(ro.ptr[3]), "v"(ro.ptr[4]),
+                 "v"(ro.ptr[5]), "v"(ro.ptr[6]), "v"(ro.ptr[7]), "v"(qf[0]), "v"(qf[1]), "v"(qf[2]),
+                 "v"(qf[3]), "v"(qf[4]), "v"(qf[5]), "v"(qf[6]), "v"(qf[7]), "i"(TILE_OFF)
+               : "memory", CT_ATTN_ASM_SCRATCH);
+}
 
 // ---------------------------------------------------------------------------
 // Forward
@@ -376,14 +427,24 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, int b, int kvh, int slice, int
     bf16x8 pf[4];
     if (visit) {
       float mx = kNegInf;
-      if (!ctx.interior(kb, t)) {
-        unsigned allow[2];
-        tile_mask(lds0 + VkStage<D>::seg_slot(t), t, ctx.seg_q, ctx.end_q, ctx.row_valid, allow);
-#pragma unroll
-        for (int kbk = 0; kbk < 2; ++kbk)
-#pragma unroll
-          for (int r = 0; r < 16; ++r)
-            s[kbk][r] = ((allow[kbk] >> r) & 1u) ? s[kbk][r] : kNegInf;
+      {
+        // What the summaries leave open for this tile. A key tile with one shared id X turns
+        // the id test into a per-query predicate (seg_q == X), which folds into the visible-end
+        // bound; only a key tile that mixes ids needs the per-key comparison.
+        const int k_uniform = uniform(kb.uniform);
+        const bool mixed_keys = k_uniform == 0;
+        const bool need_seg = ctx.mine.uniform == 0 || ctx.mine.uniform != k_uniform;
+        const bool need_causal = t * kKeyTile + kKeyTile - 1 > ctx.mine.end_min;
+        if (need_seg || need_causal) {
+          const int seg_cmp = ctx.row_valid ? ctx.seg_q : -1;
+          int last_rel = ctx.end_q - t * kKeyTile - 4 * half;
+          if (mixed_keys) {
+            mask_scores_t<true, true>(lds0 + VkStage<D>::seg_slot(t), seg_cmp, last_rel, s);
+          } else {
+            if (seg_cmp != k_uniform) last_rel = -1;  // no key of this tile is visible
+            mask_scores_t<false, true>(lds0, seg_cmp, last_rel, s);
+          }
+        }
       }
 #pragma unroll
       for (int kbk = 0; kbk < 2; ++kbk)
@@ -422,31 +483,19 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, int b, int kvh, int slice, int
     __builtin_amdgcn_s_barrier();
     // ---- MFMA phase ----
     if (!late) fetch.issue_stage(t + 1, last, next_stage, lds0);
-    if (visit) {
-#pragma unroll
-      for (int step4 = 0; step4 < 4; ++step4)
-#pragma unroll
-        for (int db = 0; db < D / 32; ++db)
-          oacc[db] = mfma32(to.load(CUR * kStage + VkStage<D>::kV, step4, db), pf[step4], oacc[db]);
-      // LDS fragment reads run kAhead fragments ahead of the MFMA that consumes them.
-      constexpr int kMfma = 4 * (D / 32), kAhead = 4;
-      __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);
-#pragma unroll
-      for (int i = 0; i < kMfma; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (i + kAhead < kMfma) __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      }
-    }
     const bool visit_next = (t + 1 <= last) && ctx.wave_visits(nb, t + 1);
-    if (visit_next) {
-      scores_t<D>(CUR * kStage + VkStage<D>::kK, ro, qf, s);
-      constexpr int kMfma = 2 * (D / 16), kAhead = 6;
-      __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+    if constexpr (D == 128) {
+      if (visit) pv_sequence_128<CUR * kStage + VkStage<D>::kV>(to, pf, oacc);
+      if (visit_next) qk_sequence_128<CUR * kStage + VkStage<D>::kK>(ro, qf, s);
+    } else {
+      if (visit) {
 #pragma unroll
-      for (int i = 0; i < kMfma; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        if (i + kAhead < kMfma) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        for (int step4 = 0; step4 < 4; ++step4)
+#pragma unroll
+          for (int db = 0; db < D / 32; ++db)
+            oacc[db] = mfma32(to.load(CUR * kStage + VkStage<D>::kV, step4, db), pf[step4], oacc[db]);
       }
+      if (visit_next) scores_t<D>(CUR * kStage + VkStage<D>::kK, ro, qf, s);
     }
     if (late) dma_wait_all();  // stage t + 1, issued at the start of this step
     __builtin_amdgcn_s_barrier();
@@ -473,7 +522,10 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, int b, int kvh, int slice, int
     bf16* obase = p.out + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
     store_rows_t<D>(oacc, inv, patch, obase, q_row_stride);
   }
-  __syncthreads();  // the store patches overlap the stages of the next item
+  // The store patches overlap the stages of the next item: its copies may start once every
+  // wavefront has read its patch back (LDS reads only; the global stores stay in flight).
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
 }
 
 // Workgroup (group, bin): walks the query tiles of one work bin for one
