@@ -35,6 +35,8 @@ def parse_args():
     parser.add_argument("--cutce-steps", type=int, default=None, help="default: min(steps, 5)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-cutce", action="store_true")
+    parser.add_argument("--cutce-recompute", action="store_true",
+                        help="cut-CE without the logits cache (backward recomputes the projection)")
     return parser.parse_args()
 
 
@@ -94,7 +96,7 @@ def bench_attention(ct, torch, steps, warmup):
     }
 
 
-def bench_cutce(ct, torch, steps, warmup):
+def bench_cutce(ct, torch, steps, warmup, logits_cache=True):
     W = ct.workloads
     config = W.CUTCE_CONFIGS["llama3_8b_head"]
     inputs = W.make_cutce_inputs(config, "cuda")
@@ -104,10 +106,18 @@ def bench_cutce(ct, torch, steps, warmup):
     dy = torch.tensor(1.0 / max(active, 1))
 
     state = {}
+    # The f32 logits cache the forward lends to the backward (the operator's default when it
+    # fits; owned by the caller, so it is allocated once like every other buffer here).
+    cache = None
+    if logits_cache:
+        cache = torch.empty(ct.cut_cross_entropy.logits_cache_bytes(config.rows, config.hidden, config.vocab),
+                            dtype=torch.uint8, device="cuda")
 
     def step():
-        nll, weight_sum, lse = ct.cutce_forward(hidden, head, targets, weights, sparse_compaction=True)
-        ct.cutce_backward(hidden, head, targets, weights, lse, dy, sparse_compaction=True)
+        nll, weight_sum, lse = ct.cutce_forward(hidden, head, targets, weights, sparse_compaction=True,
+                                                logits_cache=cache)
+        ct.cutce_backward(hidden, head, targets, weights, lse, dy, sparse_compaction=True,
+                          logits_cache=cache)
         state["loss"] = (nll, weight_sum)
 
     elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
@@ -123,6 +133,8 @@ def bench_cutce(ct, torch, steps, warmup):
     nll, weight_sum = state["loss"]
     return {
         "workload": "cut-CE fwd+bwd N=16384 d=4096 V=128256 bf16, 30% ignored, head [d, V], compaction on",
+        "logits_cache": bool(logits_cache),
+        "logits_cache_bytes": 0 if cache is None else cache.numel(),
         "active_rows": active,
         "ms_per_step": ms_per_step,
         "tokens_per_s": config.rows / (ms_per_step * 1e-3),
@@ -237,7 +249,8 @@ def main():
         }
     if not args.no_cutce:
         cut_steps = args.cutce_steps or min(args.steps, 5)
-        result["cutce"] = bench_cutce(ct, torch, cut_steps, min(args.warmup, 2))
+        result["cutce"] = bench_cutce(ct, torch, cut_steps, min(args.warmup, 2),
+                                      logits_cache=not args.cutce_recompute)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(ct, torch, attention)
     print(json.dumps(result))

@@ -20,7 +20,7 @@ CT_WORKSPACE_TOO_SMALL = -3
 CT_LAUNCH_FAILED = -4
 
 ATTN_META_WIDTH = 12
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 
 class CtError(RuntimeError):
@@ -64,6 +64,7 @@ class CutceFwdArgs(Structure):
         ("nll_sum", c_void_p), ("weight_sum", c_void_p), ("lse", c_void_p),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("shape", CutceShape), ("sparse_compaction", c_int32),
+        ("logits_cache", c_void_p), ("logits_cache_bytes", c_size_t),
     ]
 
 
@@ -73,6 +74,7 @@ class CutceBwdArgs(Structure):
         ("lse", c_void_p), ("dy", c_void_p), ("dhidden", c_void_p), ("dhead", c_void_p),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("shape", CutceShape), ("sparse_compaction", c_int32),
+        ("logits_cache", c_void_p), ("logits_cache_bytes", c_size_t),
     ]
 
 
@@ -94,6 +96,7 @@ SYMBOLS = {
     "ct_cutce_fwd_workspace_bytes": (c_size_t, [POINTER(CutceShape)]),
     "ct_cutce_bwd_workspace_min_bytes": (c_size_t, [POINTER(CutceShape)]),
     "ct_cutce_bwd_workspace_bytes": (c_size_t, [POINTER(CutceShape)]),
+    "ct_cutce_logits_cache_bytes": (c_size_t, [POINTER(CutceShape)]),
     "ct_cutce_fwd": (c_int32, [c_void_p, POINTER(CutceFwdArgs)]),
     "ct_cutce_bwd": (c_int32, [c_void_p, POINTER(CutceBwdArgs)]),
 }

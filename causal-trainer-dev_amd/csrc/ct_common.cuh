@@ -261,6 +261,18 @@ CT_DEVICE bf16x8 pack_acc8(const f32x16& c, int t) {
 CT_DEVICE u32x4 load_global16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
 CT_DEVICE void store_global16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 
+// 4-byte store to uniform_base + lane_offset + IMM bytes (scalar base, 32-bit lane offset): no
+// per-store vector address arithmetic.
+template <int IMM>
+CT_DEVICE void store_global4_s(void* uniform_base, unsigned lane_offset, float value) {
+  static_assert(IMM >= 0 && IMM < 4096, "immediate offset out of range");
+  const unsigned long long b = (unsigned long long)(uintptr_t)uniform_base;
+  const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
+  const unsigned long long base = ((unsigned long long)hi << 32) | (unsigned long long)lo;
+  asm volatile("global_store_dword %0, %1, %2 offset:%3" : : "v"(lane_offset), "v"(value), "s"(base), "n"(IMM) : "memory");
+}
+
 CT_DEVICE bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 CT_DEVICE u32x4 as_u32x4(bf16x8 v) { return __builtin_bit_cast(u32x4, v); }
 

@@ -9,14 +9,18 @@
 //   finalize fixed-order sum of the block sums -> nll_sum, weight_sum
 // Backward:
 //   dlogits  G = w * dy * (exp(logits - lse) - onehot), rounded to bf16, written
-//            to a workspace slab [rows, vocab slab]
-//   dhidden  dHidden = G head^T            (k-contiguous x k-contiguous GEMM)
-//   dhead    dHead   = hidden^T G          (both operands read transposed)
+//            vocabulary-major to a workspace slab G^T [vocab slab, rows]
+//   dhidden  dHidden = G head^T
+//   dhead    dHead   = hidden^T G
 // The reference recomputes the logits in both backward kernels
-// (src/kernels/cut_cross_entropy.py:258, :383); here they are recomputed once
-// and the bf16 G slab is shared, which keeps the reference's rounding points
-// (G is cast to bf16 before both products, :272, :396) and needs 4 GEMMs
-// instead of 5.
+// (src/kernels/cut_cross_entropy.py:258, :383); here G is formed once and shared,
+// which keeps the reference's rounding points (G is cast to bf16 before both
+// products, :272, :396). Its logits come either from a second GEMM (4 GEMMs
+// instead of the reference's 5) or, when the caller lends the forward a cache,
+// from the f32 logits the forward left there (3 GEMMs, the algorithmic count).
+// The cache is vocabulary-major [vocab, rows] like G^T: in the transposed tile
+// the GEMMs produce, the lanes of a wavefront run along the rows, so both are
+// written with contiguous stores.
 #include "ct_error.h"
 #include "ct_gemm.cuh"
 
@@ -95,7 +99,9 @@ CT_DEVICE void merge_stats(float& m, float& s, float m_o, float s_o) {
   m = m_new;
 }
 
-__global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* part, int chunks) {
+template <bool CACHE>
+__global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* part, int chunks,
+                                                          float* cache) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr smem = lds_address_of(smem_raw);
   __shared__ int unit_s;
@@ -144,6 +150,23 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
 
       const int vbase = v0 + wm + 4 * half;  // vocab id of (i, r) = vbase + 32 i + 8 (r/4) + r%4
       const bool ragged = v0 + kGemmTile > p.V;
+      if constexpr (CACHE) {
+        // cache^T[v][slot]: 32 lanes = 32 consecutive slots, 128 contiguous bytes per store.
+        // Address = wave-uniform tile origin + uniform (row, column block) offset + a 32-bit
+        // lane offset, so the stores need no per-store vector address arithmetic.
+        float* origin = cache + (size_t)(v0 + uniform(wm)) * p.n_pad + n0 + uniform(wn);
+        const unsigned lane_off = (unsigned)(4 * half * p.n_pad + j) * 4u;  // bytes
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float* row = origin + (size_t)(32 * i + 8 * (r >> 2) + (r & 3)) * p.n_pad;
+            store_global4_s<0>(row, lane_off, acc.c[i][0][r]);
+            store_global4_s<128>(row, lane_off, acc.c[i][1][r]);
+            store_global4_s<256>(row, lane_off, acc.c[i][2][r]);
+            store_global4_s<384>(row, lane_off, acc.c[i][3][r]);
+          }
+      }
 #pragma unroll
       for (int nb = 0; nb < 4; ++nb) {
         float tmax = kNegInfF;
@@ -277,15 +300,43 @@ __global__ __launch_bounds__(256) void cutce_zero_rows_kernel(const float* weigh
   for (int c = threadIdx.x; c < d / 8; c += 256) dst[c] = u32x4{0u, 0u, 0u, 0u};
 }
 
-// G[slot, v - slab0] for one 256 x 256 tile.
-__global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, const float* lse,
-                                                            const float* dy, int slab0,
-                                                            int slab_tiles, bf16* G, int ldg) {
+// Per-slot constants of the backward: (w dy, lse log2 e, target), zeros / -1 past the active rows.
+struct CutceRowParams {
+  float* fac;
+  float* lse2;
+  int* tgt;
+};
+
+__global__ __launch_bounds__(256) void cutce_rowparams_kernel(CutceParams p, const float* lse,
+                                                              const float* dy, CutceRowParams rp) {
+  const int slot = blockIdx.x * 256 + threadIdx.x;
+  if (slot >= p.n_pad) return;
+  float f = 0.f, l2 = 0.f;
+  int t = -1;
+  if (slot < p.header->n_act) {
+    const int row = p.idx[slot];
+    const float wr = p.weights[row];
+    if (wr != 0.f) {
+      f = wr * dy[0];
+      l2 = lse[row] * kLog2e;
+      t = p.targets[row];
+    }
+  }
+  rp.fac[slot] = f;
+  rp.lse2[slot] = l2;
+  rp.tgt[slot] = t;
+}
+
+CT_DEVICE float dlogit(float logit, float fac, float lse2, int tgt, int v) {
+  return fac * (exp2_fast(logit * kLog2e - lse2) - (v == tgt ? 1.f : 0.f));
+}
+
+// G^T[v - slab0][slot] for one 256 x 256 tile, logits recomputed (transposed tile as in the
+// statistics kernel: rows = vocabulary, lanes = row slots).
+__global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, CutceRowParams rp,
+                                                            int slab0, int slab_tiles, bf16* G) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr smem = lds_address_of(smem_raw);
-  __shared__ float lse2_s[kGemmTile];
-  __shared__ float fac_s[kGemmTile];
-  __shared__ int tgt_s[kGemmTile];
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
   const int row_blocks = p.n_pad / kGemmTile;
@@ -293,64 +344,76 @@ __global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, const
   const int rb = id % row_blocks, vt = id / row_blocks;
   const int n0 = rb * kGemmTile;
   const int n_act = p.header->n_act;
-  if (n0 >= n_act) return;  // G rows past the active count are never read
+  if (n0 >= n_act) return;  // G^T columns past the active count's block are never read
   const int v0 = slab0 + vt * kGemmTile;
 
-  {
-    const int slot = n0 + tid;
-    float f = 0.f, l2 = 0.f;
-    int t = -1;
-    if (slot < n_act) {
-      const int row = p.idx[slot];
-      const float wr = p.weights[row];
-      if (wr != 0.f) {
-        f = wr * dy[0];
-        l2 = lse[row] * kLog2e;
-        t = p.targets[row];
-      }
-    }
-    fac_s[tid] = f;
-    lse2_s[tid] = l2;
-    tgt_s[tid] = t;
-  }
-  KcLoader A;
-  A.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true);
-  McLoader B;
-  B.init(p.head, p.V, nullptr, v0, p.V, p.d, p.head_aligned);
+  McLoader A;
+  A.init(p.head, p.V, nullptr, v0, p.V, p.d, p.head_aligned);
+  KcLoader B;
+  B.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true);
   GemmAcc acc;
   acc.clear();
-  gemm_tile(A, B, 0, p.d, smem, acc);  // barriers inside also publish the row arrays
+  gemm_tile(A, B, 0, p.d, smem, acc);
 
+  float fac[4], lse2[4];
+  int tgt[4];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int nb = 0; nb < 4; ++nb) {
+    const int slot = n0 + wn + 32 * nb + j;
+    fac[nb] = rp.fac[slot];
+    lse2[nb] = rp.lse2[slot];
+    tgt[nb] = rp.tgt[slot];
+  }
+  bf16* gbase = G + (size_t)(v0 - slab0 + wm + 4 * half) * p.n_pad + n0 + wn + j;
 #pragma unroll
-    for (int qd = 0; qd < 4; ++qd) {
-      const int r0 = wm + 32 * i + 8 * qd + 4 * half;
-      const f32x4 l4 = *reinterpret_cast<const f32x4*>(lse2_s + r0);
-      const f32x4 f4 = *reinterpret_cast<const f32x4*>(fac_s + r0);
-      const int4 t4 = *reinterpret_cast<const int4*>(tgt_s + r0);
-      const int tg[4] = {t4.x, t4.y, t4.z, t4.w};
+  for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        bf16* grow = G + (size_t)(n0 + r0 + e) * ldg + (v0 - slab0);
+    for (int r = 0; r < 16; ++r) {
+      const int vrel = 32 * i + 8 * (r >> 2) + (r & 3);
+      const int v = v0 + wm + 4 * half + vrel;
+      bf16* dst = gbase + (size_t)vrel * p.n_pad;
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-          const int col = wn + 32 * nb + j;
-          const int v = v0 + col;
-          float g = 0.f;
-          if (f4[e] != 0.f && v < p.V) {
-            const float prob = exp2_fast(acc.c[i][nb][4 * qd + e] * kLog2e - l4[e]);
-            g = f4[e] * (prob - (v == tg[e] ? 1.f : 0.f));
-          }
-          grow[col] = (bf16)g;
-        }
+      for (int nb = 0; nb < 4; ++nb) {
+        const float g = (fac[nb] != 0.f && v < p.V) ? dlogit(acc.c[i][nb][r], fac[nb], lse2[nb], tgt[nb], v) : 0.f;
+        dst[32 * nb] = (bf16)g;
       }
     }
-  }
 }
 
-// dHidden[idx[slot], n] (+)= sum_v G[slot, v] head[n, slab0 + v]
-__global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const bf16* G, int ldg,
+// Same G^T from the f32 logits the forward left in its cache: one pass over memory, 8 slots
+// per thread. grid = (slab rows, ceil(n_pad / 2048)).
+__global__ __launch_bounds__(256) void cutce_dlogits_cached_kernel(CutceParams p, CutceRowParams rp,
+                                                                   const float* cache, int slab0,
+                                                                   bf16* G) {
+  const int vrel = blockIdx.x, v = slab0 + vrel;
+  const int slot0 = (blockIdx.y * 256 + threadIdx.x) * 8;
+  const int n_act = p.header->n_act;
+  if (slot0 >= (n_act + kGemmTile - 1) / kGemmTile * kGemmTile) return;
+  bf16x8 out;
+  if (v < p.V) {
+    const float* src = cache + (size_t)v * p.n_pad + slot0;
+    const f32x4 a = *reinterpret_cast<const f32x4*>(src);
+    const f32x4 b = *reinterpret_cast<const f32x4*>(src + 4);
+    const f32x4 f0 = *reinterpret_cast<const f32x4*>(rp.fac + slot0);
+    const f32x4 f1 = *reinterpret_cast<const f32x4*>(rp.fac + slot0 + 4);
+    const f32x4 l0 = *reinterpret_cast<const f32x4*>(rp.lse2 + slot0);
+    const f32x4 l1 = *reinterpret_cast<const f32x4*>(rp.lse2 + slot0 + 4);
+    const i32x4 t0 = *reinterpret_cast<const i32x4*>(rp.tgt + slot0);
+    const i32x4 t1 = *reinterpret_cast<const i32x4*>(rp.tgt + slot0 + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      out[e] = (bf16)(f0[e] != 0.f ? dlogit(a[e], f0[e], l0[e], t0[e], v) : 0.f);
+      out[4 + e] = (bf16)(f1[e] != 0.f ? dlogit(b[e], f1[e], l1[e], t1[e], v) : 0.f);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = (bf16)0.f;
+  }
+  store_global16(G + (size_t)vrel * p.n_pad + slot0, as_u32x4(out));
+}
+
+// dHidden[idx[slot], n] (+)= sum_v G^T[v, slot] head[n, slab0 + v]
+__global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const bf16* G,
                                                             int slab0, int slab_width, int mode,
                                                             float* dh_acc, bf16* dhidden) {
   // mode: 0 = single slab (store bf16), 1 = first slab (store f32), 2 = middle
@@ -366,8 +429,8 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
   const int n_act = p.header->n_act;
   if (n0 >= n_act) return;
 
-  KcLoader A;
-  A.init(G, ldg, nullptr, n0, p.n_pad, slab_width, true, false);
+  McLoader A;
+  A.init(G, p.n_pad, nullptr, n0, p.n_pad, slab_width, true);
   KcLoader B;
   B.init(p.head + slab0, p.V, nullptr, c0, p.d, min(slab_width, p.V - slab0), p.head_aligned, false);
   GemmAcc acc;
@@ -394,9 +457,9 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
     }
 }
 
-// dHead[m, slab0 + v] = sum_slot hidden[idx[slot], m] G[slot, v]
-__global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const bf16* G, int ldg,
-                                                          int slab0, int slab_tiles, bf16* dhead) {
+// dHead[m, slab0 + v] = sum_slot hidden[idx[slot], m] G^T[v, slot]
+__global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const bf16* G, int slab0,
+                                                          int slab_tiles, bf16* dhead) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr smem = lds_address_of(smem_raw);
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
@@ -409,11 +472,11 @@ __global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const b
   const int k_end = min(p.n_pad, (n_act + kBK - 1) / kBK * kBK);
 
   McLoader A;
-  // Rows n_act .. k_end-1 are valid memory: G holds zeros there (written by the
-  // dlogits kernel for the whole 256-row block) and idx repeats the first active row.
+  // Slots n_act .. k_end-1 are valid memory: G^T holds zeros there (the dlogits kernels
+  // write whole 256-slot blocks) and idx repeats the first active row.
   A.init(p.hidden, p.d, p.idx, m0, p.d, k_end, p.hidden_aligned);
-  McLoader B;
-  B.init(G, ldg, nullptr, v0, ldg, k_end, true);
+  KcLoader B;
+  B.init(G, p.n_pad, nullptr, v0, slab_tiles * kGemmTile, k_end, true, false);
   GemmAcc acc;
   acc.clear();
   gemm_tile(A, B, 0, k_end, smem, acc);
@@ -458,12 +521,12 @@ static FwdLayout fwd_layout(const ct_cutce_shape& s) {
 }
 
 struct BwdLayout {
-  size_t header, idx, g, acc, total;
+  size_t header, idx, rowparams, g, acc, total;
   int slab_cols;  // multiple of 256
   int slabs;
 };
 static size_t bwd_fixed_bytes(int n_pad) {
-  return align_up(sizeof(CutceHeader), 256) + align_up((size_t)n_pad * sizeof(int), 256);
+  return align_up(sizeof(CutceHeader), 256) + 4 * align_up((size_t)n_pad * sizeof(int), 256);
 }
 // Largest slab that fits in `bytes` (0 if even one tile column does not).
 static BwdLayout bwd_layout(const ct_cutce_shape& s, size_t bytes) {
@@ -472,6 +535,7 @@ static BwdLayout bwd_layout(const ct_cutce_shape& s, size_t bytes) {
   BwdLayout L = {};
   L.header = 0;
   L.idx = align_up(sizeof(CutceHeader), 256);
+  L.rowparams = L.idx + align_up((size_t)n_pad * sizeof(int), 256);
   L.g = bwd_fixed_bytes(n_pad);
   const size_t per_tile = (size_t)n_pad * kGemmTile * sizeof(bf16);
   const size_t acc_bytes = align_up((size_t)n_pad * s.hidden * sizeof(float), 256);
@@ -525,6 +589,11 @@ extern "C" size_t ct_cutce_fwd_workspace_bytes(const ct_cutce_shape* shape) {
   return fwd_layout(*shape).total;
 }
 
+extern "C" size_t ct_cutce_logits_cache_bytes(const ct_cutce_shape* shape) {
+  if (!shape || shape->rows <= 0 || shape->vocab <= 0) return 0;
+  return (size_t)padded_rows(shape->rows) * vocab_tile_count(shape->vocab) * kGemmTile * sizeof(float);
+}
+
 extern "C" size_t ct_cutce_bwd_workspace_bytes(const ct_cutce_shape* shape) {
   if (!shape || shape->rows <= 0 || shape->vocab <= 0) return 0;
   const int n_pad = padded_rows(shape->rows);
@@ -570,6 +639,12 @@ extern "C" int32_t ct_cutce_fwd(void* stream_, const ct_cutce_fwd_args* a) {
     return fail(CT_WORKSPACE_TOO_SMALL, "ct_cutce_fwd: workspace %zu < %zu bytes",
                 a->workspace_bytes, L.total);
   CT_REQUIRE(is_aligned16(a->workspace), "ct_cutce_fwd: workspace must be 16-byte aligned");
+  if (a->logits_cache) {
+    CT_REQUIRE(is_aligned16(a->logits_cache), "ct_cutce_fwd: logits cache must be 16-byte aligned");
+    if (a->logits_cache_bytes < ct_cutce_logits_cache_bytes(&a->shape))
+      return fail(CT_WORKSPACE_TOO_SMALL, "ct_cutce_fwd: logits cache %zu < %zu bytes",
+                  a->logits_cache_bytes, ct_cutce_logits_cache_bytes(&a->shape));
+  }
   hipStream_t stream = (hipStream_t)stream_;
   char* ws = static_cast<char*>(a->workspace);
   CutceParams p = make_params(a->hidden, a->head, a->targets, a->weights, a->shape, ws);
@@ -584,10 +659,16 @@ extern "C" int32_t ct_cutce_fwd(void* stream_, const ct_cutce_fwd_args* a) {
   if ((rc = scope1.done())) return rc;
 
   const size_t smem = GemmSmem::kBytes;
-  if ((rc = set_smem(cutce_stats_kernel, smem, "ct_cutce_fwd"))) return rc;
+  if ((rc = set_smem(cutce_stats_kernel<false>, smem, "ct_cutce_fwd"))) return rc;
+  if ((rc = set_smem(cutce_stats_kernel<true>, smem, "ct_cutce_fwd"))) return rc;
   const int persistent = min(device_cu_count(), chunks * row_blocks);
   LaunchScope scope2("cutce_stats_kernel", stream);
-  hipLaunchKernelGGL(cutce_stats_kernel, dim3(persistent), dim3(256), smem, stream, p, part, chunks);
+  if (a->logits_cache)
+    hipLaunchKernelGGL(cutce_stats_kernel<true>, dim3(persistent), dim3(256), smem, stream, p, part,
+                       chunks, static_cast<float*>(a->logits_cache));
+  else
+    hipLaunchKernelGGL(cutce_stats_kernel<false>, dim3(persistent), dim3(256), smem, stream, p, part,
+                       chunks, static_cast<float*>(nullptr));
   if ((rc = scope2.done())) return rc;
 
   LaunchScope scope3("cutce_merge_kernel", stream);
@@ -620,8 +701,19 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
   float* dh_acc = L.slabs > 1 ? reinterpret_cast<float*>(ws + L.acc) : nullptr;
   bf16* dhidden = reinterpret_cast<bf16*>(a->dhidden);
   bf16* dhead = reinterpret_cast<bf16*>(a->dhead);
+  const float* cache = static_cast<const float*>(a->logits_cache);
+  if (cache) {
+    CT_REQUIRE(is_aligned16(cache), "ct_cutce_bwd: logits cache must be 16-byte aligned");
+    if (a->logits_cache_bytes < ct_cutce_logits_cache_bytes(&a->shape))
+      return fail(CT_WORKSPACE_TOO_SMALL, "ct_cutce_bwd: logits cache %zu < %zu bytes",
+                  a->logits_cache_bytes, ct_cutce_logits_cache_bytes(&a->shape));
+  }
   const int row_blocks = p.n_pad / kGemmTile;
-  const int ldg = L.slab_cols;
+  const size_t params_stride = align_up((size_t)p.n_pad * sizeof(int), 256);
+  CutceRowParams rp;
+  rp.fac = reinterpret_cast<float*>(ws + L.rowparams);
+  rp.lse2 = reinterpret_cast<float*>(ws + L.rowparams + params_stride);
+  rp.tgt = reinterpret_cast<int*>(ws + L.rowparams + 2 * params_stride);
   const size_t smem = GemmSmem::kBytes;
   if ((rc = set_smem(cutce_dlogits_kernel, smem, "ct_cutce_bwd"))) return rc;
   if ((rc = set_smem(cutce_dhidden_kernel, smem, "ct_cutce_bwd"))) return rc;
@@ -635,6 +727,10 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
   hipLaunchKernelGGL(cutce_zero_rows_kernel, dim3(p.N), dim3(256), 0, stream, p.weights, p.N, p.d,
                      dhidden);
   if ((rc = scope6.done())) return rc;
+  LaunchScope scope10("cutce_rowparams_kernel", stream);
+  hipLaunchKernelGGL(cutce_rowparams_kernel, dim3(row_blocks), dim3(256), 0, stream, p, a->lse, a->dy,
+                     rp);
+  if ((rc = scope10.done())) return rc;
 
   const int tiles = vocab_tile_count(p.V);
   const int tiles_per_slab = L.slab_cols / kGemmTile;
@@ -642,19 +738,26 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
     const int slab0 = s * L.slab_cols;
     const int slab_tiles = min(tiles_per_slab, tiles - s * tiles_per_slab);
     const int slab_width = slab_tiles * kGemmTile;
-    LaunchScope scope7("cutce_dlogits_kernel", stream);
-    hipLaunchKernelGGL(cutce_dlogits_kernel, dim3(slab_tiles * row_blocks), dim3(256), smem, stream,
-                       p, a->lse, a->dy, slab0, slab_tiles, G, ldg);
-    if ((rc = scope7.done())) return rc;
+    if (cache) {
+      LaunchScope scope11("cutce_dlogits_cached_kernel", stream);
+      hipLaunchKernelGGL(cutce_dlogits_cached_kernel, dim3(slab_width, (p.n_pad + 2047) / 2048),
+                         dim3(256), 0, stream, p, rp, cache, slab0, G);
+      if ((rc = scope11.done())) return rc;
+    } else {
+      LaunchScope scope7("cutce_dlogits_kernel", stream);
+      hipLaunchKernelGGL(cutce_dlogits_kernel, dim3(slab_tiles * row_blocks), dim3(256), smem, stream,
+                         p, rp, slab0, slab_tiles, G);
+      if ((rc = scope7.done())) return rc;
+    }
     const int mode = L.slabs == 1 ? 0 : (s == 0 ? 1 : (s == L.slabs - 1 ? 3 : 2));
     LaunchScope scope8("cutce_dhidden_kernel", stream);
     hipLaunchKernelGGL(cutce_dhidden_kernel, dim3(row_blocks * ((p.d + kGemmTile - 1) / kGemmTile)), dim3(256), smem,
-                       stream, p, G, ldg, slab0, slab_width, mode, dh_acc, dhidden);
+                       stream, p, G, slab0, slab_width, mode, dh_acc, dhidden);
     if ((rc = scope8.done())) return rc;
     if (dhead) {
       LaunchScope scope9("cutce_dhead_kernel", stream);
       hipLaunchKernelGGL(cutce_dhead_kernel, dim3(((p.d + kGemmTile - 1) / kGemmTile) * slab_tiles), dim3(256), smem,
-                         stream, p, G, ldg, slab0, slab_tiles, dhead);
+                         stream, p, G, slab0, slab_tiles, dhead);
       if ((rc = scope9.done())) return rc;
     }
   }

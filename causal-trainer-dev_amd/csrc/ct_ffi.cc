@@ -121,7 +121,7 @@ ffi::Error CutceFwd(hipStream_t stream, ffi::Buffer<ffi::BF16> hidden, ffi::Buff
                     ffi::Buffer<ffi::S32> targets, ffi::Buffer<ffi::F32> weights,
                     ffi::ResultBuffer<ffi::F32> nll_sum, ffi::ResultBuffer<ffi::F32> weight_sum,
                     ffi::ResultBuffer<ffi::F32> lse, ffi::ResultBuffer<ffi::U8> workspace,
-                    bool sparse_compaction) {
+                    ffi::ResultBuffer<ffi::U8> logits_cache, bool sparse_compaction) {
   if (hidden.dimensions().size() != 2 || head.dimensions().size() != 2)
     return ffi::Error::InvalidArgument("hidden must be [rows, hidden] and head [hidden, vocab]");
   ct_cutce_fwd_args a = {};
@@ -136,13 +136,18 @@ ffi::Error CutceFwd(hipStream_t stream, ffi::Buffer<ffi::BF16> hidden, ffi::Buff
   a.workspace_bytes = workspace->size_bytes();
   a.shape = cut_shape(hidden, head);
   a.sparse_compaction = sparse_compaction ? 1 : 0;
+  // a cache result shorter than one tile means "no cache" (XLA has no optional results)
+  if (logits_cache->size_bytes() >= 256 * 256 * sizeof(float)) {
+    a.logits_cache = logits_cache->untyped_data();
+    a.logits_cache_bytes = logits_cache->size_bytes();
+  }
   return status_to_error(ct_cutce_fwd(stream, &a));
 }
 
 ffi::Error CutceBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> hidden, ffi::Buffer<ffi::BF16> head,
                     ffi::Buffer<ffi::S32> targets, ffi::Buffer<ffi::F32> weights,
                     ffi::Buffer<ffi::F32> lse, ffi::Buffer<ffi::F32> dy,
-                    ffi::ResultBuffer<ffi::BF16> dhidden, ffi::ResultBuffer<ffi::BF16> dhead,
+                    ffi::Buffer<ffi::U8> logits_cache, ffi::ResultBuffer<ffi::BF16> dhidden, ffi::ResultBuffer<ffi::BF16> dhead,
                     ffi::ResultBuffer<ffi::U8> workspace, bool sparse_compaction,
                     bool head_trainable) {
   if (hidden.dimensions().size() != 2 || head.dimensions().size() != 2)
@@ -160,6 +165,10 @@ ffi::Error CutceBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> hidden, ffi::Buff
   a.workspace_bytes = workspace->size_bytes();
   a.shape = cut_shape(hidden, head);
   a.sparse_compaction = sparse_compaction ? 1 : 0;
+  if (logits_cache.size_bytes() >= 256 * 256 * sizeof(float)) {
+    a.logits_cache = logits_cache.untyped_data();
+    a.logits_cache_bytes = logits_cache.size_bytes();
+  }
   return status_to_error(ct_cutce_bwd(stream, &a));
 }
 
@@ -216,6 +225,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_cutce_fwd, CutceFwd,
                                   .Ret<ffi::Buffer<ffi::F32>>()
                                   .Ret<ffi::Buffer<ffi::F32>>()
                                   .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
                                   .Attr<bool>("sparse_compaction"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_cutce_bwd, CutceBwd,
@@ -226,6 +236,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_cutce_bwd, CutceBwd,
                                   .Arg<ffi::Buffer<ffi::F32>>()
                                   .Arg<ffi::Buffer<ffi::F32>>()
                                   .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::U8>>()
                                   .Ret<ffi::Buffer<ffi::BF16>>()
                                   .Ret<ffi::Buffer<ffi::BF16>>()
                                   .Ret<ffi::Buffer<ffi::U8>>()

@@ -4,7 +4,7 @@
 meaning, validation errors and custom-VJP contract
 (src/causal_trainer/kernels/cut_cross_entropy.py:828-958, :524-670): it
 returns ``(nll_sum, weight_sum)`` as f32 scalars, saves
-``(hidden, head, targets, weights, lse)`` and no logits, gives no cotangent to
+``(hidden, head, targets, weights, lse)``, gives no cotangent to
 targets / weights, ignores the cotangent of ``weight_sum``, and with
 ``lm_head_trainable=False`` never launches the dHead kernel and returns no
 head gradient. Tensors are torch tensors on a ROCm device; the work is done by
@@ -12,6 +12,14 @@ libct_hotpath.so through its C ABI.
 
 ``loss = nll_sum / max(weight_sum, 1)`` stays with the caller
 (src/causal_trainer/training/losses.py:234-237).
+
+One deliberate difference in the residual. The reference keeps no logits because
+a TPU core has little memory, and pays for it by recomputing the projection in
+each backward kernel. A MI355X has 288 GB: when the f32 logits of the active
+rows fit in ``LOGITS_CACHE_LIMIT_BYTES`` the forward also leaves them in a cache
+that lives until the backward of the loss (the adjacent step of a training
+iteration), and the backward then runs 3 GEMMs instead of 4. Above the limit, or
+with ``logits_cache=False``, nothing but ``lse`` is kept and logits are recomputed.
 """
 
 from __future__ import annotations
@@ -24,14 +32,27 @@ from . import _lib
 from .efficient_attention import _mesh_sizes
 
 _HIDDEN_ALIGN = 128
+# Largest logits cache the operator allocates by itself (f32 [vocab, rows], both padded to 256).
+LOGITS_CACHE_LIMIT_BYTES = 24 << 30
 
 
 def _shape_struct(rows: int, hidden: int, vocab: int) -> _lib.CutceShape:
     return _lib.CutceShape(rows=rows, hidden=hidden, vocab=vocab)
 
 
-def cutce_forward(hidden, head, targets, weights, *, sparse_compaction: bool = False):
-    """Flat forward: hidden [N, d], head [d, V] -> (nll_sum, weight_sum, lse [N])."""
+def logits_cache_bytes(rows: int, hidden: int, vocab: int) -> int:
+    """Size of the optional f32 logits cache for this problem."""
+
+    return int(_lib.load().ct_cutce_logits_cache_bytes(_shape_struct(rows, hidden, vocab)))
+
+
+def cutce_forward(hidden, head, targets, weights, *, sparse_compaction: bool = False,
+                  logits_cache=None):
+    """Flat forward: hidden [N, d], head [d, V] -> (nll_sum, weight_sum, lse [N]).
+
+    ``logits_cache``: optional uint8 device tensor of ``logits_cache_bytes(...)`` bytes that
+    the forward fills for ``cutce_backward``.
+    """
 
     lib = _lib.load()
     rows, width = hidden.shape
@@ -46,6 +67,8 @@ def cutce_forward(hidden, head, targets, weights, *, sparse_compaction: bool = F
         weight_sum=scalars[1:].data_ptr(), lse=lse.data_ptr(),
         workspace=workspace.data_ptr(), workspace_bytes=workspace.numel(),
         shape=shape, sparse_compaction=int(bool(sparse_compaction)),
+        logits_cache=_lib.pointer(logits_cache),
+        logits_cache_bytes=0 if logits_cache is None else logits_cache.numel(),
     )
     with torch.cuda.device(device):
         _lib.check(lib.ct_cutce_fwd(_lib.current_stream(), args))
@@ -53,8 +76,13 @@ def cutce_forward(hidden, head, targets, weights, *, sparse_compaction: bool = F
 
 
 def cutce_backward(hidden, head, targets, weights, lse, dy, *, sparse_compaction: bool = False,
-                   lm_head_trainable: bool = True, workspace_bytes: int | None = None):
-    """Flat backward: returns (dhidden [N, d], dhead [d, V] or None)."""
+                   lm_head_trainable: bool = True, workspace_bytes: int | None = None,
+                   logits_cache=None):
+    """Flat backward: returns (dhidden [N, d], dhead [d, V] or None).
+
+    ``logits_cache``: the tensor a forward with the same ``sparse_compaction`` filled, or None
+    to recompute the logits.
+    """
 
     lib = _lib.load()
     rows, width = hidden.shape
@@ -72,6 +100,8 @@ def cutce_backward(hidden, head, targets, weights, lse, dy, *, sparse_compaction
         dhidden=dhidden.data_ptr(), dhead=_lib.pointer(dhead),
         workspace=workspace.data_ptr(), workspace_bytes=workspace.numel(),
         shape=shape, sparse_compaction=int(bool(sparse_compaction)),
+        logits_cache=_lib.pointer(logits_cache),
+        logits_cache_bytes=0 if logits_cache is None else logits_cache.numel(),
     )
     with torch.cuda.device(device):
         _lib.check(lib.ct_cutce_bwd(_lib.current_stream(), args))
@@ -80,11 +110,19 @@ def cutce_backward(hidden, head, targets, weights, lse, dy, *, sparse_compaction
 
 class _CutCE(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, head, targets, weights, lm_head_trainable, sparse_compaction):
+    def forward(ctx, hidden, head, targets, weights, lm_head_trainable, sparse_compaction,
+                logits_cache):
+        cache = None
+        if logits_cache and (hidden.requires_grad or head.requires_grad):
+            size = logits_cache_bytes(hidden.shape[0], hidden.shape[1], head.shape[1])
+            if size <= LOGITS_CACHE_LIMIT_BYTES:
+                cache = torch.empty(size, dtype=torch.uint8, device=hidden.device)
         nll_sum, weight_sum, lse = cutce_forward(hidden, head, targets, weights,
-                                                 sparse_compaction=sparse_compaction)
-        # The complete residual: no logits (reference :587-593).
+                                                 sparse_compaction=sparse_compaction,
+                                                 logits_cache=cache)
+        # The reference's residual (:587-593) plus, when it fits, the f32 logits cache.
         ctx.save_for_backward(hidden, head, targets, weights, lse)
+        ctx.logits_cache = cache
         ctx.lm_head_trainable = lm_head_trainable
         ctx.sparse_compaction = sparse_compaction
         ctx.mark_non_differentiable(weight_sum)
@@ -96,14 +134,18 @@ class _CutCE(torch.autograd.Function):
         dhidden, dhead = cutce_backward(
             hidden, head, targets, weights, lse, nll_cotangent,
             sparse_compaction=ctx.sparse_compaction, lm_head_trainable=ctx.lm_head_trainable,
+            logits_cache=ctx.logits_cache,
         )
-        return dhidden, dhead, None, None, None, None
+        ctx.logits_cache = None
+        return dhidden, dhead, None, None, None, None, None
 
 
 def pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weights, *, mesh=None,
                                     sparse_compaction: bool = False,
-                                    lm_head_trainable: bool = True, local_chunk_size: int = 0):
-    """Return ``(nll_sum, weight_sum)`` without materialising logits.
+                                    lm_head_trainable: bool = True, local_chunk_size: int = 0,
+                                    logits_cache: bool = True):
+    """Return ``(nll_sum, weight_sum)``; logits are only ever kept in the bounded cache
+    described in the module docstring (``logits_cache=False`` disables it).
 
     hidden_states ``[B, S, d]``, lm_head_kernel ``[d, V]`` (same float dtype, bf16),
     targets int32 ``[B, S]``, weights f32 ``[B, S]``; a row is ignored iff its weight is 0.
@@ -156,8 +198,9 @@ def pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weig
     return _CutCE.apply(
         hidden_states.reshape(-1, width).contiguous(), lm_head_kernel.contiguous(),
         targets.reshape(-1).contiguous(), weights.reshape(-1).contiguous(),
-        bool(lm_head_trainable), bool(sparse_compaction),
+        bool(lm_head_trainable), bool(sparse_compaction), bool(logits_cache),
     )
 
 
-__all__ = ["cutce_backward", "cutce_forward", "pallas_cut_linear_cross_entropy"]
+__all__ = ["LOGITS_CACHE_LIMIT_BYTES", "cutce_backward", "cutce_forward", "logits_cache_bytes",
+           "pallas_cut_linear_cross_entropy"]

@@ -100,41 +100,55 @@ def make_efficient_attention():
     return attention
 
 
-def make_cut_cross_entropy(*, sparse_compaction: bool, lm_head_trainable: bool):
-    """Returns ``cut_ce(hidden[N, d], head[d, V], targets[N], weights[N]) -> (nll_sum, weight_sum)``."""
+def make_cut_cross_entropy(*, sparse_compaction: bool, lm_head_trainable: bool,
+                           logits_cache_limit_bytes: int = 24 << 30):
+    """Returns ``cut_ce(hidden[N, d], head[d, V], targets[N], weights[N]) -> (nll_sum, weight_sum)``.
+
+    When the f32 logits cache of the problem fits in ``logits_cache_limit_bytes`` the forward
+    under differentiation also returns it as a residual and the backward skips the logit
+    recomputation; otherwise the residual is the reference's (no logits).
+    """
 
     import jax
     import jax.numpy as jnp
 
     register()
 
-    def forward(hidden, head, targets, weights):
+    def forward(hidden, head, targets, weights, cache_bytes):
         rows, width = hidden.shape
         scalar = jax.ShapeDtypeStruct((1,), jnp.float32)
         shapes = (scalar, scalar, jax.ShapeDtypeStruct((rows,), jnp.float32),
-                  jax.ShapeDtypeStruct((_workspace_bytes("fwd", rows, width, head.shape[1]),), jnp.uint8))
-        nll, weight_sum, lse, _ = jax.ffi.ffi_call("ct_ffi_cutce_fwd", shapes)(
+                  jax.ShapeDtypeStruct((_workspace_bytes("fwd", rows, width, head.shape[1]),), jnp.uint8),
+                  jax.ShapeDtypeStruct((max(cache_bytes, 16),), jnp.uint8))   # 16 bytes = "no cache"
+        nll, weight_sum, lse, _, cache = jax.ffi.ffi_call("ct_ffi_cutce_fwd", shapes)(
             hidden, head, targets, weights, sparse_compaction=sparse_compaction)
-        return nll[0], weight_sum[0], lse
+        return nll[0], weight_sum[0], lse, cache
+
+    def cache_bytes_for(hidden, head):
+        from . import _lib
+
+        shape = _lib.CutceShape(rows=hidden.shape[0], hidden=hidden.shape[1], vocab=head.shape[1])
+        size = int(_lib.load().ct_cutce_logits_cache_bytes(shape))
+        return size if size <= logits_cache_limit_bytes else 0
 
     @jax.custom_vjp
     def cut_ce(hidden, head, targets, weights):
-        nll, weight_sum, _ = forward(hidden, head, targets, weights)
+        nll, weight_sum, _, _ = forward(hidden, head, targets, weights, 0)
         return nll, weight_sum
 
     def cut_ce_fwd(hidden, head, targets, weights):
-        nll, weight_sum, lse = forward(hidden, head, targets, weights)
-        return (nll, weight_sum), (hidden, head, targets, weights, lse)         # no logits
+        nll, weight_sum, lse, cache = forward(hidden, head, targets, weights, cache_bytes_for(hidden, head))
+        return (nll, weight_sum), (hidden, head, targets, weights, lse, cache)
 
     def cut_ce_bwd(residual, cotangents):
-        hidden, head, targets, weights, lse = residual
+        hidden, head, targets, weights, lse, cache = residual
         nll_cotangent, _ = cotangents
         rows, width = hidden.shape
         shapes = (jax.ShapeDtypeStruct(hidden.shape, hidden.dtype), jax.ShapeDtypeStruct(head.shape, head.dtype),
                   jax.ShapeDtypeStruct((_workspace_bytes("bwd", rows, width, head.shape[1]),), jnp.uint8))
         dhidden, dhead, _ = jax.ffi.ffi_call("ct_ffi_cutce_bwd", shapes)(
             hidden, head, targets, weights, lse, jnp.reshape(nll_cotangent.astype(jnp.float32), (1,)),
-            sparse_compaction=sparse_compaction, head_trainable=lm_head_trainable)
+            cache, sparse_compaction=sparse_compaction, head_trainable=lm_head_trainable)
         return dhidden, (dhead if lm_head_trainable else None), None, None
 
     cut_ce.defvjp(cut_ce_fwd, cut_ce_bwd)

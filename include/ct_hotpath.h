@@ -188,6 +188,19 @@ size_t ct_cutce_fwd_workspace_bytes(const ct_cutce_shape* shape);
  */
 size_t ct_cutce_bwd_workspace_min_bytes(const ct_cutce_shape* shape);
 size_t ct_cutce_bwd_workspace_bytes(const ct_cutce_shape* shape);
+/*
+ * Bytes of the optional logits cache (f32, vocabulary-major, rows and
+ * vocabulary padded to 256). When the caller lends one to ct_cutce_fwd and
+ * hands the same buffer to ct_cutce_bwd, the backward forms its bf16 dlogits
+ * from the cached f32 logits instead of repeating the projection: 3 GEMMs per
+ * step instead of 4 (the reference runs 5, src/kernels/cut_cross_entropy.py:258,
+ * :383). No reference counterpart: the reference never keeps logits because a
+ * TPU core has 32 GB; at N = 16384, V = 128256 the cache is 8.4 GB of 288 GB and
+ * only lives from the forward of the loss to its backward, the adjacent step.
+ * Both calls must use the same sparse_compaction flag (the cache is indexed by
+ * the compacted row order).
+ */
+size_t ct_cutce_logits_cache_bytes(const ct_cutce_shape* shape);
 
 typedef struct ct_cutce_fwd_args {
   const uint16_t* hidden;  /* bf16 [rows, hidden] */
@@ -201,12 +214,14 @@ typedef struct ct_cutce_fwd_args {
   size_t workspace_bytes;
   ct_cutce_shape shape;
   int32_t sparse_compaction; /* gather active rows first (same results) */
+  void* logits_cache;        /* NULL, or ct_cutce_logits_cache_bytes() of device memory to fill */
+  size_t logits_cache_bytes;
 } ct_cutce_fwd_args;
 
 /*
  * nll_sum = sum_i w_i (logsumexp_v(hidden_i . head[:, v]) - hidden_i . head[:, t_i]),
- * weight_sum = sum_i w_i, lse_i saved for the backward. Logits are never
- * written to memory.
+ * weight_sum = sum_i w_i, lse_i saved for the backward. Logits are not
+ * written to memory unless the caller lends a logits cache.
  * Replaces: _cut_stats_pallas + _loss_and_lse + _compact_active_rows
  * (src/kernels/cut_cross_entropy.py:85-222, :474-521, :673-694).
  */
@@ -226,6 +241,8 @@ typedef struct ct_cutce_bwd_args {
   size_t workspace_bytes;
   ct_cutce_shape shape;
   int32_t sparse_compaction;
+  const void* logits_cache;  /* NULL (logits are recomputed), or the buffer ct_cutce_fwd filled */
+  size_t logits_cache_bytes;
 } ct_cutce_bwd_args;
 
 /*

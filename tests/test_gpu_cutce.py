@@ -41,11 +41,19 @@ def _case(seed, rows, width, vocab, pattern="random", hidden_scale=1.0, head_sca
     return hidden, head, torch.from_numpy(targets), torch.from_numpy(weights)
 
 
-def _gpu(ct, device, hidden, head, targets, weights, dy, *, compaction, trainable=True, workspace=None):
+def _gpu(ct, device, hidden, head, targets, weights, dy, *, compaction, trainable=True, workspace=None,
+         cache=False):
     hd, wd, td, ws = hidden.to(device), head.to(device), targets.to(device), weights.to(device)
-    nll, weight_sum, lse = ct.cutce_forward(hd, wd, td, ws, sparse_compaction=compaction)
+    logits_cache = None
+    if cache:
+        size = ct.cut_cross_entropy.logits_cache_bytes(hidden.shape[0], hidden.shape[1], head.shape[1])
+        # poisoned: every logit the backward uses must have been written by the forward
+        logits_cache = torch.full((size,), 0xFF, dtype=torch.uint8, device=device)
+    nll, weight_sum, lse = ct.cutce_forward(hd, wd, td, ws, sparse_compaction=compaction,
+                                            logits_cache=logits_cache)
     dhidden, dhead = ct.cutce_backward(hd, wd, td, ws, lse, torch.tensor(dy), sparse_compaction=compaction,
-                                       lm_head_trainable=trainable, workspace_bytes=workspace)
+                                       lm_head_trainable=trainable, workspace_bytes=workspace,
+                                       logits_cache=logits_cache)
     torch.cuda.synchronize()
     return float(nll), float(weight_sum), lse.cpu(), dhidden.cpu(), None if dhead is None else dhead.cpu()
 
@@ -73,10 +81,27 @@ def _check(results, hidden, head, targets, weights, dy):
 @pytest.mark.parametrize("rows,width,vocab", [(256, 128, 256), (300, 128, 258), (1000, 256, 1500),
                                               (513, 384, 1031), (64, 128, 40)])
 @pytest.mark.parametrize("compaction", [True, False])
-def test_forward_backward_match_oracle(ct, gpu, rows, width, vocab, compaction):
-    print("case", rows, width, vocab, compaction, flush=True)
+@pytest.mark.parametrize("cache", [False, True])
+def test_forward_backward_match_oracle(ct, gpu, rows, width, vocab, compaction, cache):
+    print("case", rows, width, vocab, compaction, cache, flush=True)
     case = _case(rows + vocab, rows, width, vocab)
-    _check(_gpu(ct, gpu, *case, 0.37, compaction=compaction), *case, 0.37)
+    _check(_gpu(ct, gpu, *case, 0.37, compaction=compaction, cache=cache), *case, 0.37)
+
+
+def test_cached_logits_give_the_recomputed_gradients(ct, gpu):
+    # the cache holds the same f32 logits the recomputation produces, so G and both gradients
+    # agree to the last bit; also through the slab walk of a small workspace
+    case = _case(21, 900, 256, 1500)
+    plain = _gpu(ct, gpu, *case, 0.5, compaction=True)
+    cached = _gpu(ct, gpu, *case, 0.5, compaction=True, cache=True)
+    assert plain[0] == cached[0] and torch.equal(plain[2], cached[2])
+    assert torch.equal(plain[3], cached[3]) and torch.equal(plain[4], cached[4])
+    import ctypes
+    shape = ct._lib.CutceShape(900, 256, 1500)
+    least = ct._lib.load().ct_cutce_bwd_workspace_min_bytes(ctypes.byref(shape))
+    slabs = _gpu(ct, gpu, *case, 0.5, compaction=True, cache=True, workspace=least)
+    _check(slabs, *case, 0.5)
+    assert torch.equal(slabs[4], cached[4])
 
 
 @pytest.mark.parametrize("pattern", ["trailing", "alternating", "middle", "inactive"])
