@@ -35,9 +35,35 @@ def parse_args():
     parser.add_argument("--cutce-steps", type=int, default=None, help="default: min(steps, 5)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-cutce", action="store_true")
+    parser.add_argument("--calibration-copy-bytes", type=int, default=0,
+                        help="also launch one plain device copy of this many bytes (for scaling "
+                             "FETCH_SIZE / WRITE_SIZE when the run is under rocprofv3 --pmc)")
     parser.add_argument("--cutce-recompute", action="store_true",
                         help="cut-CE without the logits cache (backward recomputes the projection)")
     return parser.parse_args()
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` (fetch + write) from the committed counter summary
+    profiles/traffic.json, which causal-trainer-dev_amd/rocprof_traffic.py writes from two
+    rocprofv3 --pmc runs of this same script (FETCH_SIZE, WRITE_SIZE, each scaled by the
+    calibration copy). None when the kernel has not been measured."""
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "traffic.json")
+    try:
+        with open(path) as handle:
+            entry = json.load(handle)["kernels"].get(kernel)
+    except (OSError, ValueError, KeyError):
+        return None
+    return None if entry is None else entry["fetch_bytes"] + entry["write_bytes"]
+
+
+def calibration_copy(ct, torch, nbytes):
+    source = torch.ones(nbytes, dtype=torch.uint8, device="cuda")
+    target = torch.empty_like(source)
+    ct._lib.check(ct._lib.load().ct_calibration_copy(ct._lib.current_stream(), target.data_ptr(),
+                                                     source.data_ptr(), nbytes))
+    torch.cuda.synchronize()
 
 
 def timed_region(torch, step, steps, warmup, timer_factory):
@@ -238,7 +264,7 @@ def main():
             "unit": "TFLOP/s",
             "frac": dominant["algorithmic_tflops"] / PEAK_BF16_TFLOPS,
             "avg_launch_ms": dominant["avg_ms"],
-            "traffic": None,
+            "traffic": measured_traffic(dominant["kernel"]),
         },
         "kernels": attention["kernels"],
     }
@@ -247,6 +273,8 @@ def main():
             "bound": "hbm", "achieved": delta["algorithmic_gbps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
             "frac": delta["algorithmic_gbps"] / PEAK_HBM_GBPS, "avg_launch_ms": delta["avg_ms"],
         }
+    if args.calibration_copy_bytes:
+        calibration_copy(ct, torch, args.calibration_copy_bytes)
     if not args.no_cutce:
         cut_steps = args.cutce_steps or min(args.steps, 5)
         result["cutce"] = bench_cutce(ct, torch, cut_steps, min(args.warmup, 2),

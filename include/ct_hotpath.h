@@ -169,6 +169,14 @@ int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* args);
 int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16_t* dout,
                       float* delta, int64_t rows, int32_t head_dim);
 
+/*
+ * Measurement aid, no reference counterpart: copies `bytes` (a multiple of 16,
+ * both pointers 16-byte aligned) device to device with a plain kernel. Run
+ * under the same hardware counters as the hot-path kernels it gives the factor
+ * between what FETCH_SIZE / WRITE_SIZE report and bytes actually moved.
+ */
+int32_t ct_calibration_copy(void* stream, void* dst, const void* src, size_t bytes);
+
 /* ------------------------------------------------------------------------
  * Cut cross-entropy
  * --------------------------------------------------------------------- */
