@@ -33,7 +33,8 @@ constexpr float kNegInfF = -__builtin_inff();
 struct CutceHeader {
   int n_act;
   int counter;
-  int pad[14];
+  int xcd_counter[8];  // per-XCD work counters of the statistics kernel
+  int pad[6];
 };
 
 struct CutceParams {
@@ -61,6 +62,7 @@ __global__ __launch_bounds__(1024) void cutce_index_kernel(const float* weights,
       header->n_act = N;
       header->counter = 0;
     }
+    if (tid < 8) header->xcd_counter[tid] = 0;
     return;
   }
   int carry = 0;
@@ -87,6 +89,7 @@ __global__ __launch_bounds__(1024) void cutce_index_kernel(const float* weights,
     header->n_act = carry;
     header->counter = 0;
   }
+  if (tid < 8) header->xcd_counter[tid] = 0;
 }
 
 // ---------------------------------------------------------------------------
@@ -107,17 +110,46 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
   __shared__ int unit_s;
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
-  const int row_blocks = p.n_pad / kGemmTile;
   const int vocab_tiles = (p.V + kGemmTile - 1) / kGemmTile;
-  const int total = chunks * row_blocks;
   const int n_act = p.header->n_act;
 
+  // Work order. A unit is (vocabulary chunk, row block). Each XCD has its own L2, so the
+  // workgroups of one XCD should work on units that share operands at the same time: the
+  // (chunk, row block) grid is walked in blocks of kChunkGroup x kRowGroup units (32 units = the
+  // 32 compute units of an XCD: 4 head tiles and 8 hidden blocks feed 32 GEMM tiles), the
+  // sequence of blocks is cut into 8 equal ranges, and an XCD takes the units of its range
+  // through its own counter. Indices that fall outside the grid (ragged edges) are skipped.
+  // An XCD that runs dry helps the next one.
+  constexpr int kChunkGroup = 4, kRowGroup = 8, kXcds = 8;
+  const int active_blocks = (n_act + kGemmTile - 1) / kGemmTile;
+  const int row_groups = (active_blocks + kRowGroup - 1) / kRowGroup;
+  const int chunk_groups = (chunks + kChunkGroup - 1) / kChunkGroup;
+  const int padded_total = chunk_groups * row_groups * kChunkGroup * kRowGroup;
+  const int per_xcd = (padded_total + kXcds - 1) / kXcds;
+  unsigned xcc_id;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_id));
+  const int my_xcd = (int)(xcc_id & 7u);
+  int helping = 0;  // how many XCDs further the counter in use belongs to
+
   for (;;) {
-    if (tid == 0) unit_s = atomicAdd(&p.header->counter, 1);
-    __syncthreads();
-    const int unit = unit_s;
-    if (unit >= total) break;
-    const int chunk = unit / row_blocks, rb = unit % row_blocks;
+    int index = -1;
+    while (helping < kXcds) {
+      const int x = (my_xcd + helping) % kXcds;
+      if (tid == 0) unit_s = atomicAdd(&p.header->xcd_counter[x], 1);
+      __syncthreads();
+      const int local = unit_s;
+      __syncthreads();
+      if (local < per_xcd && x * per_xcd + local < padded_total) {
+        index = x * per_xcd + local;
+        break;
+      }
+      ++helping;
+    }
+    if (index < 0) break;
+    const int in_block = index % (kChunkGroup * kRowGroup), block = index / (kChunkGroup * kRowGroup);
+    const int chunk = (block / row_groups) * kChunkGroup + in_block / kRowGroup;
+    const int rb = (block % row_groups) * kRowGroup + in_block % kRowGroup;
+    if (chunk >= chunks || rb >= active_blocks) continue;
     const int n0 = rb * kGemmTile;
     const int my_slot = n0 + tid;
     const int active = my_slot < n_act && p.weights[p.idx[my_slot]] != 0.f;
