@@ -344,7 +344,11 @@ static int launch_dkv(hipStream_t stream, const AttnParams& p) {
   const int grid = p.dkv_max_entries * p.Hkv;  // entries beyond the list's length exit at once
   LaunchScope scope3("attn_dkv_kernel", stream);
   hipLaunchKernelGGL((attn_dkv_kernel<D>), dim3(grid), dim3(256), smem, stream, p);
-  return scope3.done();
+  rc = scope3.done();
+  if (rc) return rc;
+  LaunchScope scope9("attn_dkv_reduce_kernel", stream);
+  hipLaunchKernelGGL((attn_dkv_reduce_kernel<D>), dim3(grid), dim3(256), 4 * 32 * D * 2, stream, p);
+  return scope9.done();
 }
 
 template <int D>

@@ -349,6 +349,63 @@ __global__ __launch_bounds__(1024) void attn_dkv_schedule_kernel(const int* meta
   }
 }
 
+// f32 partial sums of one chunk of a split key tile.
+template <int D>
+struct DkvPartial {
+  static constexpr int kPerWave = (D / 32) * 16 * 64;  // floats of one accumulator set of a wavefront
+  static constexpr int kPerTensor = 4 * kPerWave;      // dK (or dV) of the 4 wavefronts
+  static constexpr size_t kPerChunk = 2 * kPerTensor;
+};
+template <int D>
+CT_DEVICE size_t dkv_partial_offset(int slot, int Hkv, int kvh, int wave) {
+  return ((size_t)slot * Hkv + kvh) * DkvPartial<D>::kPerChunk + (size_t)wave * DkvPartial<D>::kPerWave;
+}
+
+// Adds the chunks of every split key tile in chunk order (fixed order: the result does not
+// depend on timing) and writes dK, dV. One workgroup per (entry, KV head); only the entry of
+// chunk 0 of a split tile has work.
+template <int D>
+__global__ __launch_bounds__(256) void attn_dkv_reduce_kernel(AttnParams p) {
+  extern __shared__ __align__(16) char smem_raw[];
+  const lds_addr lds0 = lds_address_of(smem_raw);
+  const int l = lane_id(), w = threadIdx.x >> 6;
+  const int nrb = p.S / 32;
+  const int kvh = blockIdx.x % p.Hkv, entry = blockIdx.x / p.Hkv;
+  if (entry >= uniform(p.dkv_header[0])) return;
+  const int2 work_entry = p.dkv_entries[entry];
+  const int tile = uniform(work_entry.x), packed = uniform(work_entry.y);
+  const int chunk = packed & 255, nsplit = (packed >> 8) & 255, slot0 = (unsigned)packed >> 16;
+  if (chunk != 0 || nsplit <= 1) return;
+  const int b = tile / (nrb / 4), kt = tile % (nrb / 4);
+  f32x16 dkacc[D / 32], dvacc[D / 32];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db) {
+    dkacc[db] = zero16();
+    dvacc[db] = zero16();
+  }
+  for (int c = 0; c < nsplit; ++c) {
+    const float* src = p.dkv_partials + dkv_partial_offset<D>(slot0 + c, p.Hkv, kvh, w) + l * 4;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int q4 = 0; q4 < 4; ++q4) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>(src + (db * 4 + q4) * 256);
+        const f32x4 cv = *reinterpret_cast<const f32x4*>(src + DkvPartial<D>::kPerTensor + (db * 4 + q4) * 256);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          dkacc[db][4 * q4 + e] += a[e];
+          dvacc[db][4 * q4 + e] += cv[e];
+        }
+      }
+  }
+  const lds_addr patch = lds0 + w * 32 * D * 2;
+  const size_t kv_row_stride = (size_t)p.Hkv * D;
+  const size_t out_off = (((size_t)b * p.S + (kt * 4 + w) * 32) * p.Hkv + kvh) * D;
+  store_rows<D>(dkacc, patch, p.dk + out_off, kv_row_stride);
+  __builtin_amdgcn_wave_barrier();
+  store_rows<D>(dvacc, patch, p.dv + out_off, kv_row_stride);
+}
+
 template <int D>
 __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   extern __shared__ __align__(16) char smem_raw[];
@@ -482,41 +539,23 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   }
 
   if (nsplit > 1) {
-    // Leave this chunk's sums as f32, laid out [dK | dV][wavefront][d block][register][lane].
-    constexpr int kPerWave = (D / 32) * 16 * 64;
-    constexpr size_t kPerChunk = 2 * 4 * kPerWave;
-    float* mine = p.dkv_partials + ((size_t)(slot0 + chunk) * p.Hkv + kvh) * kPerChunk + w * kPerWave + l;
+    // A chunk of a split tile leaves its sums as f32 for attn_dkv_reduce_kernel:
+    // [dK | dV][wavefront][d block][register quad][lane][4], 16 bytes per lane and store.
+    float* mine = p.dkv_partials + dkv_partial_offset<D>(slot0 + chunk, p.Hkv, kvh, w) + l * 4;
 #pragma unroll
     for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        mine[(db * 16 + r) * 64] = dkacc[db][r];
-        mine[4 * kPerWave + (db * 16 + r) * 64] = dvacc[db][r];
-      }
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0)
-      lds_store<int>(lds0 + QdoStage<D>::kLastFlag,
-                     atomicAdd(&p.dkv_counters[tile * p.Hkv + kvh], 1) == nsplit - 1);
-    __syncthreads();
-    if (!uniform(lds_load<int>(lds0 + QdoStage<D>::kLastFlag))) return;
-    __threadfence();
-    // Last chunk to arrive: add all chunks in chunk order.
+      for (int q4 = 0; q4 < 4; ++q4) {
+        f32x4 a, c;
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db) {
-      dkacc[db] = zero16();
-      dvacc[db] = zero16();
-    }
-    for (int c = 0; c < nsplit; ++c) {
-      const float* src = p.dkv_partials + ((size_t)(slot0 + c) * p.Hkv + kvh) * kPerChunk + w * kPerWave + l;
-#pragma unroll
-      for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          dkacc[db][r] += src[(db * 16 + r) * 64];
-          dvacc[db][r] += src[4 * kPerWave + (db * 16 + r) * 64];
+        for (int e = 0; e < 4; ++e) {
+          a[e] = dkacc[db][4 * q4 + e];
+          c[e] = dvacc[db][4 * q4 + e];
         }
-    }
+        *reinterpret_cast<f32x4*>(mine + (db * 4 + q4) * 256) = a;
+        *reinterpret_cast<f32x4*>(mine + DkvPartial<D>::kPerTensor + (db * 4 + q4) * 256) = c;
+      }
+    return;
   }
 
   const lds_addr patch = vpatch;  // V fragments are no longer needed
