@@ -87,7 +87,7 @@ SYMBOLS = {
     "ct_abi_version": (c_int32, []),
     "ct_calibration_copy": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
     "ct_attn_meta_bytes": (c_size_t, [c_int32, c_int32]),
-    "ct_attn_bwd_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32]),
+    "ct_attn_bwd_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32]),
     "ct_attn_prepare": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "ct_attn_block_summary": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
                                         c_void_p]),

@@ -351,19 +351,27 @@ static int launch_dkv(hipStream_t stream, const AttnParams& p) {
   return scope9.done();
 }
 
+// lse2 == nullptr: delta in row order (b, s, h); otherwise delta and lse * log2(e) head-major.
 template <int D>
 static int launch_delta(hipStream_t stream, const bf16* out, const bf16* dout, float* delta,
-                        long rows) {
+                        long rows, const float* lse = nullptr, float* lse2 = nullptr, int S = 0,
+                        int Hq = 0) {
   const long threads = rows * (D / 8);
+  const dim3 grid((unsigned)((threads + 255) / 256));
   LaunchScope scope4("attn_delta_kernel", stream);
-  hipLaunchKernelGGL((attn_delta_kernel<D>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0,
-                     stream, out, dout, delta, rows);
+  if (lse2)
+    hipLaunchKernelGGL((attn_delta_kernel<D, true>), grid, dim3(256), 0, stream, out, dout, delta,
+                       rows, lse, lse2, S, Hq);
+  else
+    hipLaunchKernelGGL((attn_delta_kernel<D, false>), grid, dim3(256), 0, stream, out, dout, delta,
+                       rows, lse, lse2, S, Hq);
   return scope4.done();
 }
 
 template <int D>
 static int dispatch_bwd(hipStream_t stream, const AttnParams& p) {
-  int rc = launch_delta<D>(stream, p.out, p.dout, p.delta, (long)p.B * p.S * p.Hq);
+  int rc = launch_delta<D>(stream, p.out, p.dout, p.delta, (long)p.B * p.S * p.Hq, p.lse, p.lse2,
+                           p.S, p.Hq);
   if (rc) return rc;
   switch (heads_per_group(p.Hq, p.Hkv)) {
     case 4: rc = launch_dq<D, 4>(stream, p); break;
@@ -383,10 +391,12 @@ extern "C" size_t ct_attn_meta_bytes(int32_t batch, int32_t seq) {
   return meta_total_ints(batch, seq / 32) * sizeof(int32_t);
 }
 
-extern "C" size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t kv_heads,
-                                             int32_t head_dim) {
-  if (batch <= 0 || seq <= 0 || kv_heads <= 0 || head_dim <= 0 || seq % kDkvKeys != 0) return 0;
-  return dkv_layout(batch, seq, kv_heads, head_dim).total;
+extern "C" size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t q_heads,
+                                             int32_t kv_heads, int32_t head_dim) {
+  if (batch <= 0 || seq <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 ||
+      seq % kDkvKeys != 0)
+    return 0;
+  return dkv_layout(batch, seq, q_heads, kv_heads, head_dim).total;
 }
 
 extern "C" int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
@@ -511,7 +521,7 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   p.Hq = a->q_heads;
   p.Hkv = a->kv_heads;
   p.scale = round_to_bf16(a->scale);
-  const DkvLayout L = dkv_layout(a->batch, a->seq, a->kv_heads, a->head_dim);
+  const DkvLayout L = dkv_layout(a->batch, a->seq, a->q_heads, a->kv_heads, a->head_dim);
   if (a->workspace_bytes < L.total)
     return fail(CT_WORKSPACE_TOO_SMALL, "ct_attn_bwd: workspace %zu < %zu bytes", a->workspace_bytes,
                 L.total);
@@ -520,6 +530,7 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   p.dkv_counters = reinterpret_cast<int*>(ws + L.counters);
   p.dkv_entries = reinterpret_cast<int2*>(ws + L.entries);
   p.dkv_partials = reinterpret_cast<float*>(ws + L.partials);
+  p.lse2 = reinterpret_cast<float*>(ws + L.lse2);
   p.dkv_max_entries = L.max_entries;
   p.dkv_max_partials = L.max_partials;
   return a->head_dim == 128 ? dispatch_bwd<128>((hipStream_t)stream, p)

@@ -32,8 +32,9 @@ __global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
   const TrFragOffsets<D / 8, KSlots::kAccum> to(lds0);
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
-  const float lse2 = p.lse[ctx.stat_off] * kLog2e;
-  const float delta_q = p.delta[ctx.stat_off];
+  const size_t stat_t = ((size_t)ctx.work.b * p.Hq + ctx.work.h) * p.S + ctx.pos;  // head-major
+  const float lse2 = p.lse2[stat_t];
+  const float delta_q = p.delta[stat_t];
 
   bf16x8 qf[D / 16], dof[D / 16];
 #pragma unroll
@@ -68,15 +69,28 @@ __global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
       f32x16 s[2], dp[2];
       scores_t<D>(CUR * kStage + KvStage<D>::kK, ro, qf, s);
       scores_t<D>(CUR * kStage + KvStage<D>::kV, ro, dof, dp);
-      unsigned allow[2] = {0xffffffffu, 0xffffffffu};
-      if (!ctx.interior(kb, t))
-        tile_mask(stage + KvStage<D>::kSeg, t, ctx.seg_q, ctx.end_q, ctx.row_valid, allow);
+      {
+        // Same specialisation as the forward: masked scores become -inf, so their
+        // probability exp2(-inf) is exactly 0 and so is dS.
+        const int k_uniform = uniform(kb.uniform);
+        const bool need_seg = ctx.mine.uniform == 0 || ctx.mine.uniform != k_uniform;
+        const bool need_causal = t * kKeyTile + kKeyTile - 1 > ctx.mine.end_min;
+        if (need_seg || need_causal) {
+          const int seg_cmp = ctx.row_valid ? ctx.seg_q : -1;
+          int last_rel = ctx.end_q - t * kKeyTile - 4 * half;
+          if (k_uniform == 0) {
+            mask_scores_t<true, true>(stage + KvStage<D>::kSeg, seg_cmp, last_rel, s);
+          } else {
+            if (seg_cmp != k_uniform) last_rel = -1;
+            mask_scores_t<false, true>(stage, seg_cmp, last_rel, s);
+          }
+        }
+      }
 #pragma unroll
       for (int kbk = 0; kbk < 2; ++kbk)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float prob =
-              ((allow[kbk] >> r) & 1u) ? exp2_fast(fmaf(s[kbk][r], kLog2e, -lse2)) : 0.f;
+          const float prob = exp2_fast(fmaf(s[kbk][r], kLog2e, -lse2));
           s[kbk][r] = prob * (dp[kbk][r] - delta_q);
         }
       accumulate_t<D>(CUR * kStage + KvStage<D>::kK, to, s, dqacc);
@@ -122,47 +136,40 @@ struct QdoStage {
   static constexpr int kTotalBytes = kLastFlag + 16;
 };
 
-// Per-row statistics of a query block, carried in registers by lanes 0..31 of the workgroup.
-struct QueryRowRegs {
-  float lse2, delta;
-  int seg, end;
-};
-
-// Starts the asynchronous copy of Q and dO rows of query block qb into `stage`.
+// Starts the asynchronous copy of query block qb of head h into `stage`: Q and dO rows, and
+// the per-row statistics. The four statistics arrays (lse2, delta: head-major f32; segment ids,
+// visible ends: i32) are 128 contiguous bytes each for the 32 rows, and sit in the stage in that
+// order, so lanes 0..31 of wavefront 0 fetch them with one copy instruction (8 lanes per
+// array). Without visible ends (plain causal) the last 8 lanes stay idle.
 template <int D>
-CT_DEVICE void qdo_fetch(QueryRowRegs& r, const TileDma<kQueryTile, D / 8>& dma, const AttnParams& p,
-                         int b, int h, int qb, lds_addr stage) {
+CT_DEVICE void qdo_fetch(const TileDma<kQueryTile, D / 8>& dma, const AttnParams& p, int b, int h,
+                         int qb, lds_addr stage) {
   const int tid = threadIdx.x;
   const size_t origin = (((size_t)b * p.S + qb * kQueryTile) * p.Hq + h) * D;
   dma.issue(reinterpret_cast<const char*>(p.q + origin), stage + QdoStage<D>::kQ);
   dma.issue(reinterpret_cast<const char*>(p.dout + origin), stage + QdoStage<D>::kDo);
-  if (tid < kQueryTile) {
-    const int pos = qb * kQueryTile + tid;
-    const size_t so = ((size_t)b * p.S + pos) * p.Hq + h;
-    r.lse2 = p.lse[so] * kLog2e;
-    r.delta = p.delta[so];
-    r.seg = p.seg[(size_t)b * p.S + pos];
-    r.end = p.end ? p.end[(size_t)b * p.S + pos] : pos;
+  if (tid < (p.end ? 32 : 24)) {
+    const size_t head_major = ((size_t)b * p.Hq + h) * p.S + qb * kQueryTile;
+    const size_t row_major = (size_t)b * p.S + qb * kQueryTile;
+    const int which = tid >> 3, part = tid & 7;
+    const char* src = which == 0   ? reinterpret_cast<const char*>(p.lse2 + head_major)
+                      : which == 1 ? reinterpret_cast<const char*>(p.delta + head_major)
+                      : which == 2 ? reinterpret_cast<const char*>(p.seg + row_major)
+                                   : reinterpret_cast<const char*>(p.end + row_major);
+    dma16(src + part * 16, stage + QdoStage<D>::kLse);
   }
 }
 
-// After this thread's copies have landed (dma_wait_all), fold the softmax scale
-// into its own Q slots in place (bf16 multiply, as the forward does) and publish
-// the row statistics. A barrier must follow.
+// After this thread's copies have landed (dma_wait_all), fold the softmax scale into its own
+// Q slots in place (bf16 multiply, as the forward does). A barrier must follow.
 template <int D>
-CT_DEVICE void qdo_commit(const QueryRowRegs& r, lds_addr stage, float scale) {
+CT_DEVICE void qdo_commit(lds_addr stage, float scale) {
   constexpr int kSlots = kQueryTile * (D / 8) / 256;
   const int tid = threadIdx.x;
 #pragma unroll
   for (int n = 0; n < kSlots; ++n) {
     const lds_addr slot = stage + QdoStage<D>::kQ + (n * 256 + tid) * 16;
     lds_store<u32x4>(slot, as_u32x4(scale_bf16x8(as_bf16x8(lds_load<u32x4>(slot)), scale)));
-  }
-  if (tid < kQueryTile) {
-    lds_store<float>(stage + QdoStage<D>::kLse + tid * 4, r.lse2);
-    lds_store<float>(stage + QdoStage<D>::kDelta + tid * 4, r.delta);
-    lds_store<int>(stage + QdoStage<D>::kSeg + tid * 4, r.seg);
-    lds_store<int>(stage + QdoStage<D>::kEnd + tid * 4, r.end);
   }
 }
 
@@ -439,6 +446,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
 
   const int key = my_rb * 32 + j;
   const int seg_k = p.seg[(size_t)b * p.S + key];
+  const bool has_end = p.end != nullptr;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
   const size_t kv_off = (((size_t)b * p.S + key) * p.Hkv + kvh) * D;
 
@@ -472,10 +480,9 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   }
   const TileDma<kQueryTile, D / 8> dma((size_t)p.Hq * D * 2);
   if (it < items) {
-    QueryRowRegs regs;
-    qdo_fetch<D>(regs, dma, p, b, head, qb, lds0);
+    qdo_fetch<D>(dma, p, b, head, qb, lds0);
     dma_wait_all();
-    qdo_commit<D>(regs, lds0, p.scale);
+    qdo_commit<D>(lds0, p.scale);
   }
   __syncthreads();
 
@@ -488,8 +495,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
       qb_next = q_lo;
       ++head_next;
     }
-    QueryRowRegs regs;
-    if (more) qdo_fetch<D>(regs, dma, p, b, head_next, qb_next, lds0 + (CUR ^ 1) * kStage);
+    if (more) qdo_fetch<D>(dma, p, b, head_next, qb_next, lds0 + (CUR ^ 1) * kStage);
 
     const MetaPtr qm = meta_const(meta_b + qb * kMetaW);
     const int q_min = uniform(qm[kMinNz]), q_max = uniform(qm[kMaxId]),
@@ -511,12 +517,13 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
         i32x4 seg4, end4;
         if (!interior) {
           seg4 = lds_load<i32x4>(stage + QdoStage<D>::kSeg + r0 * 4);
-          end4 = lds_load<i32x4>(stage + QdoStage<D>::kEnd + r0 * 4);
+          if (has_end) end4 = lds_load<i32x4>(stage + QdoStage<D>::kEnd + r0 * 4);
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = 4 * qd + e;
-          const bool ok = interior || (seg4[e] == seg_k && seg_k != 0 && key <= end4[e]);
+          const int visible_end = has_end ? end4[e] : qb * kQueryTile + r0 + e;
+          const bool ok = interior || (seg4[e] == seg_k && seg_k != 0 && key <= visible_end);
           const float pr = ok ? exp2_fast(fmaf(s[r], kLog2e, -lse4[e])) : 0.f;
           prob[r] = pr;
           dp[r] = pr * (dp[r] - del4[e]);
@@ -526,7 +533,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
       accumulate_keys<D>(CUR * kStage + QdoStage<D>::kQ, to, dp, dkacc);
     }
     dma_wait_all();
-    if (more) qdo_commit<D>(regs, lds0 + (CUR ^ 1) * kStage, p.scale);
+    if (more) qdo_commit<D>(lds0 + (CUR ^ 1) * kStage, p.scale);
     __syncthreads();
     ++it;
     qb = qb_next;

@@ -44,7 +44,8 @@ struct AttnParams {
   bf16* out;        // forward: written; backward: forward output
   float* lse;
   const bf16* dout;
-  float* delta;
+  float* delta;     // backward: rowsum(out * dout), head-major [B, Hq, S]
+  float* lse2;      // backward: lse * log2(e), head-major [B, Hq, S]
   bf16* dq;
   bf16* dk;
   bf16* dv;
@@ -557,10 +558,14 @@ attn_fwd_kernel(AttnParams p) {
 // ---------------------------------------------------------------------------
 // delta[row] = sum_d f32(out[row, d]) * f32(dout[row, d])      (HBM bound)
 // One 16-byte load per lane per tensor; D/8 lanes share a row.
+// HEAD_MAJOR: rows are (b, s, h) flattened; the result goes to [B, Hq, S] order together
+// with lse * log2(e), so that the backward kernels read the 32 rows of a query block of one
+// head as 128 contiguous bytes.
 // ---------------------------------------------------------------------------
-template <int D>
+template <int D, bool HEAD_MAJOR>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* out, const bf16* dout,
-                                                         float* delta, long rows) {
+                                                         float* delta, long rows, const float* lse,
+                                                         float* lse2, int S, int Hq) {
   constexpr int LPR = D / 8;  // lanes per row
   const long gid = (long)blockIdx.x * 256 + threadIdx.x;
   const long row = gid / LPR;
@@ -574,7 +579,18 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* out, const 
   }
 #pragma unroll
   for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-  if (row < rows && c == 0) delta[row] = acc;
+  if (row < rows && c == 0) {
+    if constexpr (HEAD_MAJOR) {
+      const long bs = row / Hq;
+      const int h = (int)(row % Hq);
+      const long b = bs / S, pos = bs % S;
+      const long dst = (b * Hq + h) * S + pos;
+      delta[dst] = acc;
+      lse2[dst] = lse[row] * kLog2e;
+    } else {
+      delta[row] = acc;
+    }
+  }
 }
 
 }  // namespace ct

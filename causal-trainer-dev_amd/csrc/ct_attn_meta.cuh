@@ -106,12 +106,12 @@ constexpr int kDkvKeys = 128;      // keys per dK/dV tile
 
 struct DkvLayout {
   int max_entries, max_partials;
-  size_t header, counters, entries, partials, total;
+  size_t header, counters, entries, lse2, partials, total;
 };
 
 // Sum over tiles of the chunk count is at most tiles + total_items / target and the
 // target is at least total_items * kv_heads / (2 * kDkvSlots).
-__host__ inline DkvLayout dkv_layout(int B, int S, int Hkv, int D) {
+__host__ inline DkvLayout dkv_layout(int B, int S, int Hq, int Hkv, int D) {
   DkvLayout L;
   const int tiles = B * (S / kDkvKeys);
   const int extra = (2 * kDkvSlots + Hkv - 1) / Hkv + 1;
@@ -121,7 +121,9 @@ __host__ inline DkvLayout dkv_layout(int B, int S, int Hkv, int D) {
   L.header = 0;
   L.counters = 256;
   L.entries = L.counters + up((size_t)tiles * Hkv * sizeof(int));
-  L.partials = L.entries + up((size_t)L.max_entries * 2 * sizeof(int));
+  // lse * log2(e), head-major [B, Hq, S] (the caller's delta scratch holds delta the same way)
+  L.lse2 = L.entries + up((size_t)L.max_entries * 2 * sizeof(int));
+  L.partials = L.lse2 + up((size_t)B * S * Hq * sizeof(float));
   L.total = L.partials + (size_t)L.max_partials * Hkv * 2 * kDkvKeys * D * sizeof(float);
   return L;
 }

@@ -361,7 +361,7 @@ def _attn_backward(query, key, value, metadata, out, lse, dout, scale):
     dk = torch.empty_like(key)
     dv = torch.empty_like(value)
     delta = torch.empty_like(lse)
-    workspace_bytes = int(_lib.load().ct_attn_bwd_workspace_bytes(batch, sequence, key.shape[2], head_dim))
+    workspace_bytes = int(_lib.load().ct_attn_bwd_workspace_bytes(batch, sequence, query.shape[2], key.shape[2], head_dim))
     workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=query.device)
     args = _lib.AttnBwdArgs(
         q=query.data_ptr(), k=key.data_ptr(), v=value.data_ptr(),

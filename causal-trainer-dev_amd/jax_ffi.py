@@ -87,7 +87,7 @@ def make_efficient_attention():
         has_end = attention_end is not None
         from . import _lib
 
-        scratch = int(_lib.load().ct_attn_bwd_workspace_bytes(q.shape[0], q.shape[1], k.shape[2], q.shape[3]))
+        scratch = int(_lib.load().ct_attn_bwd_workspace_bytes(q.shape[0], q.shape[1], q.shape[2], k.shape[2], q.shape[3]))
         shapes = (jax.ShapeDtypeStruct(q.shape, q.dtype), jax.ShapeDtypeStruct(k.shape, k.dtype),
                   jax.ShapeDtypeStruct(v.shape, v.dtype), jax.ShapeDtypeStruct(lse.shape, jnp.float32),
                   jax.ShapeDtypeStruct((scratch,), jnp.uint8))

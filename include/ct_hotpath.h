@@ -140,7 +140,7 @@ typedef struct ct_attn_bwd_args {
   uint16_t* dq;                 /* bf16 [batch, seq, q_heads, head_dim] */
   uint16_t* dk;                 /* bf16 [batch, seq, kv_heads, head_dim] */
   uint16_t* dv;                 /* bf16 [batch, seq, kv_heads, head_dim] */
-  float* delta;                 /* f32 scratch [batch, seq, q_heads] */
+  float* delta;                 /* f32 scratch, batch * seq * q_heads elements (private layout) */
   void* workspace;              /* scratch, ct_attn_bwd_workspace_bytes(); contents need not be kept */
   size_t workspace_bytes;
   int32_t batch, seq, q_heads, kv_heads, head_dim;
@@ -152,7 +152,8 @@ typedef struct ct_attn_bwd_args {
  * separate workgroups) and the f32 partial sums of such chunks. 0 for an
  * unsupported shape. No reference counterpart (the reference's dK/dV kernel
  * accumulates in its f32 output window, src/kernels/efficient_attention.py:1545-1549). */
-size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t kv_heads, int32_t head_dim);
+size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads,
+                                   int32_t head_dim);
 
 /*
  * dq, dk, dv from the saved (q, k, v, out, lse) and dout. Four launches:

@@ -28,8 +28,8 @@ def test_size_queries_need_no_gpu(ct):
     bins = sum(33 + 4 * ((nrb + pb - 1) // pb) for pb in (2, 4, 8))
     assert library.ct_attn_meta_bytes(4, 4096) == (4 * (nrb * 12 + 2 * nrb + nrb // 4) + bins) * 4
     assert library.ct_attn_meta_bytes(0, 128) == 0
-    assert 0 < library.ct_attn_bwd_workspace_bytes(4, 4096, 8, 128) < 1 << 30
-    assert library.ct_attn_bwd_workspace_bytes(4, 4000, 8, 128) == 0
+    assert 0 < library.ct_attn_bwd_workspace_bytes(4, 4096, 32, 8, 128) < 1 << 30
+    assert library.ct_attn_bwd_workspace_bytes(4, 4000, 32, 8, 128) == 0
     shape = ct._lib.CutceShape(16384, 4096, 128256)
     fwd = library.ct_cutce_fwd_workspace_bytes(ctypes.byref(shape))
     full = library.ct_cutce_bwd_workspace_bytes(ctypes.byref(shape))
