@@ -509,22 +509,37 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
         dp = mfma32(ro.load(CUR * kStage + QdoStage<D>::kDo, 0, ks), ro.load(vpatch_off, 0, ks), dp);
       const bool interior = tile_is_interior(q_uni, q_end_min, my_uni, my_rb * 32 + 31);
       f32x16 prob;
+      if (!interior) {
+        // Masked scores become -inf (their probability is then exactly 0). Written with
+        // bitwise logic and selects only: the per-element tests must not turn into branches.
+        const int seg_k_or_never = seg_k != 0 ? seg_k : -1;  // ids are >= 0
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const int r0 = 8 * qd + 4 * half;  // first of 4 consecutive query rows
+          const i32x4 seg4 = lds_load<i32x4>(stage + QdoStage<D>::kSeg + r0 * 4);
+          i32x4 end4;
+          if (has_end) {
+            end4 = lds_load<i32x4>(stage + QdoStage<D>::kEnd + r0 * 4);
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) end4[e] = qb * kQueryTile + r0 + e;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const bool ok = (seg4[e] == seg_k_or_never) & (key <= end4[e]);
+            s[4 * qd + e] = ok ? s[4 * qd + e] : kNegInf;
+          }
+        }
+      }
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
-        const int r0 = 8 * qd + 4 * half;  // first of 4 consecutive query rows
+        const int r0 = 8 * qd + 4 * half;
         const f32x4 lse4 = lds_load<f32x4>(stage + QdoStage<D>::kLse + r0 * 4);
         const f32x4 del4 = lds_load<f32x4>(stage + QdoStage<D>::kDelta + r0 * 4);
-        i32x4 seg4, end4;
-        if (!interior) {
-          seg4 = lds_load<i32x4>(stage + QdoStage<D>::kSeg + r0 * 4);
-          if (has_end) end4 = lds_load<i32x4>(stage + QdoStage<D>::kEnd + r0 * 4);
-        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = 4 * qd + e;
-          const int visible_end = has_end ? end4[e] : qb * kQueryTile + r0 + e;
-          const bool ok = interior || (seg4[e] == seg_k && seg_k != 0 && key <= visible_end);
-          const float pr = ok ? exp2_fast(fmaf(s[r], kLog2e, -lse4[e])) : 0.f;
+          const float pr = exp2_fast(fmaf(s[r], kLog2e, -lse4[e]));
           prob[r] = pr;
           dp[r] = pr * (dp[r] - del4[e]);
         }
