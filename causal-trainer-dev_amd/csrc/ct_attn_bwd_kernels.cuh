@@ -173,10 +173,17 @@ CT_DEVICE void qdo_commit(lds_addr stage, float scale) {
   }
 }
 
+// Fragment address structures of the dK/dV kernel: the register-lean ones where the tile is
+// wide enough for them (the kernel is at the register limit).
+template <int D>
+using DkvRowFrags = std::conditional_t<(D / 8 >= 16), RowFragCompact<D / 8>, RowFragOffsets<D / 8>>;
+template <int D>
+using DkvTrFrags = std::conditional_t<(D / 8 >= 16), TrFragCompact<D / 8, KSlots::kAccum>,
+                                      TrFragOffsets<D / 8, KSlots::kAccum>>;
+
 // X (32 rows of an LDS tile) times register fragments: C[row, key] = sum_d X[row, d] F[key, d].
 template <int D>
-CT_DEVICE f32x16 rows_times_frags(int tile_off, const RowFragOffsets<D / 8>& ro,
-                                  const bf16x8* frags) {
+CT_DEVICE f32x16 rows_times_frags(int tile_off, const DkvRowFrags<D>& ro, const bf16x8* frags) {
   f32x16 c = zero16();
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) c = mfma32(ro.load(tile_off, 0, ks), frags[ks], c);
@@ -186,8 +193,8 @@ CT_DEVICE f32x16 rows_times_frags(int tile_off, const RowFragOffsets<D / 8>& ro,
 // acc (32 keys x D) += W^T X, W in accumulator layout (rows = the 32 tile rows,
 // cols = keys), X the 32-row LDS tile read transposed.
 template <int D>
-CT_DEVICE void accumulate_keys(int tile_off, const TrFragOffsets<D / 8, KSlots::kAccum>& to,
-                               const f32x16& wt, f32x16* acc) {
+CT_DEVICE void accumulate_keys(int tile_off, const DkvTrFrags<D>& to, const f32x16& wt,
+                               f32x16* acc) {
 #pragma unroll
   for (int step = 0; step < 2; ++step) {
     const bf16x8 aop = pack_acc8(wt, step);
@@ -429,8 +436,8 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   const int b = tile / (nrb / 4), kt = tile % (nrb / 4);
   const int g = p.Hq / p.Hkv;
   const int* meta_b = p.meta + (size_t)b * nrb * kMetaW;
-  const RowFragOffsets<D / 8> ro(lds0);
-  const TrFragOffsets<D / 8, KSlots::kAccum> to(lds0);
+  const DkvRowFrags<D> ro(lds0);
+  const DkvTrFrags<D> to(lds0);
 
   int q_lo = INT_MAX, q_hi = -1;
 #pragma unroll
@@ -459,7 +466,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) {
     kf[ks] = as_bf16x8(load_global16(p.k + kv_off + 16 * ks + 8 * half));
-    lds_store<u32x4>(ro.ptr[ks] + vpatch_off, load_global16(p.v + kv_off + 16 * ks + 8 * half));
+    lds_store<u32x4>(ro.addr(vpatch_off, 0, ks), load_global16(p.v + kv_off + 16 * ks + 8 * half));
   }
   f32x16 dkacc[D / 32], dvacc[D / 32];
 #pragma unroll

@@ -204,8 +204,11 @@ struct RowFragOffsets {
 #pragma unroll
     for (int ks = 0; ks < kSteps; ++ks) ptr[ks] = base + tile_byte_offset<CPR>(row, 2 * ks + half);
   }
+  CT_DEVICE lds_addr addr(int tile_off, int rb, int ks) const {
+    return ptr[ks] + (tile_off + rb * kRowBlockBytes);
+  }
   CT_DEVICE bf16x8 load(int tile_off, int rb, int ks) const {
-    return lds_load<bf16x8>(ptr[ks] + (tile_off + rb * kRowBlockBytes));
+    return lds_load<bf16x8>(addr(tile_off, rb, ks));
   }
 };
 
@@ -243,6 +246,60 @@ struct TrFragOffsets {
     const int off = tile_off + ks * kStepBytes + (cb >> 2) * 256;
     const bf16x4_vs lo = lds_load_tr(ptr[0][cb & 3] + off);
     const bf16x4_vs hi = lds_load_tr(ptr[1][cb & 3] + off);
+    bf16x8 out;
+    out[0] = lo[0]; out[1] = lo[1]; out[2] = lo[2]; out[3] = lo[3];
+    out[4] = hi[0]; out[5] = hi[1]; out[6] = hi[2]; out[7] = hi[3];
+    return out;
+  }
+};
+
+// Register-lean variants of the two structures above for kernels that cannot afford 8 address
+// registers per operand: the swizzle is an XOR of the chunk index with a lane constant, and the
+// chunk index of a fragment is (compile-time constant) XOR (lane constant), so a fragment
+// address is (constant ^ lane term) + lane base: one v_xad_u32 per read instead of a register
+// held for the whole kernel. CPR >= 16 only (the 4-bit swizzle).
+template <int CPR>
+struct RowFragCompact {
+  static_assert(CPR >= 16, "compact offsets need the 4-bit swizzle");
+  static constexpr int kRowBlockBytes = 32 * CPR * 16;
+  lds_addr row_base;  // start of this lane's row
+  unsigned x16;       // (half ^ swizzle(row)) * 16
+  CT_DEVICE explicit RowFragCompact(lds_addr base) {
+    const int l = lane_id(), row = l & 31, half = l >> 5;
+    row_base = base + row * CPR * 16;
+    x16 = (unsigned)((half ^ swizzle<CPR>(row)) << 4);
+  }
+  CT_DEVICE lds_addr addr(int tile_off, int rb, int ks) const {
+    const unsigned chunk_bytes = ((unsigned)(2 * ks) << 4) ^ x16;
+    return row_base + chunk_bytes + (tile_off + rb * kRowBlockBytes);
+  }
+  CT_DEVICE bf16x8 load(int tile_off, int rb, int ks) const {
+    return lds_load<bf16x8>(addr(tile_off, rb, ks));
+  }
+};
+
+template <int CPR, KSlots MAP>
+struct TrFragCompact {
+  static_assert(CPR >= 16, "compact offsets need the 4-bit swizzle");
+  static constexpr int kStepBytes = 16 * CPR * 16;
+  lds_addr row_base[2];  // per read of the pair: row start + the 8-byte half inside the chunk
+  unsigned y16[2];       // ((chunk bits below the column block) ^ swizzle(row)) * 16
+  CT_DEVICE explicit TrFragCompact(lds_addr base) {
+    const int l = lane_id(), p = l & 15, q16 = (l >> 4) & 1, half = l >> 5;
+#pragma unroll
+    for (int second = 0; second < 2; ++second) {
+      const int row = (MAP == KSlots::kNatural ? 8 * half + 4 * second : 4 * half + 8 * second) +
+                      (p >> 2);
+      const int col_low = 16 * q16 + 4 * (p & 3);  // column inside the 32-column block
+      row_base[second] = base + row * CPR * 16 + (col_low & 4) * 2;
+      y16[second] = (unsigned)(((col_low >> 3) ^ swizzle<CPR>(row)) << 4);
+    }
+  }
+  CT_DEVICE bf16x8 load(int tile_off, int ks, int cb) const {
+    const int off = tile_off + ks * kStepBytes + (cb >> 2) * 256;
+    const unsigned block = (unsigned)((cb & 3) * 4) << 4;
+    const bf16x4_vs lo = lds_load_tr(row_base[0] + (block ^ y16[0]) + off);
+    const bf16x4_vs hi = lds_load_tr(row_base[1] + (block ^ y16[1]) + off);
     bf16x8 out;
     out[0] = lo[0]; out[1] = lo[1]; out[2] = lo[2]; out[3] = lo[3];
     out[4] = hi[0]; out[5] = hi[1]; out[6] = hi[2]; out[7] = hi[3];
