@@ -22,3 +22,5 @@ from .cut_cross_entropy import (  # noqa: F401,E402
     cutce_forward,
     pallas_cut_linear_cross_entropy,
 )
+from . import cut_cross_entropy, prep, profiling  # noqa: F401,E402
+from .prep import canonicalize_segment_ids, shifted_targets_and_weights  # noqa: F401,E402

@@ -78,6 +78,16 @@ class CutceBwdArgs(Structure):
     ]
 
 
+class ShiftedTargetsArgs(Structure):
+    _fields_ = [
+        ("input_ids", c_void_p), ("attention_mask", c_void_p), ("segment_ids", c_void_p),
+        ("assistant_mask", c_void_p), ("loss_mask", c_void_p), ("labels", c_void_p),
+        ("targets", c_void_p), ("weights", c_void_p),
+        ("scratch", c_void_p), ("scratch_bytes", c_size_t),
+        ("batch", c_int32), ("seq", c_int32), ("ignore_index", c_int32),
+    ]
+
+
 LAUNCH_HOOK = ctypes.CFUNCTYPE(None, c_void_p, ctypes.c_char_p, c_int32, c_void_p)
 
 # name -> (restype, argtypes); every symbol include/ct_hotpath.h declares.
@@ -86,6 +96,9 @@ SYMBOLS = {
     "ct_last_error": (ctypes.c_char_p, []),
     "ct_abi_version": (c_int32, []),
     "ct_calibration_copy": (c_int32, [c_void_p, c_void_p, c_void_p, c_size_t]),
+    "ct_canonicalize_segment_ids": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
+    "ct_shifted_targets_scratch_bytes": (c_size_t, [c_int32, c_int32]),
+    "ct_shifted_targets_and_weights": (c_int32, [c_void_p, POINTER(ShiftedTargetsArgs)]),
     "ct_attn_meta_bytes": (c_size_t, [c_int32, c_int32]),
     "ct_attn_bwd_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32]),
     "ct_attn_prepare": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),

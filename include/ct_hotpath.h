@@ -170,6 +170,48 @@ int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* args);
 int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16_t* dout,
                       float* delta, int64_t rows, int32_t head_dim);
 
+/* ------------------------------------------------------------------------
+ * Preparation steps directly in front of the hot paths (they define the
+ * ignored-token sets, so they are bit-exact integer kernels)
+ * --------------------------------------------------------------------- */
+
+/*
+ * canonical_ids[b, s] = one-based index of the contiguous valid run that holds
+ * position s, 0 where attention_mask[b, s] == 0. A run starts at a valid
+ * position whose predecessor is invalid or has a different segment id;
+ * segment_ids may be NULL (all zero). int32 [batch, seq] in and out.
+ * Replaces: canonicalize_segment_ids (src/modeling/rotary.py:13-50).
+ */
+int32_t ct_canonicalize_segment_ids(void* stream, const int32_t* attention_mask,
+                                    const int32_t* segment_ids, int32_t batch, int32_t seq,
+                                    int32_t* canonical_ids);
+
+typedef struct ct_shifted_targets_args {
+  const int32_t* input_ids;       /* int32 [batch, seq] */
+  const int32_t* attention_mask;  /* int32 [batch, seq] or NULL (all valid); valid iff == 1 */
+  const int32_t* segment_ids;     /* int32 [batch, seq] or NULL */
+  const int32_t* assistant_mask;  /* int32 [batch, seq] or NULL; counts where != 0 */
+  const float* loss_mask;         /* f32 [batch, seq] or NULL; may be fractional */
+  const int32_t* labels;          /* int32 [batch, seq] or NULL (= input_ids) */
+  int32_t* targets;               /* int32 out [batch, seq - 1]; 0 where the weight is not > 0 */
+  float* weights;                 /* f32 out [batch, seq - 1] */
+  void* scratch;                  /* ct_shifted_targets_scratch_bytes(), only read with segment_ids */
+  size_t scratch_bytes;
+  int32_t batch, seq;
+  int32_t ignore_index;           /* the reference default is -100 */
+} ct_shifted_targets_args;
+
+size_t ct_shifted_targets_scratch_bytes(int32_t batch, int32_t seq);
+
+/*
+ * Shifted next-token targets and their loss weights: an edge s -> s + 1 counts
+ * iff both tokens are valid, the label is not ignore_index and, with segment
+ * ids, both lie in the same canonical run; assistant_mask and loss_mask are
+ * read at the target position. The output feeds ct_cutce_fwd unchanged.
+ * Replaces: _shifted_targets_and_weights (src/training/losses.py:21-85).
+ */
+int32_t ct_shifted_targets_and_weights(void* stream, const ct_shifted_targets_args* args);
+
 /*
  * Measurement aid, no reference counterpart: copies `bytes` (a multiple of 16,
  * both pointers 16-byte aligned) device to device with a plain kernel. Run
