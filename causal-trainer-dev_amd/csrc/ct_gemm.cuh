@@ -26,7 +26,10 @@
 // The choice is uniform over the workgroup.
 #pragma once
 
+#include <type_traits>
+
 #include "ct_common.cuh"
+#include "ct_gemm_asm.inc"
 
 namespace ct {
 
@@ -83,11 +86,13 @@ struct KcLoader {
     }
     fast = aligned && (alias_invalid_rows || m0 + kGemmTile <= rows_valid) && k_valid % kGemmBK == 0;
   }
+  // copies N0 .. N1-1 of the thread's NCH 16-byte slots
+  template <int N0 = 0, int N1 = NCH>
   CT_DEVICE void dma(int k0, lds_addr tile) const {
     const int wave = uniform(threadIdx.x >> 6);
     const char* p = base + (size_t)k0 * 2;
 #pragma unroll
-    for (int n = 0; n < NCH; ++n) dma16_s(p, voff[n], tile + (n * 256 + wave * 64) * 16);
+    for (int n = N0; n < N1; ++n) dma16_s(p, voff[n], tile + (n * 256 + wave * 64) * 16);
   }
   CT_DEVICE void fetch(int k0) {
     const int k = k0 + chunk * 8;
@@ -144,6 +149,8 @@ struct McLoader {
       voff[n] = (unsigned)(((row_index ? 0 : (long)r * ld) + c) * 2);
     }
   }
+  // copies N0 .. N1-1 of the thread's NCH 16-byte slots (N0 even, N1 = N0 + 2 or NCH)
+  template <int N0 = 0, int N1 = NCH>
   CT_DEVICE void dma(int k0, lds_addr tile) const {
     const int wave = uniform(threadIdx.x >> 6);
     if (row_index) {
@@ -151,23 +158,25 @@ struct McLoader {
       // with scalar loads (tracked by lgkmcnt, so they do not force the copies
       // still in flight to drain the way a vector load would).
       typedef int i32x2 __attribute__((ext_vector_type(2)));
-      const int* ip = row_index + k0 + 2 * wave;
-      i32x2 pair[NCH];
-      asm volatile(
-          "s_load_dwordx2 %0, %4, 0x0\n\ts_load_dwordx2 %1, %4, 0x20\n\t"
-          "s_load_dwordx2 %2, %4, 0x40\n\ts_load_dwordx2 %3, %4, 0x60\n\ts_waitcnt lgkmcnt(0)"
-          : "=&s"(pair[0]), "=&s"(pair[1]), "=&s"(pair[2]), "=&s"(pair[3])
-          : "s"(ip)
-          : "memory");
+      const int* ip = row_index + k0 + 2 * wave + 8 * N0;
       const bool upper = lane_id() >= 32;
 #pragma unroll
-      for (int n = 0; n < NCH; ++n)
-        dma16(base + (size_t)(upper ? pair[n][1] : pair[n][0]) * ld * 2 + voff[n],
+      for (int n = N0; n < N1; n += 2) {
+        i32x2 p0, p1;
+        asm volatile(
+            "s_load_dwordx2 %0, %2, 0x0\n\ts_load_dwordx2 %1, %2, 0x20\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(p0), "=&s"(p1)
+            : "s"(ip + 8 * (n - N0))
+            : "memory");
+        dma16(base + (size_t)(upper ? p0[1] : p0[0]) * ld * 2 + voff[n],
               tile + (n * 256 + wave * 64) * 16);
+        dma16(base + (size_t)(upper ? p1[1] : p1[0]) * ld * 2 + voff[n + 1],
+              tile + ((n + 1) * 256 + wave * 64) * 16);
+      }
     } else {
       const char* p = base + (size_t)k0 * ld * 2;
 #pragma unroll
-      for (int n = 0; n < NCH; ++n) dma16_s(p, voff[n], tile + (n * 256 + wave * 64) * 16);
+      for (int n = N0; n < N1; ++n) dma16_s(p, voff[n], tile + (n * 256 + wave * 64) * 16);
     }
   }
   CT_DEVICE void fetch(int k0) {
@@ -226,10 +235,20 @@ CT_DEVICE void mfma_block(const GemmFrags& f, GemmAcc& acc) {
     for (int jn = 0; jn < 4; ++jn) acc.c[i][jn] = mfma32(f.a[i], f.b[jn], acc.c[i][jn]);
 }
 
-// s_waitcnt vmcnt(N) for N in {0, 8, 16} (expcnt / lgkmcnt left at "no wait").
+template <int I0, int I1>
+CT_DEVICE void mfma_rows(const GemmFrags& f, GemmAcc& acc) {
+#pragma unroll
+  for (int i = I0; i < I1; ++i)
+#pragma unroll
+    for (int jn = 0; jn < 4; ++jn) acc.c[i][jn] = mfma32(f.a[i], f.b[jn], acc.c[i][jn]);
+}
+
+// s_waitcnt vmcnt(N) for N in {0, 8, 12, 16} (expcnt / lgkmcnt left at "no wait").
 CT_DEVICE void wait_vmcnt(int outstanding) {
   if (outstanding >= 16)
     __builtin_amdgcn_s_waitcnt(0x0F70 | (1 << 14));  // vmcnt = 16
+  else if (outstanding >= 12)
+    __builtin_amdgcn_s_waitcnt(0x0F70 | 12);
   else if (outstanding >= 8)
     __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
   else
@@ -239,6 +258,43 @@ CT_DEVICE void wait_lds() { __builtin_amdgcn_s_waitcnt(0xC07F); }  // lgkmcnt(0)
 // Execution barrier without the memory fence of __syncthreads() (which would wait for
 // every copy in flight); callers order their own LDS traffic with the waits above.
 CT_DEVICE void workgroup_barrier() { __builtin_amdgcn_s_barrier(); }
+
+// The pipelined main loop with a fixed instruction order (see gen_gemm_asm.py), for an
+// m-contiguous A without row gather, a k-contiguous B and a step count that is a positive
+// multiple of 4. Entered with the copies of steps 0..2 issued and step 0 landed for every
+// wavefront; returns with nothing in flight and the LDS tiles free.
+CT_DEVICE unsigned long long uniform64(const void* p) {
+  const unsigned long long b = (unsigned long long)(uintptr_t)p;
+  const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
+  return ((unsigned long long)hi << 32) | (unsigned long long)lo;
+}
+CT_DEVICE void gemm_loop_scheduled(const McLoader& A, const KcLoader& B, int k_begin, int steps,
+                                   lds_addr smem, const McLoader::FragOffsets& afo,
+                                   const KcLoader::FragOffsets& bfo, int wm, int wn, GemmAcc& acc) {
+  const int wave = uniform(threadIdx.x >> 6);
+  // sources of the copies of step 3
+  const unsigned long long src_a =
+      uniform64(A.base + (size_t)(k_begin + 3 * kGemmBK) * (size_t)A.ld * 2);
+  const unsigned long long src_b = uniform64(B.base + (size_t)(k_begin + 3 * kGemmBK) * 2);
+  const unsigned stride_a = (unsigned)uniform((int)(kGemmBK * A.ld * 2));
+  const unsigned steps_u = (unsigned)uniform(steps);
+  const unsigned lds_wave = (unsigned)uniform((int)(uintptr_t)(smem + wave * 1024));
+  const int a_off = (wm / 128) * 256;
+  const int b_off = GemmSmem::kTileBytes + (wn / 32) * KcLoader::FragOffsets::kRowBlockBytes;
+  asm volatile(CT_GEMM_LOOP
+               : "+a"(acc.c[0][0]), "+a"(acc.c[0][1]), "+a"(acc.c[0][2]), "+a"(acc.c[0][3]),
+                 "+a"(acc.c[1][0]), "+a"(acc.c[1][1]), "+a"(acc.c[1][2]), "+a"(acc.c[1][3]),
+                 "+a"(acc.c[2][0]), "+a"(acc.c[2][1]), "+a"(acc.c[2][2]), "+a"(acc.c[2][3]),
+                 "+a"(acc.c[3][0]), "+a"(acc.c[3][1]), "+a"(acc.c[3][2]), "+a"(acc.c[3][3])
+               : "s"(src_a), "s"(src_b), "s"(stride_a), "s"(steps_u), "s"(lds_wave),
+                 "v"(afo.ptr[0][0] + a_off), "v"(afo.ptr[0][1] + a_off), "v"(afo.ptr[0][2] + a_off),
+                 "v"(afo.ptr[0][3] + a_off), "v"(afo.ptr[1][0] + a_off), "v"(afo.ptr[1][1] + a_off),
+                 "v"(afo.ptr[1][2] + a_off), "v"(afo.ptr[1][3] + a_off), "v"(bfo.ptr[0] + b_off),
+                 "v"(bfo.ptr[1] + b_off), "v"(A.voff[0]), "v"(A.voff[1]), "v"(A.voff[2]),
+                 "v"(A.voff[3]), "v"(B.voff[0]), "v"(B.voff[1]), "v"(B.voff[2]), "v"(B.voff[3])
+               : "memory", "m0", "scc", CT_GEMM_LOOP_CLOBBERS);
+}
 
 // acc += A[m-tile, k_begin:k_end] * B[n-tile, k_begin:k_end]^T. Must be called by
 // all 256 threads; ends with the LDS tiles free for reuse.
@@ -264,24 +320,35 @@ CT_DEVICE void gemm_tile(ALoader& A, BLoader& B, int k_begin, int k_end, lds_add
     }
     wait_vmcnt((min(steps, 3) - 1) * kLoadsPerStep);
     workgroup_barrier();
+    if constexpr (std::is_same<ALoader, McLoader>::value && std::is_same<BLoader, KcLoader>::value) {
+      if (steps % 4 == 0 && !A.row_index) {  // uniform
+        gemm_loop_scheduled(A, B, k_begin, steps, smem, afo, bfo, wm, wn, acc);
+        return;
+      }
+    }
     GemmFrags f0, f1;
     load_frags<ALoader, BLoader>(f0, 0, afo, bfo, 0, wm, wn);
     int stage = 0;
     for (int k = 0; k < steps; ++k) {
-      if (k + 3 < steps) {
-        const int dst = (stage + 3 * kStage) & (kRing - 1);
-        A.dma(k_begin + (k + 3) * BK, smem + dst);
-        B.dma(k_begin + (k + 3) * BK, smem + dst + kTile);
-      }
+      // The copies of step k+3 go into the stage read during step k-1 (free since the
+      // last barrier); the B half is issued between the MFMAs so that a shorter burst of
+      // copies stalls the matrix pipe.
+      const int dst = (stage + 3 * kStage) & (kRing - 1);
+      const int k_next = k_begin + (k + 3) * BK;
+      const bool more = k + 3 < steps;
       load_frags<ALoader, BLoader>(f1, stage, afo, bfo, 1, wm, wn);
-      mfma_block(f0, acc);
+      mfma_rows<0, 1>(f0, acc);
+      if (more) A.dma(k_next, smem + dst);
+      mfma_rows<1, 3>(f0, acc);
+      if (more) B.dma(k_next, smem + dst + kTile);
+      mfma_rows<3, 4>(f0, acc);
       // step k+1 must have landed: at most the copies of steps k+2, k+3 may be in flight
       wait_vmcnt(min(max(steps - k - 2, 0), 2) * kLoadsPerStep);
       wait_lds();  // our reads of this stage are done before anyone recycles it
       workgroup_barrier();
       stage = (stage + kStage) & (kRing - 1);
       if (k + 1 < steps) load_frags<ALoader, BLoader>(f0, stage, afo, bfo, 0, wm, wn);
-      mfma_block(f1, acc);
+      mfma_rows<0, 4>(f1, acc);
     }
     wait_lds();
     __syncthreads();
