@@ -332,6 +332,24 @@ __global__ __launch_bounds__(256) void cutce_zero_rows_kernel(const float* weigh
   for (int c = threadIdx.x; c < d / 8; c += 256) dst[c] = u32x4{0u, 0u, 0u, 0u};
 }
 
+// packed[slot] = hidden[idx[slot]] for the slots of every started 256-slot block. The head
+// gradient contracts over slots; with the rows packed its operand tiles are plain strided
+// copies instead of a gather through idx at every step. (idx repeats the first active row
+// past n_act, so the padding rows hold finite values; their G^T entries are zero.)
+__global__ __launch_bounds__(256) void cutce_pack_rows_kernel(CutceParams p, bf16* packed) {
+  const int slot = blockIdx.x;
+  const int n_act = p.header->n_act;
+  if (slot >= (n_act + kGemmTile - 1) / kGemmTile * kGemmTile) return;
+  const bf16* src = p.hidden + (size_t)p.idx[slot] * p.d;
+  bf16* dst = packed + (size_t)slot * p.d;
+  if (p.hidden_aligned) {
+    for (int c = threadIdx.x; c < p.d / 8; c += 256)
+      reinterpret_cast<u32x4*>(dst)[c] = reinterpret_cast<const u32x4*>(src)[c];
+  } else {
+    for (int c = threadIdx.x; c < p.d; c += 256) dst[c] = src[c];
+  }
+}
+
 // Per-slot constants of the backward: (w dy, lse log2 e, target), zeros / -1 past the active rows.
 struct CutceRowParams {
   float* fac;
@@ -489,9 +507,10 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
     }
 }
 
-// dHead[m, slab0 + v] = sum_slot hidden[idx[slot], m] G^T[v, slot]
-__global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const bf16* G, int slab0,
-                                                          int slab_tiles, bf16* dhead) {
+// dHead[m, slab0 + v] = sum_slot packed[slot, m] G^T[v, slot], packed[slot] = hidden[idx[slot]]
+__global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const bf16* packed,
+                                                          const bf16* G, int slab0, int slab_tiles,
+                                                          bf16* dhead) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr smem = lds_address_of(smem_raw);
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
@@ -501,12 +520,12 @@ __global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const b
   const int mb = id % m_blocks, vt = id / m_blocks;
   const int m0 = mb * kGemmTile, v0 = vt * kGemmTile;  // v0 relative to the slab
   const int n_act = p.header->n_act;
-  const int k_end = min(p.n_pad, (n_act + kBK - 1) / kBK * kBK);
+  // 4 contraction steps at a time; slots n_act .. k_end-1 are valid memory: G^T holds zeros
+  // there (the dlogits kernels write whole 256-slot blocks) and the packed rows are finite.
+  const int k_end = min(p.n_pad, (n_act + 4 * kBK - 1) / (4 * kBK) * (4 * kBK));
 
   McLoader A;
-  // Slots n_act .. k_end-1 are valid memory: G^T holds zeros there (the dlogits kernels
-  // write whole 256-slot blocks) and idx repeats the first active row.
-  A.init(p.hidden, p.d, p.idx, m0, p.d, k_end, p.hidden_aligned);
+  A.init(packed, p.d, nullptr, m0, p.d, k_end, true);
   KcLoader B;
   B.init(G, p.n_pad, nullptr, v0, slab_tiles * kGemmTile, k_end, true, false);
   GemmAcc acc;
@@ -553,12 +572,14 @@ static FwdLayout fwd_layout(const ct_cutce_shape& s) {
 }
 
 struct BwdLayout {
-  size_t header, idx, rowparams, g, acc, total;
+  size_t header, idx, rowparams, packed, g, acc, total;
   int slab_cols;  // multiple of 256
   int slabs;
 };
-static size_t bwd_fixed_bytes(int n_pad) {
-  return align_up(sizeof(CutceHeader), 256) + 4 * align_up((size_t)n_pad * sizeof(int), 256);
+// header, idx, 3 row parameter arrays, packed hidden rows
+static size_t bwd_fixed_bytes(int n_pad, int d) {
+  return align_up(sizeof(CutceHeader), 256) + 4 * align_up((size_t)n_pad * sizeof(int), 256) +
+         align_up((size_t)n_pad * d * sizeof(bf16), 256);
 }
 // Largest slab that fits in `bytes` (0 if even one tile column does not).
 static BwdLayout bwd_layout(const ct_cutce_shape& s, size_t bytes) {
@@ -568,7 +589,8 @@ static BwdLayout bwd_layout(const ct_cutce_shape& s, size_t bytes) {
   L.header = 0;
   L.idx = align_up(sizeof(CutceHeader), 256);
   L.rowparams = L.idx + align_up((size_t)n_pad * sizeof(int), 256);
-  L.g = bwd_fixed_bytes(n_pad);
+  L.packed = L.rowparams + 3 * align_up((size_t)n_pad * sizeof(int), 256);
+  L.g = bwd_fixed_bytes(n_pad, s.hidden);
   const size_t per_tile = (size_t)n_pad * kGemmTile * sizeof(bf16);
   const size_t acc_bytes = align_up((size_t)n_pad * s.hidden * sizeof(float), 256);
   if (bytes >= L.g + per_tile * tiles) {
@@ -629,7 +651,7 @@ extern "C" size_t ct_cutce_logits_cache_bytes(const ct_cutce_shape* shape) {
 extern "C" size_t ct_cutce_bwd_workspace_bytes(const ct_cutce_shape* shape) {
   if (!shape || shape->rows <= 0 || shape->vocab <= 0) return 0;
   const int n_pad = padded_rows(shape->rows);
-  return bwd_fixed_bytes(n_pad) +
+  return bwd_fixed_bytes(n_pad, shape->hidden) +
          (size_t)n_pad * vocab_tile_count(shape->vocab) * kGemmTile * sizeof(bf16);
 }
 
@@ -637,7 +659,8 @@ extern "C" size_t ct_cutce_bwd_workspace_min_bytes(const ct_cutce_shape* shape) 
   if (!shape || shape->rows <= 0 || shape->vocab <= 0) return 0;
   const int n_pad = padded_rows(shape->rows);
   if (vocab_tile_count(shape->vocab) == 1) return ct_cutce_bwd_workspace_bytes(shape);
-  return bwd_fixed_bytes(n_pad) + align_up((size_t)n_pad * shape->hidden * sizeof(float), 256) +
+  return bwd_fixed_bytes(n_pad, shape->hidden) +
+         align_up((size_t)n_pad * shape->hidden * sizeof(float), 256) +
          (size_t)n_pad * kGemmTile * sizeof(bf16);
 }
 
@@ -764,6 +787,13 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
                      rp);
   if ((rc = scope10.done())) return rc;
 
+  bf16* packed = reinterpret_cast<bf16*>(ws + L.packed);
+  if (dhead) {
+    LaunchScope scope12("cutce_pack_rows_kernel", stream);
+    hipLaunchKernelGGL(cutce_pack_rows_kernel, dim3(p.n_pad), dim3(256), 0, stream, p, packed);
+    if ((rc = scope12.done())) return rc;
+  }
+
   const int tiles = vocab_tile_count(p.V);
   const int tiles_per_slab = L.slab_cols / kGemmTile;
   for (int s = 0; s < L.slabs; ++s) {
@@ -789,7 +819,7 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
     if (dhead) {
       LaunchScope scope9("cutce_dhead_kernel", stream);
       hipLaunchKernelGGL(cutce_dhead_kernel, dim3(((p.d + kGemmTile - 1) / kGemmTile) * slab_tiles), dim3(256), smem,
-                         stream, p, G, slab0, slab_tiles, dhead);
+                         stream, p, packed, G, slab0, slab_tiles, dhead);
       if ((rc = scope9.done())) return rc;
     }
   }
