@@ -33,8 +33,63 @@ constexpr float kNegInfF = -__builtin_inff();
 struct CutceHeader {
   int n_act;
   int counter;
-  int xcd_counter[8];  // per-XCD work counters of the statistics kernel
-  int pad[6];
+  // per-XCD work counters: set 0 statistics kernel / hidden gradient, set 1 head gradient
+  int xcd_counter[2][8];
+  int pad[14];
+};
+
+CT_DEVICE void reset_unit_counters(CutceHeader* header) {
+  if (threadIdx.x < 16) (&header->xcd_counter[0][0])[threadIdx.x] = 0;
+}
+
+// Work order of the persistent GEMM kernels. A unit is a pair (a, b) of operand tile indices,
+// a < a_count, b < b_count; every unit is one 256 x 256 GEMM tile (or a run of them) that
+// reads tile a of one operand and tile b of the other. Each XCD has its own L2, so the
+// workgroups of one XCD should work at the same time on units that share operands: the
+// (a, b) grid is walked in blocks of kA x kB = 32 units (the 32 compute units of an XCD: 4 + 8
+// operand tiles feed 32 GEMM tiles), the sequence of blocks is cut into 8 equal ranges, and an
+// XCD takes the units of its range through its own counter. Indices that fall outside the
+// grid (ragged edges) are skipped. An XCD that runs dry helps the next one.
+struct XcdUnits {
+  static constexpr int kA = 4, kB = 8, kXcds = 8;
+  int* counters;
+  int a_count, b_count, b_groups, padded_total, per_xcd, my_xcd;
+  int helping;  // how many XCDs further the counter in use belongs to
+  CT_DEVICE void init(int* counters_, int a_count_, int b_count_) {
+    counters = counters_;
+    a_count = a_count_;
+    b_count = b_count_;
+    b_groups = (b_count + kB - 1) / kB;
+    padded_total = ((a_count + kA - 1) / kA) * b_groups * kA * kB;
+    per_xcd = (padded_total + kXcds - 1) / kXcds;
+    unsigned xcc_id;
+    asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_id));
+    my_xcd = (int)(xcc_id & 7u);
+    helping = 0;
+  }
+  // Called by all threads of the workgroup (contains barriers); false when nothing is left.
+  CT_DEVICE bool next(int& a, int& b, int* lds_slot) {
+    for (;;) {
+      int index = -1;
+      while (helping < kXcds) {
+        const int x = (my_xcd + helping) % kXcds;
+        if (threadIdx.x == 0) *lds_slot = atomicAdd(&counters[x], 1);
+        __syncthreads();
+        const int local = *lds_slot;
+        __syncthreads();
+        if (local < per_xcd && x * per_xcd + local < padded_total) {
+          index = x * per_xcd + local;
+          break;
+        }
+        ++helping;
+      }
+      if (index < 0) return false;
+      const int in_block = index % (kA * kB), block = index / (kA * kB);
+      a = (block / b_groups) * kA + in_block / kB;
+      b = (block % b_groups) * kB + in_block % kB;
+      if (a < a_count && b < b_count) return true;
+    }
+  }
 };
 
 struct CutceParams {
@@ -62,7 +117,7 @@ __global__ __launch_bounds__(1024) void cutce_index_kernel(const float* weights,
       header->n_act = N;
       header->counter = 0;
     }
-    if (tid < 8) header->xcd_counter[tid] = 0;
+    reset_unit_counters(header);
     return;
   }
   int carry = 0;
@@ -89,7 +144,7 @@ __global__ __launch_bounds__(1024) void cutce_index_kernel(const float* weights,
     header->n_act = carry;
     header->counter = 0;
   }
-  if (tid < 8) header->xcd_counter[tid] = 0;
+  reset_unit_counters(header);
 }
 
 // ---------------------------------------------------------------------------
@@ -113,43 +168,12 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
   const int vocab_tiles = (p.V + kGemmTile - 1) / kGemmTile;
   const int n_act = p.header->n_act;
 
-  // Work order. A unit is (vocabulary chunk, row block). Each XCD has its own L2, so the
-  // workgroups of one XCD should work on units that share operands at the same time: the
-  // (chunk, row block) grid is walked in blocks of kChunkGroup x kRowGroup units (32 units = the
-  // 32 compute units of an XCD: 4 head tiles and 8 hidden blocks feed 32 GEMM tiles), the
-  // sequence of blocks is cut into 8 equal ranges, and an XCD takes the units of its range
-  // through its own counter. Indices that fall outside the grid (ragged edges) are skipped.
-  // An XCD that runs dry helps the next one.
-  constexpr int kChunkGroup = 4, kRowGroup = 8, kXcds = 8;
+  // units: (vocabulary chunk, row block)
   const int active_blocks = (n_act + kGemmTile - 1) / kGemmTile;
-  const int row_groups = (active_blocks + kRowGroup - 1) / kRowGroup;
-  const int chunk_groups = (chunks + kChunkGroup - 1) / kChunkGroup;
-  const int padded_total = chunk_groups * row_groups * kChunkGroup * kRowGroup;
-  const int per_xcd = (padded_total + kXcds - 1) / kXcds;
-  unsigned xcc_id;
-  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc_id));
-  const int my_xcd = (int)(xcc_id & 7u);
-  int helping = 0;  // how many XCDs further the counter in use belongs to
-
-  for (;;) {
-    int index = -1;
-    while (helping < kXcds) {
-      const int x = (my_xcd + helping) % kXcds;
-      if (tid == 0) unit_s = atomicAdd(&p.header->xcd_counter[x], 1);
-      __syncthreads();
-      const int local = unit_s;
-      __syncthreads();
-      if (local < per_xcd && x * per_xcd + local < padded_total) {
-        index = x * per_xcd + local;
-        break;
-      }
-      ++helping;
-    }
-    if (index < 0) break;
-    const int in_block = index % (kChunkGroup * kRowGroup), block = index / (kChunkGroup * kRowGroup);
-    const int chunk = (block / row_groups) * kChunkGroup + in_block / kRowGroup;
-    const int rb = (block % row_groups) * kRowGroup + in_block % kRowGroup;
-    if (chunk >= chunks || rb >= active_blocks) continue;
+  XcdUnits units;
+  units.init(p.header->xcd_counter[0], chunks, active_blocks);
+  int chunk, rb;
+  while (units.next(chunk, rb, &unit_s)) {
     const int n0 = rb * kGemmTile;
     const int my_slot = n0 + tid;
     const int active = my_slot < n_act && p.weights[p.idx[my_slot]] != 0.f;
@@ -394,6 +418,8 @@ __global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, Cutce
   const int rb = id % row_blocks, vt = id / row_blocks;
   const int n0 = rb * kGemmTile;
   const int n_act = p.header->n_act;
+  // the two GEMM kernels that follow start from fresh work counters
+  if (blockIdx.x == 0) reset_unit_counters(p.header);
   if (n0 >= n_act) return;  // G^T columns past the active count's block are never read
   const int v0 = slab0 + vt * kGemmTile;
 
@@ -437,6 +463,8 @@ __global__ __launch_bounds__(256) void cutce_dlogits_cached_kernel(CutceParams p
                                                                    bf16* G) {
   const int vrel = blockIdx.x, v = slab0 + vrel;
   const int slot0 = (blockIdx.y * 256 + threadIdx.x) * 8;
+  // the two GEMM kernels that follow start from fresh work counters
+  if (blockIdx.x == 0 && blockIdx.y == 0) reset_unit_counters(p.header);
   const int n_act = p.header->n_act;
   if (slot0 >= (n_act + kGemmTile - 1) / kGemmTile * kGemmTile) return;
   bf16x8 out;
@@ -472,39 +500,43 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
   const lds_addr smem = lds_address_of(smem_raw);
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
-  const int row_blocks = p.n_pad / kGemmTile, col_blocks = (p.d + kGemmTile - 1) / kGemmTile;
-  int id = xcd_remap(blockIdx.x, row_blocks * col_blocks);
-  const int cb = id % col_blocks, rb = id / col_blocks;
-  const int n0 = rb * kGemmTile, c0 = cb * kGemmTile;
+  const int col_blocks = (p.d + kGemmTile - 1) / kGemmTile;
   const int n_act = p.header->n_act;
-  if (n0 >= n_act) return;
+  __shared__ int unit_s;
+  // units: (row block, column block) over the started row blocks
+  XcdUnits units;
+  units.init(p.header->xcd_counter[0], (n_act + kGemmTile - 1) / kGemmTile, col_blocks);
+  int rb, cb;
+  while (units.next(rb, cb, &unit_s)) {
+    const int n0 = rb * kGemmTile, c0 = cb * kGemmTile;
+    McLoader A;
+    A.init(G, p.n_pad, nullptr, n0, p.n_pad, slab_width, true);
+    KcLoader B;
+    B.init(p.head + slab0, p.V, nullptr, c0, p.d, min(slab_width, p.V - slab0), p.head_aligned,
+           false);
+    GemmAcc acc;
+    acc.clear();
+    gemm_tile(A, B, 0, slab_width, smem, acc);
 
-  McLoader A;
-  A.init(G, p.n_pad, nullptr, n0, p.n_pad, slab_width, true);
-  KcLoader B;
-  B.init(p.head + slab0, p.V, nullptr, c0, p.d, min(slab_width, p.V - slab0), p.head_aligned, false);
-  GemmAcc acc;
-  acc.clear();
-  gemm_tile(A, B, 0, slab_width, smem, acc);
-
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int slot = n0 + wm + 32 * i + acc_row(r, half);
-      if (slot >= n_act) continue;
-      const long row = p.idx[slot];
+      for (int r = 0; r < 16; ++r) {
+        const int slot = n0 + wm + 32 * i + acc_row(r, half);
+        if (slot >= n_act) continue;
+        const long row = p.idx[slot];
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb) {
-        const int col = c0 + wn + 32 * nb + j;
-        if (col >= p.d) continue;
-        float val = acc.c[i][nb][r];
-        float* a = dh_acc + (size_t)slot * p.d + col;
-        if (mode >= 2) val += *a;
-        if (mode == 1 || mode == 2) *a = val;
-        if (mode == 0 || mode == 3) dhidden[row * p.d + col] = (bf16)val;
+        for (int nb = 0; nb < 4; ++nb) {
+          const int col = c0 + wn + 32 * nb + j;
+          if (col >= p.d) continue;
+          float val = acc.c[i][nb][r];
+          float* a = dh_acc + (size_t)slot * p.d + col;
+          if (mode >= 2) val += *a;
+          if (mode == 1 || mode == 2) *a = val;
+          if (mode == 0 || mode == 3) dhidden[row * p.d + col] = (bf16)val;
+        }
       }
-    }
+  }
 }
 
 // dHead[m, slab0 + v] = sum_slot packed[slot, m] G^T[v, slot], packed[slot] = hidden[idx[slot]]
@@ -516,34 +548,38 @@ __global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const b
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
   const int m_blocks = (p.d + kGemmTile - 1) / kGemmTile;
-  int id = xcd_remap(blockIdx.x, m_blocks * slab_tiles);
-  const int mb = id % m_blocks, vt = id / m_blocks;
-  const int m0 = mb * kGemmTile, v0 = vt * kGemmTile;  // v0 relative to the slab
   const int n_act = p.header->n_act;
   // 4 contraction steps at a time; slots n_act .. k_end-1 are valid memory: G^T holds zeros
   // there (the dlogits kernels write whole 256-slot blocks) and the packed rows are finite.
   const int k_end = min(p.n_pad, (n_act + 4 * kBK - 1) / (4 * kBK) * (4 * kBK));
+  __shared__ int unit_s;
+  // units: (vocabulary tile of the slab, hidden column block)
+  XcdUnits units;
+  units.init(p.header->xcd_counter[1], slab_tiles, m_blocks);
+  int vt, mb;
+  while (units.next(vt, mb, &unit_s)) {
+    const int m0 = mb * kGemmTile, v0 = vt * kGemmTile;  // v0 relative to the slab
+    McLoader A;
+    A.init(packed, p.d, nullptr, m0, p.d, k_end, true);
+    KcLoader B;
+    B.init(G, p.n_pad, nullptr, v0, slab_tiles * kGemmTile, k_end, true, false);
+    GemmAcc acc;
+    acc.clear();
+    gemm_tile(A, B, 0, k_end, smem, acc);
 
-  McLoader A;
-  A.init(packed, p.d, nullptr, m0, p.d, k_end, true);
-  KcLoader B;
-  B.init(G, p.n_pad, nullptr, v0, slab_tiles * kGemmTile, k_end, true, false);
-  GemmAcc acc;
-  acc.clear();
-  gemm_tile(A, B, 0, k_end, smem, acc);
-
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int m = m0 + wm + 32 * i + acc_row(r, half);
-      if (m >= p.d) continue;
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm + 32 * i + acc_row(r, half);
+        if (m >= p.d) continue;
 #pragma unroll
-      for (int nb = 0; nb < 4; ++nb) {
-        const int v = slab0 + v0 + wn + 32 * nb + j;
-        if (v < p.V) dhead[(size_t)m * p.V + v] = (bf16)acc.c[i][nb][r];
+        for (int nb = 0; nb < 4; ++nb) {
+          const int v = slab0 + v0 + wn + 32 * nb + j;
+          if (v < p.V) dhead[(size_t)m * p.V + v] = (bf16)acc.c[i][nb][r];
+        }
       }
-    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -787,6 +823,7 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
                      rp);
   if ((rc = scope10.done())) return rc;
 
+  const int cus = device_cu_count();
   bf16* packed = reinterpret_cast<bf16*>(ws + L.packed);
   if (dhead) {
     LaunchScope scope12("cutce_pack_rows_kernel", stream);
@@ -813,12 +850,13 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
     }
     const int mode = L.slabs == 1 ? 0 : (s == 0 ? 1 : (s == L.slabs - 1 ? 3 : 2));
     LaunchScope scope8("cutce_dhidden_kernel", stream);
-    hipLaunchKernelGGL(cutce_dhidden_kernel, dim3(row_blocks * ((p.d + kGemmTile - 1) / kGemmTile)), dim3(256), smem,
+    const int col_blocks = (p.d + kGemmTile - 1) / kGemmTile;
+    hipLaunchKernelGGL(cutce_dhidden_kernel, dim3(min(cus, row_blocks * col_blocks)), dim3(256), smem,
                        stream, p, G, slab0, slab_width, mode, dh_acc, dhidden);
     if ((rc = scope8.done())) return rc;
     if (dhead) {
       LaunchScope scope9("cutce_dhead_kernel", stream);
-      hipLaunchKernelGGL(cutce_dhead_kernel, dim3(((p.d + kGemmTile - 1) / kGemmTile) * slab_tiles), dim3(256), smem,
+      hipLaunchKernelGGL(cutce_dhead_kernel, dim3(min(cus, col_blocks * slab_tiles)), dim3(256), smem,
                          stream, p, packed, G, slab0, slab_tiles, dhead);
       if ((rc = scope9.done())) return rc;
     }
