@@ -88,6 +88,16 @@ class ShiftedTargetsArgs(Structure):
     ]
 
 
+class RotaryArgs(Structure):
+    _fields_ = [
+        ("q_in", c_void_p), ("k_in", c_void_p), ("q_out", c_void_p), ("k_out", c_void_p),
+        ("cosine", c_void_p), ("sine", c_void_p), ("tokens", c_int64),
+        ("q_heads", c_int32), ("kv_heads", c_int32), ("head_dim", c_int32),
+        ("rotary_pairs", c_int32), ("rope_style", c_int32), ("inverse", c_int32),
+        ("q_scale", ctypes.c_float),
+    ]
+
+
 LAUNCH_HOOK = ctypes.CFUNCTYPE(None, c_void_p, ctypes.c_char_p, c_int32, c_void_p)
 
 # name -> (restype, argtypes); every symbol include/ct_hotpath.h declares.
@@ -99,6 +109,14 @@ SYMBOLS = {
     "ct_canonicalize_segment_ids": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "ct_shifted_targets_scratch_bytes": (c_size_t, [c_int32, c_int32]),
     "ct_shifted_targets_and_weights": (c_int32, [c_void_p, POINTER(ShiftedTargetsArgs)]),
+    "ct_position_ids": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
+    "ct_rotary_cos_sin": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p, c_void_p]),
+    "ct_apply_rotary": (c_int32, [c_void_p, POINTER(RotaryArgs)]),
+    "ct_rms_norm_fwd": (c_int32, [c_void_p, c_void_p, c_void_p, ctypes.c_float, c_int64, c_int32,
+                                  c_void_p, c_void_p]),
+    "ct_rms_norm_bwd_workspace_bytes": (c_size_t, [c_int32]),
+    "ct_rms_norm_bwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, ctypes.c_float, c_int64,
+                                  c_int32, c_void_p, c_void_p, c_void_p, c_size_t]),
     "ct_attn_meta_bytes": (c_size_t, [c_int32, c_int32]),
     "ct_attn_bwd_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32]),
     "ct_attn_prepare": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),

@@ -212,6 +212,76 @@ size_t ct_shifted_targets_scratch_bytes(int32_t batch, int32_t seq);
  */
 int32_t ct_shifted_targets_and_weights(void* stream, const ct_shifted_targets_args* args);
 
+/* ------------------------------------------------------------------------
+ * Decoder-layer neighbours of the attention operator (single HBM passes)
+ * --------------------------------------------------------------------- */
+
+/*
+ * position_ids[b, s] = distance of s from the start of its run of equal
+ * canonical ids, 0 where attention_mask[b, s] == 0. canonical_ids are the
+ * output of ct_canonicalize_segment_ids. int32 [batch, seq] in and out.
+ * Replaces: _make_position_ids_precanonicalized (src/modeling/rotary.py:82-110).
+ */
+int32_t ct_position_ids(void* stream, const int32_t* attention_mask, const int32_t* canonical_ids,
+                        int32_t batch, int32_t seq, int32_t* position_ids);
+
+/*
+ * cosine / sine [tokens, rotary_pairs] bf16 of f32(position) * inv_freq,
+ * evaluated in f32 and rounded once; no maximum-position cache.
+ * Replaces: rotary_cos_sin (src/modeling/rotary.py:132-157) with dtype bf16.
+ */
+int32_t ct_rotary_cos_sin(void* stream, const int32_t* position_ids, const float* inv_freq,
+                          int64_t tokens, int32_t rotary_pairs, uint16_t* cosine, uint16_t* sine);
+
+enum { CT_ROPE_GPT_J = 0 /* pairs (2i, 2i+1) */, CT_ROPE_GPT_NEOX = 1 /* pairs (i, i + R/2) */ };
+
+typedef struct ct_rotary_args {
+  const uint16_t* q_in;    /* bf16 [tokens, q_heads, head_dim] */
+  const uint16_t* k_in;    /* bf16 [tokens, kv_heads, head_dim] */
+  uint16_t* q_out;         /* may alias q_in */
+  uint16_t* k_out;         /* may alias k_in */
+  const uint16_t* cosine;  /* bf16 [tokens, rotary_pairs] */
+  const uint16_t* sine;
+  int64_t tokens;          /* batch * seq */
+  int32_t q_heads, kv_heads, head_dim;
+  int32_t rotary_pairs;    /* rotary_dim / 2; channels past rotary_dim pass through */
+  int32_t rope_style;      /* CT_ROPE_GPT_J (the reference default) or CT_ROPE_GPT_NEOX */
+  int32_t inverse;         /* 0: rotate (forward); 1: rotate back (gradients of q, k) */
+  float q_scale;           /* 1.0: none. Otherwise Q is also multiplied by bf16(q_scale) in
+                              bf16, after the rotation (forward) or before it (inverse):
+                              the pre-scale of src/modeling/attention.py:124, so that the
+                              attention operator can then be called with scale 1 */
+} ct_rotary_args;
+
+/*
+ * Partial rotary embedding of Q and K from precomputed tables. The rotation is
+ * evaluated in f32 from the bf16 operands and rounded once to bf16.
+ * Supported: head_dim % 8 == 0, rotary_dim % 16 == 0, rotary_dim <= head_dim.
+ * Replaces: apply_rotary_cos_sin (src/modeling/rotary.py:160-204) and its
+ * transpose under autodiff.
+ */
+int32_t ct_apply_rotary(void* stream, const ct_rotary_args* args);
+
+/*
+ * y = bf16(bf16(x * r) * scale), r = 1 / sqrt(mean(x^2) + eps) with f32
+ * statistics; x, y bf16 [rows, hidden], scale bf16 [hidden]; rstd (f32 [rows])
+ * may be NULL. hidden % 8 == 0.
+ * Replaces: rms_norm (src/modeling/architecture.py:155-162) with compute dtype bf16.
+ */
+int32_t ct_rms_norm_fwd(void* stream, const uint16_t* x, const uint16_t* scale, float eps,
+                        int64_t rows, int32_t hidden, uint16_t* y, float* rstd);
+
+size_t ct_rms_norm_bwd_workspace_bytes(int32_t hidden);
+
+/*
+ * Gradients of ct_rms_norm_fwd: dx bf16 [rows, hidden], dscale f32 [hidden]
+ * (summed over rows in a fixed order). hidden in {512, 1024, 2048, 4096, 8192}.
+ * Replaces: the autodiff transpose of rms_norm (src/modeling/architecture.py:155-162).
+ */
+int32_t ct_rms_norm_bwd(void* stream, const uint16_t* x, const uint16_t* scale, const uint16_t* dy,
+                        float eps, int64_t rows, int32_t hidden, uint16_t* dx, float* dscale,
+                        void* workspace, size_t workspace_bytes);
+
 /*
  * Measurement aid, no reference counterpart: copies `bytes` (a multiple of 16,
  * both pointers 16-byte aligned) device to device with a plain kernel. Run
