@@ -35,6 +35,7 @@ def parse_args():
     parser.add_argument("--cutce-steps", type=int, default=None, help="default: min(steps, 5)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-cutce", action="store_true")
+    parser.add_argument("--no-layer-ops", action="store_true")
     parser.add_argument("--calibration-copy-bytes", type=int, default=0,
                         help="also launch one plain device copy of this many bytes (for scaling "
                              "FETCH_SIZE / WRITE_SIZE when the run is under rocprofv3 --pmc)")
@@ -173,6 +174,65 @@ def bench_cutce(ct, torch, steps, warmup, logits_cache=True):
     }
 
 
+def bench_layer_ops(ct, torch, steps, warmup):
+    """The HBM-bound neighbours of attention at the same shape: RoPE of Q and K (partial rotary 0.5,
+    fused Q pre-scale) forward and transpose, RMSNorm forward and backward on [B*S, 4096]."""
+    W = ct.workloads
+    config = W.ATTENTION_CONFIGS["llama3_8b"]
+    tokens = config.batch * config.seq
+    hidden = config.q_heads * config.head_dim
+    g = torch.Generator(device="cuda").manual_seed(7)
+    q = torch.randn((config.batch, config.seq, config.q_heads, config.head_dim), generator=g, device="cuda").bfloat16()
+    k = torch.randn((config.batch, config.seq, config.kv_heads, config.head_dim), generator=g, device="cuda").bfloat16()
+    x = torch.randn((tokens, hidden), generator=g, device="cuda").bfloat16()
+    dy = torch.randn((tokens, hidden), generator=g, device="cuda").bfloat16()
+    scale = torch.ones(hidden, device="cuda").bfloat16()
+    positions = torch.arange(config.seq, device="cuda", dtype=torch.int32).repeat(config.batch, 1)
+    rotary_dim = config.head_dim // 2
+    inv_freq = 1.0 / (500000.0 ** (torch.arange(0, rotary_dim, 2, device="cuda", dtype=torch.float32) / rotary_dim))
+    cosine, sine = ct.rotary_cos_sin(positions, inv_freq)
+    lib, L = ct._lib.load(), ct._lib
+    q_out, k_out, y, dx = torch.empty_like(q), torch.empty_like(k), torch.empty_like(x), torch.empty_like(x)
+    dscale = torch.empty(hidden, dtype=torch.float32, device="cuda")
+    workspace = torch.empty(lib.ct_rms_norm_bwd_workspace_bytes(hidden), dtype=torch.uint8, device="cuda")
+
+    def rotary(inverse):
+        args = L.RotaryArgs(q_in=q.data_ptr(), k_in=k.data_ptr(), q_out=q_out.data_ptr(), k_out=k_out.data_ptr(),
+                            cosine=cosine.data_ptr(), sine=sine.data_ptr(), tokens=tokens, q_heads=config.q_heads,
+                            kv_heads=config.kv_heads, head_dim=config.head_dim, rotary_pairs=rotary_dim // 2,
+                            rope_style=0, inverse=inverse, q_scale=config.scale)
+        L.check(lib.ct_apply_rotary(L.current_stream(), args))
+
+    def step():
+        rotary(0)
+        rotary(1)
+        L.check(lib.ct_rms_norm_fwd(L.current_stream(), x.data_ptr(), scale.data_ptr(), 1e-6, tokens, hidden,
+                                    y.data_ptr(), None))
+        L.check(lib.ct_rms_norm_bwd(L.current_stream(), x.data_ptr(), scale.data_ptr(), dy.data_ptr(), 1e-6, tokens,
+                                    hidden, dx.data_ptr(), dscale.data_ptr(), workspace.data_ptr(), workspace.numel()))
+
+    _, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
+    qk_bytes = 2 * (q.numel() + k.numel()) * 2 + 2 * cosine.numel() * 2   # read + write Q, K; read both tables
+    algorithmic_bytes = {
+        "apply_rotary_kernel": qk_bytes,
+        "rms_norm_fwd_kernel": 2 * x.numel() * 2,
+        "rms_norm_bwd_kernel": 3 * x.numel() * 2 + workspace.numel(),
+    }
+    table = []
+    for name, durations in kernels.items():
+        entry = {"kernel": name, "launches": len(durations), "avg_ms": mean(durations)}
+        if name in algorithmic_bytes:
+            gbps = algorithmic_bytes[name] / (entry["avg_ms"] * 1e-3) / 1e9
+            entry.update({"algorithmic_bytes": algorithmic_bytes[name], "algorithmic_gbps": gbps,
+                          "frac_of_hbm_peak": gbps / PEAK_HBM_GBPS})
+        table.append(entry)
+    return {
+        "workload": "RoPE of Q [4,4096,32,128] and K [4,4096,8,128] (rotary_dim 64, gpt-j, fused Q scale) forward "
+                    "and transpose; RMSNorm forward and backward on [16384, 4096]; bf16",
+        "kernels": table,
+    }
+
+
 def cpu_baseline(ct, torch, attention):
     """The oracle (a port of the reference's pure JAX path) on the host cores, bounded sample."""
 
@@ -279,6 +339,8 @@ def main():
         cut_steps = args.cutce_steps or min(args.steps, 5)
         result["cutce"] = bench_cutce(ct, torch, cut_steps, min(args.warmup, 2),
                                       logits_cache=not args.cutce_recompute)
+    if not args.no_layer_ops:
+        result["layer_ops"] = bench_layer_ops(ct, torch, args.steps, args.warmup)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(ct, torch, attention)
     print(json.dumps(result))

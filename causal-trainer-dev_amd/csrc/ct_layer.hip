@@ -272,13 +272,33 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const uint16_t* x, co
     for (int e = 0; e < 8; ++e) prow[(lane + 64 * i) * 8 + e] = acc[i][e];
 }
 
-__global__ __launch_bounds__(256) void rms_norm_dscale_kernel(const float* partial, int waves, int d,
-                                                              float* dscale) {
-  const int col = blockIdx.x * 256 + threadIdx.x;
-  if (col >= d) return;
-  float s = 0.f;
-  for (int wv = 0; wv < waves; ++wv) s += partial[(size_t)wv * d + col];
-  dscale[col] = s;
+// dscale[col] = sum of the wavefronts' partial rows in a fixed order: thread (c, g) adds the rows
+// of sixteenth g for column 64 blockIdx.x + c (four independent chains, joined in order), then the
+// sixteen group sums are added in order.
+__global__ __launch_bounds__(1024) void rms_norm_dscale_kernel(const float* partial, int waves, int d,
+                                                               float* dscale) {
+  __shared__ float group[16][64];
+  const int c = threadIdx.x & 63, g = threadIdx.x >> 6;
+  const int col = blockIdx.x * 64 + c;
+  const int per = waves / 16;  // a multiple of 4
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  if (col < d) {
+    const float* p = partial + (size_t)g * per * d + col;
+    for (int i = 0; i < per; i += 4) {
+      s0 += p[(size_t)i * d];
+      s1 += p[(size_t)(i + 1) * d];
+      s2 += p[(size_t)(i + 2) * d];
+      s3 += p[(size_t)(i + 3) * d];
+    }
+  }
+  group[g][c] = (s0 + s1) + (s2 + s3);
+  __syncthreads();
+  if (g == 0 && col < d) {
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) s += group[k][c];
+    dscale[col] = s;
+  }
 }
 
 constexpr int kNormBwdBlocks = 512;  // 2048 wavefronts, 8 per compute unit
@@ -392,7 +412,8 @@ extern "C" int32_t ct_rms_norm_bwd(void* stream_, const uint16_t* x, const uint1
   int rc = scope.done();
   if (rc) return rc;
   LaunchScope scope2("rms_norm_dscale_kernel", stream);
-  hipLaunchKernelGGL(rms_norm_dscale_kernel, dim3((hidden + 255) / 256), dim3(256), 0, stream, partial,
+  static_assert(kNormBwdBlocks * 4 % 64 == 0, "dscale kernel splits the partial rows 16 x 4 ways");
+  hipLaunchKernelGGL(rms_norm_dscale_kernel, dim3((hidden + 63) / 64), dim3(1024), 0, stream, partial,
                      kNormBwdBlocks * 4, hidden, dscale);
   return scope2.done();
 }
