@@ -211,12 +211,33 @@ def bench_layer_ops(ct, torch, steps, warmup):
         L.check(lib.ct_rms_norm_bwd(L.current_stream(), x.data_ptr(), scale.data_ptr(), dy.data_ptr(), 1e-6, tokens,
                                     hidden, dx.data_ptr(), dscale.data_ptr(), workspace.data_ptr(), workspace.numel()))
 
+    # logits-level sparse CE at the cut-CE shape (N=16384, V=128256, 30% of the rows ignored)
+    ce = W.CUTCE_CONFIGS["llama3_8b_head"]
+    logits = torch.randn((ce.rows, ce.vocab), generator=g, device="cuda").bfloat16()
+    ce_targets = torch.randint(0, ce.vocab, (ce.rows,), generator=g, device="cuda", dtype=torch.int32)
+    ce_weights = (torch.rand((ce.rows,), generator=g, device="cuda") >= 0.3).float()
+    counted = int((ce_weights != 0).sum())
+    loss, lse = torch.empty(ce.rows, device="cuda"), torch.empty(ce.rows, device="cuda")
+    dy_rows = torch.ones(ce.rows, device="cuda")
+    dlogits = torch.empty_like(logits)
+    ce_args = L.SparseCeArgs(logits=logits.data_ptr(), targets=ce_targets.data_ptr(), weights=ce_weights.data_ptr(),
+                             rows=ce.rows, vocab=ce.vocab, logits_dtype=0, ignore_index=-100)
+    attention_step = step
+
+    def step():
+        attention_step()
+        L.check(lib.ct_sparse_ce_fwd(L.current_stream(), ce_args, loss.data_ptr(), lse.data_ptr()))
+        L.check(lib.ct_sparse_ce_bwd(L.current_stream(), ce_args, lse.data_ptr(), dy_rows.data_ptr(),
+                                     dlogits.data_ptr()))
+
     _, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
     qk_bytes = 2 * (q.numel() + k.numel()) * 2 + 2 * cosine.numel() * 2   # read + write Q, K; read both tables
     algorithmic_bytes = {
         "apply_rotary_kernel": qk_bytes,
         "rms_norm_fwd_kernel": 2 * x.numel() * 2,
         "rms_norm_bwd_kernel": 3 * x.numel() * 2 + workspace.numel(),
+        "sparse_ce_fwd_kernel": counted * ce.vocab * 2,                      # ignored rows are not read
+        "sparse_ce_bwd_kernel": (counted + ce.rows) * ce.vocab * 2,          # ... but their gradient is written
     }
     table = []
     for name, durations in kernels.items():
@@ -228,7 +249,8 @@ def bench_layer_ops(ct, torch, steps, warmup):
         table.append(entry)
     return {
         "workload": "RoPE of Q [4,4096,32,128] and K [4,4096,8,128] (rotary_dim 64, gpt-j, fused Q scale) forward "
-                    "and transpose; RMSNorm forward and backward on [16384, 4096]; bf16",
+                    "and transpose; RMSNorm forward and backward on [16384, 4096]; sparse CE on logits [16384, 128256] "
+                    "with 30% of the rows ignored; bf16",
         "kernels": table,
     }
 

@@ -22,7 +22,8 @@ from .cut_cross_entropy import (  # noqa: F401,E402
     cutce_forward,
     pallas_cut_linear_cross_entropy,
 )
-from . import cut_cross_entropy, layer_ops, prep, profiling  # noqa: F401,E402
+from . import cut_cross_entropy, layer_ops, prep, profiling, sparse_cross_entropy  # noqa: F401,E402
+from .sparse_cross_entropy import pallas_fused_sparse_cross_entropy  # noqa: F401,E402
 from .prep import canonicalize_segment_ids, shifted_targets_and_weights  # noqa: F401,E402
 from .layer_ops import (  # noqa: F401,E402
     apply_rotary_cos_sin, apply_rotary_embedding, make_position_ids, rms_norm, rotary_cos_sin,

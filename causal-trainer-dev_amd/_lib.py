@@ -98,6 +98,13 @@ class RotaryArgs(Structure):
     ]
 
 
+class SparseCeArgs(Structure):
+    _fields_ = [
+        ("logits", c_void_p), ("targets", c_void_p), ("weights", c_void_p), ("rows", c_int64),
+        ("vocab", c_int32), ("logits_dtype", c_int32), ("ignore_index", c_int32),
+    ]
+
+
 LAUNCH_HOOK = ctypes.CFUNCTYPE(None, c_void_p, ctypes.c_char_p, c_int32, c_void_p)
 
 # name -> (restype, argtypes); every symbol include/ct_hotpath.h declares.
@@ -117,6 +124,8 @@ SYMBOLS = {
     "ct_rms_norm_bwd_workspace_bytes": (c_size_t, [c_int32]),
     "ct_rms_norm_bwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, ctypes.c_float, c_int64,
                                   c_int32, c_void_p, c_void_p, c_void_p, c_size_t]),
+    "ct_sparse_ce_fwd": (c_int32, [c_void_p, POINTER(SparseCeArgs), c_void_p, c_void_p]),
+    "ct_sparse_ce_bwd": (c_int32, [c_void_p, POINTER(SparseCeArgs), c_void_p, c_void_p, c_void_p]),
     "ct_attn_meta_bytes": (c_size_t, [c_int32, c_int32]),
     "ct_attn_bwd_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32]),
     "ct_attn_prepare": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),

@@ -17,7 +17,7 @@ from pathlib import Path
 PACKAGE_DIR = Path(__file__).resolve().parent
 CSRC = PACKAGE_DIR / "csrc"
 LIBRARY = PACKAGE_DIR / "libct_hotpath.so"
-SOURCES = ("ct_error.hip", "ct_attn.hip", "ct_cutce.hip", "ct_prep.hip", "ct_layer.hip")
+SOURCES = ("ct_error.hip", "ct_attn.hip", "ct_cutce.hip", "ct_prep.hip", "ct_layer.hip", "ct_logits_ce.hip")
 
 # -packed-fp32-ops is switched off on purpose: hipcc must not form packed FP32
 # instructions from scalar float code on this target.

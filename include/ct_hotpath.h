@@ -282,6 +282,40 @@ int32_t ct_rms_norm_bwd(void* stream, const uint16_t* x, const uint16_t* scale, 
                         float eps, int64_t rows, int32_t hidden, uint16_t* dx, float* dscale,
                         void* workspace, size_t workspace_bytes);
 
+/* ------------------------------------------------------------------------
+ * Sparse cross-entropy on materialised logits (the non-fused loss backend)
+ * --------------------------------------------------------------------- */
+
+enum { CT_DTYPE_BF16 = 0, CT_DTYPE_F32 = 1 };
+
+typedef struct ct_sparse_ce_args {
+  const void* logits;      /* [rows, vocab], row-major, bf16 or f32 */
+  const int32_t* targets;  /* int32 [rows] */
+  const float* weights;    /* f32 [rows] */
+  int64_t rows;
+  int32_t vocab;
+  int32_t logits_dtype;    /* CT_DTYPE_BF16 or CT_DTYPE_F32 */
+  int32_t ignore_index;    /* the reference passes -100 */
+} ct_sparse_ce_args;
+
+/*
+ * loss[r] = weights[r] * (logsumexp(logits[r, :]) - logits[r, targets[r]]) and
+ * lse[r] = logsumexp(logits[r, :]) in f32 on rows with targets[r] != ignore_index
+ * and weights[r] != 0; both 0 on the other rows (which are not read). A target
+ * outside [0, vocab) on a counted row contributes a target logit of 0.
+ * Replaces: _replicated_loss_and_lse / _ce_stats_pallas
+ * (src/kernels/cross_entropy.py:99-251, :400-420).
+ */
+int32_t ct_sparse_ce_fwd(void* stream, const ct_sparse_ce_args* args, float* loss, float* lse);
+
+/*
+ * dlogits[r, v] = weights[r] * dy[r] * (exp(logits[r, v] - lse[r]) - [v == targets[r]])
+ * on counted rows, 0 elsewhere, in the logits dtype; dy f32 [rows].
+ * Replaces: _ce_bwd_pallas (src/kernels/cross_entropy.py:254-397).
+ */
+int32_t ct_sparse_ce_bwd(void* stream, const ct_sparse_ce_args* args, const float* lse,
+                         const float* dy, void* dlogits);
+
 /*
  * Measurement aid, no reference counterpart: copies `bytes` (a multiple of 16,
  * both pointers 16-byte aligned) device to device with a plain kernel. Run

@@ -131,6 +131,39 @@ def xla_sparse_cross_entropy_vjp(logits, targets, weights, cotangent):
     return ((prob - onehot) * factor).to(logits.dtype)
 
 
+def pallas_sparse_cross_entropy(logits, targets, weights, *, ignore_index: int = -100):
+    """(loss, lse) per row as the streaming kernel defines them (src/causal_trainer/kernels/
+    cross_entropy.py:99-190, :400-420): rows with target == ignore_index or weight == 0 give 0 for
+    both; on the other rows a target outside the vocabulary contributes a target logit of 0."""
+
+    compute = logits.float()
+    targets = torch.as_tensor(targets).long()
+    weights = torch.as_tensor(weights).float()
+    valid = (targets != ignore_index) & (weights != 0)
+    lse = torch.logsumexp(compute, dim=-1)
+    inside = (targets >= 0) & (targets < logits.shape[-1])
+    picked = compute.gather(-1, targets.clamp(0, logits.shape[-1] - 1)[..., None])[..., 0]
+    target_logit = torch.where(inside, picked, torch.zeros_like(picked))
+    zero = torch.zeros_like(lse)
+    return torch.where(valid, weights * (lse - target_logit), zero), torch.where(valid, lse, zero)
+
+
+def pallas_sparse_cross_entropy_vjp(logits, targets, weights, cotangent, *, ignore_index: int = -100):
+    """Logits cotangent of the streaming kernel (cross_entropy.py:254-323), in the logits dtype."""
+
+    compute = logits.float()
+    targets = torch.as_tensor(targets).long()
+    weights = torch.as_tensor(weights).float()
+    valid = (targets != ignore_index) & (weights != 0)
+    lse = torch.logsumexp(compute, dim=-1)
+    prob = torch.exp(compute - lse[..., None])
+    columns = torch.arange(logits.shape[-1])
+    comparable = torch.where((targets >= 0) & (targets < logits.shape[-1]), targets, torch.full_like(targets, -1))
+    onehot = (columns == comparable[..., None]).float()
+    factor = torch.where(valid, weights * torch.as_tensor(cotangent).float(), torch.zeros_like(weights))
+    return (factor[..., None] * torch.where(valid[..., None], prob - onehot, torch.zeros_like(prob))).to(logits.dtype)
+
+
 def full_logits_loss_and_grads(hidden, head, targets, weights, dy: float):
     """The reference's pure path: materialise f32 logits, sparse CE, autograd to hidden / head."""
 

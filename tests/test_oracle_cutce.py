@@ -192,3 +192,35 @@ def test_reference_seeded_fixture_regenerates():
     assert float(weight_sum) == float(weights.sum()) == float(golden["weight_sum"])
     assert float(nll) == float(golden["nll_sum"])
     np.testing.assert_array_equal(lse.numpy(), golden["lse"])
+
+
+def test_streaming_sparse_ce_oracle_agrees_with_the_xla_path_and_its_ignore_rules():
+    # the setup of the reference's tests/kernels/test_cross_entropy_tpu.py:50-98 (vocab 1280,
+    # 256 rows, weight 0.5 on the first 96 rows, target 220 kept valid), with own seeds
+    rng = np.random.default_rng(50)
+    logits = torch.from_numpy((rng.standard_normal((256, 1280)) * 0.25).astype(np.float32)).to(torch.bfloat16)
+    targets = torch.from_numpy(rng.integers(0, 1280, size=256).astype(np.int64))
+    targets[0] = 220
+    weights = torch.where(torch.arange(256) < 96, torch.tensor(0.5), torch.tensor(0.0))
+    loss, lse = ref.pallas_sparse_cross_entropy(logits, targets, weights)
+    want = ref.xla_sparse_cross_entropy(logits, targets, weights)
+    torch.testing.assert_close(loss, want, rtol=0, atol=1e-6)
+    assert torch.equal(lse[96:], torch.zeros(160)) and torch.equal(loss[96:], torch.zeros(160))
+    cot = torch.from_numpy(rng.standard_normal(256).astype(np.float32))
+    got = ref.pallas_sparse_cross_entropy_vjp(logits, targets, weights, cot)
+    assert torch.equal(got, ref.xla_sparse_cross_entropy_vjp(logits, targets, weights, cot))
+    # ignore_index rows and out-of-range targets: no loss / no one-hot, never an index error
+    t2 = targets.clone()
+    t2[1], t2[2], t2[3] = -100, 5000, -7
+    loss2, lse2 = ref.pallas_sparse_cross_entropy(logits, t2, weights)
+    assert float(loss2[1]) == 0.0 and float(lse2[1]) == 0.0
+    torch.testing.assert_close(loss2[2], 0.5 * torch.logsumexp(logits[2].float(), -1))
+    torch.testing.assert_close(loss2[3], 0.5 * torch.logsumexp(logits[3].float(), -1))
+    grad2 = ref.pallas_sparse_cross_entropy_vjp(logits, t2, weights, cot)
+    assert float(grad2[1].abs().max()) == 0.0
+    torch.testing.assert_close(grad2[2].float().sum(), 0.5 * cot[2], rtol=2e-2, atol=2e-3)   # sum of softmax = 1
+    # uniform logits: lse = log V exactly representable check
+    flat = torch.zeros((2, 1024))
+    l3, s3 = ref.pallas_sparse_cross_entropy(flat, torch.tensor([3, 4]), torch.tensor([2.0, 1.0]))
+    torch.testing.assert_close(s3, torch.full((2,), float(np.log(1024.0))))
+    torch.testing.assert_close(l3, torch.tensor([2.0, 1.0]) * float(np.log(1024.0)))
