@@ -210,7 +210,13 @@ template <int D>
 CT_DEVICE void store_rows_t(const f32x16* acc, float row_scale, lds_addr patch, bf16* gbase,
                             size_t row_stride) {
   constexpr int CPR = D / 8;
-  const int l = lane_id(), j = l & 31, half = l >> 5;
+  int l = lane_id();
+  // The 16 patch addresses below depend on the lane only. Hoisted out of a caller's loop they
+  // would be 16 registers held for the whole kernel (and, once spilled, 16 scratch reloads
+  // with a full memory wait each per call), so the lane id is made opaque here and the
+  // addresses are recomputed where they are used.
+  asm volatile("" : "+v"(l));
+  const int j = l & 31, half = l >> 5;
 #pragma unroll
   for (int db = 0; db < D / 32; ++db) {
 #pragma unroll
