@@ -516,13 +516,17 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
         dp = mfma32(ro.load(CUR * kStage + QdoStage<D>::kDo, 0, ks), ro.load(vpatch_off, 0, ks), dp);
       const bool interior = tile_is_interior(q_uni, q_end_min, my_uni, my_rb * 32 + 31);
       f32x16 prob;
+      // The row offsets below depend on the lane only; hoisted out of the loop they become
+      // spilled registers whose reloads wait for every copy in flight. Recompute them here.
+      int half_here = half;
+      asm volatile("" : "+v"(half_here));
       if (!interior) {
         // Masked scores become -inf (their probability is then exactly 0). Written with
         // bitwise logic and selects only: the per-element tests must not turn into branches.
         const int seg_k_or_never = seg_k != 0 ? seg_k : -1;  // ids are >= 0
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
-          const int r0 = 8 * qd + 4 * half;  // first of 4 consecutive query rows
+          const int r0 = 8 * qd + 4 * half_here;  // first of 4 consecutive query rows
           const i32x4 seg4 = lds_load<i32x4>(stage + QdoStage<D>::kSeg + r0 * 4);
           i32x4 end4;
           if (has_end) {
@@ -540,7 +544,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
       }
 #pragma unroll
       for (int qd = 0; qd < 4; ++qd) {
-        const int r0 = 8 * qd + 4 * half;
+        const int r0 = 8 * qd + 4 * half_here;
         const f32x4 lse4 = lds_load<f32x4>(stage + QdoStage<D>::kLse + r0 * 4);
         const f32x4 del4 = lds_load<f32x4>(stage + QdoStage<D>::kDelta + r0 * 4);
 #pragma unroll

@@ -173,7 +173,11 @@ CT_DEVICE void tile_mask(lds_addr segk, int tile, int seg_q, int end_q, bool row
 // 32 kb + 8 (r / 4) + r % 4.
 template <bool SEG, bool CAUSAL>
 CT_DEVICE void mask_scores_t(lds_addr segk, int seg_q_or_never, int last_rel, f32x16* s) {
-  const int half = lane_id() >> 5;
+  // (opaque, so that the lane's share of the addresses below is recomputed here rather than
+  // kept in a register across the caller's loop, where it ends up spilled)
+  int lane = lane_id();
+  asm volatile("" : "+v"(lane));
+  const int half = lane >> 5;
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
