@@ -338,7 +338,7 @@ static int launch_dkv(hipStream_t stream, const AttnParams& p) {
   LaunchScope scope7("attn_dkv_schedule_kernel", stream);
   hipLaunchKernelGGL(attn_dkv_schedule_kernel, dim3(1), dim3(1024), 0, stream, p.meta, p.B, p.S,
                      p.Hkv, p.Hq / p.Hkv, p.dkv_max_entries, p.dkv_max_partials, p.dkv_header,
-                     p.dkv_counters, p.dkv_entries);
+                     p.dkv_entries);
   int rc = scope7.done();
   if (rc) return rc;
   const int grid = p.dkv_max_entries * p.Hkv;  // entries beyond the list's length exit at once
@@ -527,7 +527,6 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
                 L.total);
   char* ws = static_cast<char*>(a->workspace);
   p.dkv_header = reinterpret_cast<int*>(ws + L.header);
-  p.dkv_counters = reinterpret_cast<int*>(ws + L.counters);
   p.dkv_entries = reinterpret_cast<int2*>(ws + L.entries);
   p.dkv_partials = reinterpret_cast<float*>(ws + L.partials);
   p.lse2 = reinterpret_cast<float*>(ws + L.lse2);

@@ -131,9 +131,7 @@ struct QdoStage {
   static constexpr int kPatchBytes = 4 * 32 * D * 2;
   // resident V rows of the workgroup's 128 keys (32 per wavefront), after the two stages
   static constexpr int kVResident = 2 * kBytes;
-  // one flag word after the patch: "this workgroup is the last chunk of its tile to finish"
-  static constexpr int kLastFlag = 2 * kBytes + kPatchBytes;
-  static constexpr int kTotalBytes = kLastFlag + 16;
+  static constexpr int kTotalBytes = 2 * kBytes + kPatchBytes;
 };
 
 // Starts the asynchronous copy of query block qb of head h into `stage`: Q and dO rows, and
@@ -247,18 +245,17 @@ CT_DEVICE int dkv_split_count(int items, int target) {
 
 // Builds the dK/dV work list (one workgroup of 1024 threads): chunk target from
 // the total amount of work, chunk count per tile, entries bucketed by
-// decreasing work, arrival counters cleared.
+// decreasing work.
 __global__ __launch_bounds__(1024) void attn_dkv_schedule_kernel(const int* meta, int B, int S,
                                                                  int Hkv, int g, int max_entries,
                                                                  int max_partials, int* header,
-                                                                 int* counters, int2* entries) {
+                                                                 int2* entries) {
   __shared__ long long red[1024];
   __shared__ int hist[256];
   __shared__ int fill[256];
   __shared__ int carry;
   const int tid = threadIdx.x;
   const int nrb = S / 32, ntiles = B * (nrb / 4);
-  for (int i = tid; i < ntiles * Hkv; i += 1024) counters[i] = 0;
 
   auto block_sum = [&](long long v) {
     red[tid] = v;

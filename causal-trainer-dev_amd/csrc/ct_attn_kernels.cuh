@@ -53,7 +53,6 @@ struct AttnParams {
   float scale;      // already rounded to bf16
   // dK/dV work list (backward only)
   int* dkv_header;
-  int* dkv_counters;
   int2* dkv_entries;
   float* dkv_partials;
   int dkv_max_entries, dkv_max_partials;

@@ -106,7 +106,7 @@ constexpr int kDkvKeys = 128;      // keys per dK/dV tile
 
 struct DkvLayout {
   int max_entries, max_partials;
-  size_t header, counters, entries, lse2, partials, total;
+  size_t header, entries, lse2, partials, total;
 };
 
 // Sum over tiles of the chunk count is at most tiles + total_items / target and the
@@ -119,8 +119,7 @@ __host__ inline DkvLayout dkv_layout(int B, int S, int Hq, int Hkv, int D) {
   L.max_partials = min(2 * extra, L.max_entries);
   auto up = [](size_t v) { return (v + 255) / 256 * 256; };
   L.header = 0;
-  L.counters = 256;
-  L.entries = L.counters + up((size_t)tiles * Hkv * sizeof(int));
+  L.entries = 256;
   // lse * log2(e), head-major [B, Hq, S] (the caller's delta scratch holds delta the same way)
   L.lse2 = L.entries + up((size_t)L.max_entries * 2 * sizeof(int));
   L.partials = L.lse2 + up((size_t)B * S * Hq * sizeof(float));

@@ -172,6 +172,105 @@ ffi::Error CutceBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> hidden, ffi::Buff
   return status_to_error(ct_cutce_bwd(stream, &a));
 }
 
+// ---- decoder-layer neighbours and the logits-level loss ----------------------------------
+
+ffi::Error PositionIds(hipStream_t stream, ffi::Buffer<ffi::S32> attention_mask,
+                       ffi::Buffer<ffi::S32> canonical_ids, ffi::ResultBuffer<ffi::S32> positions) {
+  const auto dims = attention_mask.dimensions();
+  if (dims.size() != 2) return ffi::Error::InvalidArgument("attention_mask must be [batch, sequence]");
+  return status_to_error(ct_position_ids(stream, attention_mask.typed_data(), canonical_ids.typed_data(),
+                                         (int32_t)dims[0], (int32_t)dims[1], positions->typed_data()));
+}
+
+ffi::Error RotaryCosSin(hipStream_t stream, ffi::Buffer<ffi::S32> positions, ffi::Buffer<ffi::F32> inv_freq,
+                        ffi::ResultBuffer<ffi::BF16> cosine, ffi::ResultBuffer<ffi::BF16> sine) {
+  const auto dims = positions.dimensions();
+  if (dims.size() != 2) return ffi::Error::InvalidArgument("position_ids must be [batch, sequence]");
+  return status_to_error(ct_rotary_cos_sin(stream, positions.typed_data(), inv_freq.typed_data(),
+                                           (int64_t)dims[0] * dims[1], (int32_t)inv_freq.element_count(),
+                                           bits_out(cosine), bits_out(sine)));
+}
+
+// forward (inverse = false) and the transpose used for the gradients (inverse = true)
+ffi::Error ApplyRotary(hipStream_t stream, ffi::Buffer<ffi::BF16> q, ffi::Buffer<ffi::BF16> k,
+                       ffi::Buffer<ffi::BF16> cosine, ffi::Buffer<ffi::BF16> sine,
+                       ffi::ResultBuffer<ffi::BF16> q_out, ffi::ResultBuffer<ffi::BF16> k_out,
+                       int32_t rope_style, bool inverse, float q_scale) {
+  const auto qd = q.dimensions();
+  const auto kd = k.dimensions();
+  const auto cd = cosine.dimensions();
+  if (qd.size() != 4 || kd.size() != 4 || cd.size() != 3)
+    return ffi::Error::InvalidArgument("query and key must be [batch, sequence, heads, head_dim], tables [batch, sequence, pairs]");
+  ct_rotary_args a = {};
+  a.q_in = bits(q);
+  a.k_in = bits(k);
+  a.q_out = bits_out(q_out);
+  a.k_out = bits_out(k_out);
+  a.cosine = bits(cosine);
+  a.sine = bits(sine);
+  a.tokens = (int64_t)qd[0] * qd[1];
+  a.q_heads = (int32_t)qd[2];
+  a.kv_heads = (int32_t)kd[2];
+  a.head_dim = (int32_t)qd[3];
+  a.rotary_pairs = (int32_t)cd[2];
+  a.rope_style = rope_style;
+  a.inverse = inverse ? 1 : 0;
+  a.q_scale = q_scale;
+  return status_to_error(ct_apply_rotary(stream, &a));
+}
+
+ffi::Error RmsNormFwd(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi::BF16> scale,
+                      ffi::ResultBuffer<ffi::BF16> y, float eps) {
+  const auto dims = x.dimensions();
+  if (dims.empty()) return ffi::Error::InvalidArgument("rms_norm needs at least one axis");
+  const int64_t hidden = dims.back();
+  return status_to_error(ct_rms_norm_fwd(stream, bits(x), bits(scale), eps,
+                                         hidden ? (int64_t)x.element_count() / hidden : 0, (int32_t)hidden,
+                                         bits_out(y), nullptr));
+}
+
+ffi::Error RmsNormBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> x, ffi::Buffer<ffi::BF16> scale,
+                      ffi::Buffer<ffi::BF16> dy, ffi::ResultBuffer<ffi::BF16> dx,
+                      ffi::ResultBuffer<ffi::F32> dscale, ffi::ResultBuffer<ffi::U8> workspace, float eps) {
+  const auto dims = x.dimensions();
+  if (dims.empty()) return ffi::Error::InvalidArgument("rms_norm needs at least one axis");
+  const int64_t hidden = dims.back();
+  return status_to_error(ct_rms_norm_bwd(stream, bits(x), bits(scale), bits(dy), eps,
+                                         hidden ? (int64_t)x.element_count() / hidden : 0, (int32_t)hidden,
+                                         bits_out(dx), dscale->typed_data(), workspace->untyped_data(),
+                                         workspace->size_bytes()));
+}
+
+ct_sparse_ce_args sparse_ce_args(const ffi::AnyBuffer& logits, const ffi::Buffer<ffi::S32>& targets,
+                                 const ffi::Buffer<ffi::F32>& weights) {
+  ct_sparse_ce_args a = {};
+  const auto dims = logits.dimensions();
+  a.logits = logits.untyped_data();
+  a.targets = targets.typed_data();
+  a.weights = weights.typed_data();
+  a.vocab = dims.empty() ? 0 : (int32_t)dims.back();
+  a.rows = a.vocab ? (int64_t)logits.element_count() / a.vocab : 0;
+  a.logits_dtype = logits.element_type() == ffi::BF16 ? CT_DTYPE_BF16
+                   : logits.element_type() == ffi::F32 ? CT_DTYPE_F32 : -1;
+  a.ignore_index = -100;
+  return a;
+}
+
+ffi::Error SparseCeFwd(hipStream_t stream, ffi::AnyBuffer logits, ffi::Buffer<ffi::S32> targets,
+                       ffi::Buffer<ffi::F32> weights, ffi::ResultBuffer<ffi::F32> loss,
+                       ffi::ResultBuffer<ffi::F32> lse) {
+  const ct_sparse_ce_args a = sparse_ce_args(logits, targets, weights);
+  return status_to_error(ct_sparse_ce_fwd(stream, &a, loss->typed_data(), lse->typed_data()));
+}
+
+ffi::Error SparseCeBwd(hipStream_t stream, ffi::AnyBuffer logits, ffi::Buffer<ffi::S32> targets,
+                       ffi::Buffer<ffi::F32> weights, ffi::Buffer<ffi::F32> lse, ffi::Buffer<ffi::F32> dy,
+                       ffi::Result<ffi::AnyBuffer> dlogits) {
+  const ct_sparse_ce_args a = sparse_ce_args(logits, targets, weights);
+  return status_to_error(ct_sparse_ce_bwd(stream, &a, lse.typed_data(), dy.typed_data(),
+                                          dlogits->untyped_data()));
+}
+
 }  // namespace
 
 #define CT_STREAM Ctx<ffi::PlatformStream<hipStream_t>>()
@@ -242,3 +341,62 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_cutce_bwd, CutceBwd,
                                   .Ret<ffi::Buffer<ffi::U8>>()
                                   .Attr<bool>("sparse_compaction")
                                   .Attr<bool>("head_trainable"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_position_ids, PositionIds,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::S32>>());
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_rotary_cos_sin, RotaryCosSin,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>());
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_apply_rotary, ApplyRotary,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Attr<int32_t>("rope_style")
+                                  .Attr<bool>("inverse")
+                                  .Attr<float>("q_scale"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_rms_norm_fwd, RmsNormFwd,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Attr<float>("eps"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_rms_norm_bwd, RmsNormBwd,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Arg<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::BF16>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<float>("eps"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_sparse_ce_fwd, SparseCeFwd,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>());
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_sparse_ce_bwd, SparseCeBwd,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::AnyBuffer>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::AnyBuffer>());
