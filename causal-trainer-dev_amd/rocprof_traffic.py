@@ -14,6 +14,7 @@ text summary into ``--out``.
 from __future__ import annotations
 
 import argparse
+import re
 import collections
 import csv
 import glob
@@ -25,6 +26,11 @@ COPY_KERNEL = "ct_calibration_copy_kernel"
 
 
 def _short(name: str) -> str:
+    # counter runs may report the mangled name: _ZN2ct<len><kernel name>I...E...
+    mangled = re.match(r"_ZN2ct(\d+)", name)
+    if mangled:
+        start = mangled.end()
+        return name[start:start + int(mangled.group(1))]
     name = name.split("(")[0].replace("void ", "").strip()
     name = name.split("<")[0]
     return name.split("::")[-1]
