@@ -321,7 +321,8 @@ static int launch_dq(hipStream_t stream, const AttnParams& p) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
   }
-  const int grid = (p.S / (32 * PB)) * (p.Hq / HS) * p.B;
+  (void)PB;
+  const int grid = (p.Hq / HS) * kBins * 2;  // (head slice, KV head) groups x work bins x tile halves
   LaunchScope scope2("attn_dq_kernel", stream);
   hipLaunchKernelGGL((attn_dq_kernel<D, HS>), dim3(grid), dim3(256), smem, stream, p);
   return scope2.done();

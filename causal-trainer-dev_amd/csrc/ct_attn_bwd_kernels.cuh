@@ -20,16 +20,26 @@ namespace ct {
 // ---------------------------------------------------------------------------
 // dQ
 // ---------------------------------------------------------------------------
-template <int D, int HS>
-__global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
-  extern __shared__ __align__(16) char smem_raw[];
-  const lds_addr lds0 = lds_address_of(smem_raw);
-  constexpr int kStage = KvStage<D>::kBytes;
+// Fragment address structures of the backward kernels: the register-lean ones where the tile
+// is wide enough for them (both kernels are at the register limit).
+template <int D>
+using LeanRowFrags = std::conditional_t<(D / 8 >= 16), RowFragCompact<D / 8>, RowFragOffsets<D / 8>>;
+template <int D>
+using LeanTrFrags = std::conditional_t<(D / 8 >= 16), TrFragCompact<D / 8, KSlots::kAccum>,
+                                       TrFragOffsets<D / 8, KSlots::kAccum>>;
 
-  const QueryTileContext<D, HS> ctx(p);
+// One query tile (4 / HS row blocks x HS heads of one KV head), start to finish.
+template <int D, int HS>
+CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int qt, lds_addr lds0) {
+  constexpr int kStage = KvStage<D>::kBytes;
+  // (the fragment pointers are rebuilt per item from an opaque base: kept across the item loop
+  // they end up spilled and reloaded in the key-tile loop)
+  asm volatile("" : "+v"(lds0));
+  const LeanRowFrags<D> ro(lds0);
+  const LeanTrFrags<D> to(lds0);
+
+  const QueryTileContext<D, HS> ctx(p, b, kvh, slice, qt);
   const int l = lane_id(), half = l >> 5, w = threadIdx.x >> 6;
-  const RowFragOffsets<D / 8> ro(lds0);
-  const TrFragOffsets<D / 8, KSlots::kAccum> to(lds0);
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
   const size_t stat_t = ((size_t)ctx.work.b * p.Hq + ctx.work.h) * p.S + ctx.pos;  // head-major
@@ -106,9 +116,42 @@ __global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
     step(std::integral_constant<int, 1>{});
   }
 
-  const lds_addr patch = lds0 + w * 32 * D * 2;
-  bf16* gbase = p.dq + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
-  store_rows_t<D>(dqacc, p.scale, patch, gbase, q_row_stride);
+  if (ctx.active) {
+    const lds_addr patch = lds0 + w * 32 * D * 2;
+    bf16* gbase = p.dq + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
+    store_rows_t<D>(dqacc, p.scale, patch, gbase, q_row_stride);
+  }
+  // the store patches overlap the stages of the next item: its copies may start once every
+  // wavefront has read its patch back
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __syncthreads();
+}
+
+// Workgroup (group, bin, parity): walks the query tiles of one work bin for one (head slice, KV
+// head) group. The bins are those of the forward for tiles twice as tall; of each such tile
+// this workgroup takes the upper or the lower half, so that two workgroups share a compute
+// unit with near equal work. The group is the fast index: a group stays on one XCD and its
+// K / V rows in that XCD's L2.
+template <int D, int HS>
+__global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
+  extern __shared__ __align__(16) char smem_raw[];
+  const lds_addr lds0 = lds_address_of(smem_raw);
+  constexpr int PB = 4 / HS;
+  const int nrb = p.S / 32;
+  const int slices = (p.Hq / p.Hkv) / HS;
+  const int groups = slices * p.Hkv;
+  const int group = blockIdx.x % groups, rest = blockIdx.x / groups;
+  const int bin = rest % kBins, parity = rest / kBins;
+  const int kvh = group % p.Hkv, slice = group / p.Hkv;
+  const MetaPtr region = meta_const(p.meta + bin_region_offset(p.B, nrb, 2 * PB));
+  const int tpr = bin_tiles_per_row(nrb, 2 * PB);
+  const int it_end = uniform(region[bin + 1]);
+  for (int it = uniform(region[bin]); it < it_end; ++it) {
+    const int item = uniform(region[kBins + 1 + it]);
+    const int qt = 2 * (item % tpr) + parity;
+    if (qt * PB >= nrb) continue;  // the lower half of a partial last tile
+    attn_dq_item<D, HS>(p, item / tpr, kvh, slice, qt, lds0);
+  }
 }
 
 // ---------------------------------------------------------------------------

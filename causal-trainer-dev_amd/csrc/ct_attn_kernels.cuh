@@ -128,9 +128,8 @@ struct QueryWork {
 
 // S^T (two 32-key blocks) = K_tile Q^T for this wavefront's 32 queries.
 // `tile_off` is the tile's byte offset from the LDS base the offsets were built on.
-template <int D>
-CT_DEVICE void scores_t(int tile_off, const RowFragOffsets<D / 8>& ro, const bf16x8* qf,
-                        f32x16* s) {
+template <int D, class RowFrags>
+CT_DEVICE void scores_t(int tile_off, const RowFrags& ro, const bf16x8* qf, f32x16* s) {
   s[0] = zero16();
   s[1] = zero16();
 #pragma unroll
@@ -195,9 +194,8 @@ CT_DEVICE void mask_scores_t(lds_addr segk, int seg_q_or_never, int last_rel, f3
 
 // acc (D x 32 queries, transposed) += X^T W^T where X is a 64-row LDS tile read
 // transposed and W^T are the accumulator-layout weights wt[2].
-template <int D>
-CT_DEVICE void accumulate_t(int tile_off, const TrFragOffsets<D / 8, KSlots::kAccum>& to,
-                            const f32x16* wt, f32x16* acc) {
+template <int D, class TrFrags>
+CT_DEVICE void accumulate_t(int tile_off, const TrFrags& to, const f32x16* wt, f32x16* acc) {
 #pragma unroll
   for (int step = 0; step < 4; ++step) {
     const bf16x8 bop = pack_acc8(wt[step >> 1], step & 1);
