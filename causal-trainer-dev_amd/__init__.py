@@ -28,3 +28,6 @@ from .prep import canonicalize_segment_ids, shifted_targets_and_weights  # noqa:
 from .layer_ops import (  # noqa: F401,E402
     apply_rotary_cos_sin, apply_rotary_embedding, make_position_ids, rms_norm, rotary_cos_sin,
 )
+from . import maskgit, packing  # noqa: F401,E402
+from .maskgit import MaskGITBatchTransform  # noqa: F401,E402
+from .packing import best_fit_decreasing, collate, pack_examples, pad_example, pad_examples  # noqa: F401,E402

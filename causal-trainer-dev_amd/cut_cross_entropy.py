@@ -20,6 +20,17 @@ rows fit in ``LOGITS_CACHE_LIMIT_BYTES`` the forward also leaves them in a cache
 that lives until the backward of the loss (the adjacent step of a training
 iteration), and the backward then runs 3 GEMMs instead of 4. Above the limit, or
 with ``logits_cache=False``, nothing but ``lse`` is kept and logits are recomputed.
+
+``local_chunk_size`` (:697-825). The reference's chunk loop bounds what one TPU core
+holds at a time: it gathers one chunk of token rows across the tensor-parallel axis,
+compacts inside the chunk, adds each chunk's ``(nll, weight)`` to f32 totals and the head
+gradient to an f32 accumulator that is rounded once. On one GPU there is nothing to
+gather, and the kernels here already walk the rows in 256-row units with f32
+accumulators rounded once and an f64 loss sum, so a positive chunk size selects the
+same launches: a row's statistics and gradients do not depend on which chunk or slot
+it sits in (compaction is a stable permutation), and only the order of the final
+additions differs, inside the operator's tolerances. The option is validated as in
+the reference and otherwise changes nothing.
 """
 
 from __future__ import annotations
@@ -191,9 +202,6 @@ def pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weig
     active = {axis: int(size) for axis, size in sizes.items() if int(size) != 1}
     if active:
         raise ValueError(f"this build runs on one GPU; mesh axes larger than 1: {active}")
-    if local_chunk_size:
-        raise ValueError("local_chunk_size needs a tensor-parallel mesh; this build runs on one GPU")
-
     width = hidden_states.shape[-1]
     return _CutCE.apply(
         hidden_states.reshape(-1, width).contiguous(), lm_head_kernel.contiguous(),

@@ -17,6 +17,8 @@ Functions and what they follow:
   compact_active_rows           src/kernels/cut_cross_entropy.py:673-694
   cut_forward                   src/kernels/cut_cross_entropy.py:85-156, :474-521
   cut_backward                  src/kernels/cut_cross_entropy.py:225-278, :349-403, :597-667
+  chunked_cut_forward / chunked_cut_backward
+                                src/kernels/cut_cross_entropy.py:697-825 on a one-device mesh
   xla_sparse_cross_entropy(+vjp)  src/kernels/fused_cross_entropy.py:64-109
   cut_f64                       float64 evaluation of the same mathematics
 """
@@ -109,6 +111,72 @@ def cut_backward(hidden, head, targets, weights, lse, dy: float, *, head_trainab
     dhidden = (g.float() @ head.float().T).to(hidden.dtype)
     dhead = (hidden.float().T @ g.float()).to(head.dtype) if head_trainable else None
     return dhidden, dhead
+
+
+def _row_chunks(rows: int, chunk_size: int):
+    """Row ranges of the zero-padded chunk grid (cut_cross_entropy.py:697-708)."""
+
+    if chunk_size <= 0:
+        raise ValueError("chunk_size must be positive")
+    return [(start, min(start + chunk_size, rows)) for start in range(0, rows, chunk_size)]
+
+
+def chunked_cut_forward(hidden, head, targets, weights, chunk_size: int, *, sparse_compaction: bool = False):
+    """The row-chunk loop of the reference without a vocabulary axis (:723-741).
+
+    Every chunk is padded to chunk_size with zero-weight rows, optionally compacted on its own,
+    and adds its (nll, weight) to f32 running totals in chunk order. Returns the totals and
+    the per-row lse (padding rows dropped, in original row order).
+    """
+
+    targets = torch.as_tensor(targets)
+    weights = torch.as_tensor(weights).float()
+    rows = hidden.shape[0]
+    nll_total = torch.zeros((), dtype=torch.float32)
+    weight_total = torch.zeros((), dtype=torch.float32)
+    lse_rows = torch.zeros(rows, dtype=torch.float32)
+    for start, stop in _row_chunks(rows, chunk_size):
+        pad = chunk_size - (stop - start)
+        h = torch.cat([hidden[start:stop], hidden.new_zeros(pad, hidden.shape[1])])
+        t = torch.cat([targets[start:stop], targets.new_zeros(pad)])
+        w = torch.cat([weights[start:stop], weights.new_zeros(pad)])
+        if sparse_compaction:
+            h, t, w, indices, slot_valid = compact_active_rows(h, t, w)
+        nll, weight, lse = cut_forward(h, head, t, w)
+        nll_total = nll_total + nll
+        weight_total = weight_total + weight
+        if sparse_compaction:
+            full = torch.zeros(chunk_size, dtype=torch.float32)
+            full[indices[slot_valid]] = lse[slot_valid]
+            lse = full
+        lse_rows[start:stop] = lse[: stop - start]
+    return nll_total, weight_total, lse_rows
+
+
+def chunked_cut_backward(hidden, head, targets, weights, lse, dy: float, chunk_size: int, *,
+                         head_trainable: bool = True):
+    """Backward of the chunk loop (:767-822): dHidden per chunk from f32 products rounded once;
+    dHead added up in f32 over the chunks and rounded once at the end."""
+
+    targets = torch.as_tensor(targets).long()
+    weights = torch.as_tensor(weights).float()
+    rows = hidden.shape[0]
+    dhidden = torch.zeros_like(hidden)
+    dhead_acc = torch.zeros(head.shape, dtype=torch.float32) if head_trainable else None
+    vocab = head.shape[1]
+    for start, stop in _row_chunks(rows, chunk_size):
+        h, t, w = hidden[start:stop], targets[start:stop], weights[start:stop]
+        logits = _logits_f32(h, head)
+        valid = (w != 0)[:, None]
+        prob = torch.where(valid, torch.exp(logits - lse[start:stop, None]), 0.0)
+        onehot = torch.zeros_like(prob)
+        hit = torch.nonzero((t >= 0) & (t < vocab) & (w != 0)).flatten()
+        onehot[hit, t[hit]] = 1.0
+        g = ((w * float(dy))[:, None] * (prob - onehot)).to(torch.bfloat16)
+        dhidden[start:stop] = (g.float() @ head.float().T).to(hidden.dtype)
+        if head_trainable:
+            dhead_acc += h.float().T @ g.float()
+    return dhidden, (dhead_acc.to(head.dtype) if head_trainable else None)
 
 
 def xla_sparse_cross_entropy(logits, targets, weights):

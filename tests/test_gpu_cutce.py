@@ -166,6 +166,53 @@ def test_reference_seeded_fixture_and_frozen_head(ct, gpu):
         ct.pallas_cut_linear_cross_entropy(hd, wd, targets.to(gpu), weights.to(gpu), mesh={"fsdp": 2})
 
 
+@pytest.mark.parametrize("compaction,trainable", [(False, True), (True, True), (False, False)])
+def test_chunked_option_against_the_chunk_loop_oracle(ct, gpu, compaction, trainable):
+    # the one-device case of the reference's tests/kernels/test_tiled_cut.py:89-128:
+    # chunks of 128 over 2 x 386 rows (ragged last chunk), cotangent 0.37
+    from oracle import cutce_ref
+
+    golden = np.load("tests/golden/cutce_rng460.npz")
+    hidden = torch.from_numpy(golden["hidden"]).view(torch.bfloat16)
+    head = torch.from_numpy(golden["head"]).view(torch.bfloat16)
+    targets, weights = torch.from_numpy(golden["targets"]), torch.from_numpy(golden["weights"])
+    flat = hidden.reshape(-1, 128)
+    want_nll, want_weight, lse = cutce_ref.chunked_cut_forward(flat, head, targets.reshape(-1), weights.reshape(-1),
+                                                               128, sparse_compaction=compaction)
+    want_dh, want_dw = cutce_ref.chunked_cut_backward(flat, head, targets.reshape(-1), weights.reshape(-1), lse,
+                                                      0.37, 128, head_trainable=trainable)
+    hd = hidden.to(gpu).requires_grad_(True)
+    wd = head.to(gpu).requires_grad_(True)
+    nll, weight_sum = ct.pallas_cut_linear_cross_entropy(hd, wd, targets.to(gpu), weights.to(gpu), mesh=None,
+                                                         sparse_compaction=compaction, lm_head_trainable=trainable,
+                                                         local_chunk_size=128)
+    (nll * 0.37 + weight_sum * 0.0).backward()
+    assert float(nll) == pytest.approx(float(want_nll), rel=LOSS_RTOL)
+    assert float(weight_sum) == float(want_weight)
+    assert relative_l2(hd.grad.cpu().reshape(-1, 128), want_dh) < GRAD_RTOL
+    assert (hd.grad.cpu()[weights == 0] == 0).all()
+    if trainable:
+        assert relative_l2(wd.grad.cpu(), want_dw) < GRAD_RTOL
+    else:
+        assert wd.grad is None
+
+
+def test_chunked_option_all_masked_rows_and_frozen_head(ct, gpu):
+    # tests/kernels/test_tiled_cut.py:138-155
+    golden = np.load("tests/golden/cutce_rng460.npz")
+    hidden = torch.from_numpy(golden["hidden"]).view(torch.bfloat16)[:1, :199].contiguous()
+    head = torch.from_numpy(golden["head"]).view(torch.bfloat16)
+    hd = hidden.to(gpu).requires_grad_(True)
+    wd = head.to(gpu).requires_grad_(True)
+    targets = torch.full((1, 199), -100, dtype=torch.int32, device=gpu)
+    nll, weight_sum = ct.pallas_cut_linear_cross_entropy(hd, wd, targets, torch.zeros(1, 199, device=gpu), mesh=None,
+                                                         sparse_compaction=True, lm_head_trainable=False,
+                                                         local_chunk_size=128)
+    nll.backward()
+    assert float(nll) == float(weight_sum) == 0.0
+    assert wd.grad is None and not hd.grad.any()
+
+
 def test_closed_form_uniform_logits(ct, gpu):
     # zero hidden => nll = sum(w) log V (reference: tests/training/test_losses.py:125-252)
     rows, vocab = 300, 1000

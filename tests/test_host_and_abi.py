@@ -125,6 +125,10 @@ def test_cutce_argument_errors(ct):
         fn(hidden, head, targets, weights, local_chunk_size=True)
     with pytest.raises(ValueError, match="non-negative"):
         fn(hidden, head, targets, weights, local_chunk_size=-1)
+    # tests/kernels/test_tiled_cut.py:158-166: every invalid chunk size names the option
+    for invalid in (True, 1.5, "128", -1):
+        with pytest.raises((TypeError, ValueError), match="local_chunk_size"):
+            fn(hidden, head, targets, weights, local_chunk_size=invalid)
     with pytest.raises(RuntimeError, match="only on a ROCm GPU"):
         fn(hidden, head, targets, weights)
 

@@ -224,3 +224,53 @@ def test_streaming_sparse_ce_oracle_agrees_with_the_xla_path_and_its_ignore_rule
     l3, s3 = ref.pallas_sparse_cross_entropy(flat, torch.tensor([3, 4]), torch.tensor([2.0, 1.0]))
     torch.testing.assert_close(s3, torch.full((2,), float(np.log(1024.0))))
     torch.testing.assert_close(l3, torch.tensor([2.0, 1.0]) * float(np.log(1024.0)))
+
+
+@pytest.mark.parametrize("compaction", [False, True])
+def test_chunked_loop_meets_the_reference_expectations_on_its_seeded_data(compaction):
+    # tests/kernels/test_tiled_cut.py:89-128 on a one-device mesh: chunks of 128 over 2 x 386
+    # rows (a ragged last chunk), cotangent 0.37, checked against log_softmax + autograd
+    from tests.golden import make_golden
+
+    fixture = make_golden.cutce_fixture()
+    hidden, head = fixture["hidden"].reshape(-1, 128), fixture["head"]
+    targets = torch.from_numpy(fixture["targets"].reshape(-1))
+    weights = torch.from_numpy(fixture["weights"].reshape(-1))
+    nll, weight_sum, lse = ref.chunked_cut_forward(hidden, head, targets, weights, 128,
+                                                  sparse_compaction=compaction)
+    dhidden, dhead = ref.chunked_cut_backward(hidden, head, targets, weights, lse, 0.37, 128)
+
+    h64 = hidden.double().requires_grad_(True)
+    w64 = head.double().requires_grad_(True)
+    logp = torch.log_softmax(h64 @ w64, -1)
+    expected = -(logp.gather(1, targets.long().clamp(min=0)[:, None])[:, 0] * weights.double()).sum()
+    (0.37 * expected).backward()
+    assert float(nll) == pytest.approx(float(expected), rel=2e-5, abs=2e-3)
+    assert float(weight_sum) == float(weights.sum())
+    for got, want in ((dhidden, h64.grad), (dhead, w64.grad)):
+        assert float((got.double() - want).norm() / want.norm()) < 0.025
+    assert not dhidden[weights == 0].any()
+    assert ref.chunked_cut_backward(hidden, head, targets, weights, lse, 0.37, 128, head_trainable=False)[1] is None
+
+    # the chunk loop is the unchunked operator up to the order of f32 additions
+    base_nll, base_weight, base_lse = ref.cut_forward(hidden, head, targets, weights)
+    base_dhidden, base_dhead = ref.cut_backward(hidden, head, targets, weights, base_lse, 0.37)
+    assert float(nll) == pytest.approx(float(base_nll), rel=1e-6)
+    assert float(weight_sum) == float(base_weight)
+    torch.testing.assert_close(lse, base_lse, rtol=1e-6, atol=1e-6)
+    torch.testing.assert_close(dhidden.float(), base_dhidden.float(), rtol=0, atol=2.0 ** -8 * float(base_dhidden.abs().max()))
+    assert float((dhead.float() - base_dhead.float()).norm() / base_dhead.float().norm()) < 4e-3
+
+
+def test_chunked_loop_all_masked_rows():
+    # tests/kernels/test_tiled_cut.py:138-155: 199 rows, every weight zero, frozen head
+    from tests.golden import make_golden
+
+    fixture = make_golden.cutce_fixture()
+    hidden, head = fixture["hidden"].reshape(-1, 128)[:199], fixture["head"]
+    targets = torch.full((199,), -100, dtype=torch.int32)
+    weights = torch.zeros(199)
+    nll, weight_sum, lse = ref.chunked_cut_forward(hidden, head, targets, weights, 128, sparse_compaction=True)
+    assert float(nll) == float(weight_sum) == 0.0
+    dhidden, dhead = ref.chunked_cut_backward(hidden, head, targets, weights, lse, 1.0, 128, head_trainable=False)
+    assert dhead is None and not dhidden.any()
