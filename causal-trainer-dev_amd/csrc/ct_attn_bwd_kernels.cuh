@@ -30,10 +30,11 @@ using LeanTrFrags = std::conditional_t<(D / 8 >= 16), TrFragCompact<D / 8, KSlot
 
 // One query tile (4 / HS row blocks x HS heads of one KV head), start to finish.
 template <int D, int HS>
-CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int qt, lds_addr lds0) {
+CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int qt, const lds_addr lds_base) {
   constexpr int kStage = KvStage<D>::kBytes;
   // (the fragment pointers are rebuilt per item from an opaque base: kept across the item loop
   // they end up spilled and reloaded in the key-tile loop)
+  lds_addr lds0 = lds_base;
   asm volatile("" : "+v"(lds0));
   const LeanRowFrags<D> ro(lds0);
   const LeanTrFrags<D> to(lds0);
@@ -103,7 +104,7 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
           const float prob = exp2_fast(fmaf(s[kbk][r], kLog2e, -lse2));
           s[kbk][r] = prob * (dp[kbk][r] - delta_q);
         }
-      accumulate_t<D>(CUR * kStage + KvStage<D>::kK, to, s, dqacc);
+      accumulate_t<D>(CUR * kStage + KvStage<D>::kK, LeanTrFrags<D>::fresh(lds_base), s, dqacc);
     }
     dma_wait_all();
     __syncthreads();
@@ -198,19 +199,6 @@ CT_DEVICE void qdo_fetch(const TileDma<kQueryTile, D / 8>& dma, const AttnParams
                       : which == 2 ? reinterpret_cast<const char*>(p.seg + row_major)
                                    : reinterpret_cast<const char*>(p.end + row_major);
     dma16(src + part * 16, stage + QdoStage<D>::kLse);
-  }
-}
-
-// After this thread's copies have landed (dma_wait_all), fold the softmax scale into its own
-// Q slots in place (bf16 multiply, as the forward does). A barrier must follow.
-template <int D>
-CT_DEVICE void qdo_commit(lds_addr stage, float scale) {
-  constexpr int kSlots = kQueryTile * (D / 8) / 256;
-  const int tid = threadIdx.x;
-#pragma unroll
-  for (int n = 0; n < kSlots; ++n) {
-    const lds_addr slot = stage + QdoStage<D>::kQ + (n * 256 + tid) * 16;
-    lds_store<u32x4>(slot, as_u32x4(scale_bf16x8(as_bf16x8(lds_load<u32x4>(slot)), scale)));
   }
 }
 
@@ -515,6 +503,11 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
     dvacc[db] = zero16();
   }
 
+  // The Q tiles stay unscaled in LDS: the softmax scale enters the exponent in f32
+  // (S = scale * (Q K^T); the forward rounded scale * Q to bf16 first, a difference of one
+  // bf16 rounding per element of Q) and dK = scale * (dS^T Q) is scaled once at the end.
+  const float scale_log2e = p.scale * kLog2e;
+
   // Work items: (head of the group, query block) pairs, flattened; query block fastest.
   const int nq = (q_lo <= q_hi) ? (q_hi - q_lo + 1) : 0;
   const int per_chunk = (nq * g + nsplit - 1) / nsplit;
@@ -529,7 +522,6 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   if (it < items) {
     qdo_fetch<D>(dma, p, b, head, qb, lds0);
     dma_wait_all();
-    qdo_commit<D>(lds0, p.scale);
   }
   __syncthreads();
 
@@ -590,7 +582,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = 4 * qd + e;
-          const float pr = exp2_fast(fmaf(s[r], kLog2e, -lse4[e]));
+          const float pr = exp2_fast(fmaf(s[r], scale_log2e, -lse4[e]));
           prob[r] = pr;
           dp[r] = pr * (dp[r] - del4[e]);
         }
@@ -599,7 +591,6 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
       accumulate_keys<D>(CUR * kStage + QdoStage<D>::kQ, to, dp, dkacc);
     }
     dma_wait_all();
-    if (more) qdo_commit<D>(lds0 + (CUR ^ 1) * kStage, p.scale);
     __syncthreads();
     ++it;
     qb = qb_next;
@@ -610,6 +601,11 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
     if (it >= items) break;
     step(std::integral_constant<int, 1>{});
   }
+
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) dkacc[db][e] *= p.scale;
 
   if (nsplit > 1) {
     // A chunk of a split tile leaves its sums as f32 for attn_dkv_reduce_kernel:

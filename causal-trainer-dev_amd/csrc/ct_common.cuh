@@ -45,6 +45,14 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
 CT_DEVICE int lane_id() { return threadIdx.x & 63; }
+// The lane id read from the execution mask at the point of use (all lanes active). Being a
+// volatile asm without inputs it is neither hoisted out of a loop nor kept in a register
+// across one: values derived from it are recomputed where they are needed.
+CT_DEVICE int lane_id_here() {
+  int l;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+  return l;
+}
 
 CT_DEVICE int uniform(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
@@ -242,6 +250,7 @@ struct TrFragOffsets {
       }
     }
   }
+  CT_DEVICE static TrFragOffsets fresh(lds_addr base) { return TrFragOffsets(base); }
   CT_DEVICE bf16x8 load(int tile_off, int ks, int cb) const {
     const int off = tile_off + ks * kStepBytes + (cb >> 2) * 256;
     const bf16x4_vs lo = lds_load_tr(ptr[0][cb & 3] + off);
@@ -284,8 +293,9 @@ struct TrFragCompact {
   static constexpr int kStepBytes = 16 * CPR * 16;
   lds_addr row_base[2];  // per read of the pair: row start + the 8-byte half inside the chunk
   unsigned y16[2];       // ((chunk bits below the column block) ^ swizzle(row)) * 16
-  CT_DEVICE explicit TrFragCompact(lds_addr base) {
-    const int l = lane_id(), p = l & 15, q16 = (l >> 4) & 1, half = l >> 5;
+  CT_DEVICE explicit TrFragCompact(lds_addr base) : TrFragCompact(base, lane_id()) {}
+  CT_DEVICE TrFragCompact(lds_addr base, int l) {
+    const int p = l & 15, q16 = (l >> 4) & 1, half = l >> 5;
 #pragma unroll
     for (int second = 0; second < 2; ++second) {
       const int row = (MAP == KSlots::kNatural ? 8 * half + 4 * second : 4 * half + 8 * second) +
@@ -295,6 +305,10 @@ struct TrFragCompact {
       y16[second] = (unsigned)(((col_low >> 3) ^ swizzle<CPR>(row)) << 4);
     }
   }
+  // The same addresses rebuilt at the point of use: nothing lane-dependent is then live
+  // across the caller's loop (where, once spilled, each such value costs a scratch reload
+  // whose wait also drains the asynchronous copies in flight).
+  CT_DEVICE static TrFragCompact fresh(lds_addr base) { return TrFragCompact(base, lane_id_here()); }
   CT_DEVICE bf16x8 load(int tile_off, int ks, int cb) const {
     const int off = tile_off + ks * kStepBytes + (cb >> 2) * 256;
     const unsigned block = (unsigned)((cb & 3) * 4) << 4;
