@@ -180,25 +180,26 @@ struct QdoStage {
 
 // Starts the asynchronous copy of query block qb of head h into `stage`: Q and dO rows, and
 // the per-row statistics. The four statistics arrays (lse2, delta: head-major f32; segment ids,
-// visible ends: i32) are 128 contiguous bytes each for the 32 rows, and sit in the stage in that
-// order, so lanes 0..31 of wavefront 0 fetch them with one copy instruction (8 lanes per
-// array). Without visible ends (plain causal) the last 8 lanes stay idle.
+// visible ends: i32) are 128 contiguous bytes each for the 32 rows and sit in the stage in that
+// order; wavefront w fetches array w with its first 8 lanes (one copy instruction, the source
+// chosen with scalar selects), so no wavefront carries a divergent address computation.
+// Without visible ends (plain causal) wavefront 3 has nothing to fetch.
 template <int D>
 CT_DEVICE void qdo_fetch(const TileDma<kQueryTile, D / 8>& dma, const AttnParams& p, int b, int h,
                          int qb, lds_addr stage) {
-  const int tid = threadIdx.x;
   const size_t origin = (((size_t)b * p.S + qb * kQueryTile) * p.Hq + h) * D;
   dma.issue(reinterpret_cast<const char*>(p.q + origin), stage + QdoStage<D>::kQ);
   dma.issue(reinterpret_cast<const char*>(p.dout + origin), stage + QdoStage<D>::kDo);
-  if (tid < (p.end ? 32 : 24)) {
+  const int which = uniform(threadIdx.x >> 6);
+  if (which < (p.end ? 4 : 3)) {
     const size_t head_major = ((size_t)b * p.Hq + h) * p.S + qb * kQueryTile;
     const size_t row_major = (size_t)b * p.S + qb * kQueryTile;
-    const int which = tid >> 3, part = tid & 7;
     const char* src = which == 0   ? reinterpret_cast<const char*>(p.lse2 + head_major)
                       : which == 1 ? reinterpret_cast<const char*>(p.delta + head_major)
                       : which == 2 ? reinterpret_cast<const char*>(p.seg + row_major)
                                    : reinterpret_cast<const char*>(p.end + row_major);
-    dma16(src + part * 16, stage + QdoStage<D>::kLse);
+    const unsigned lane = threadIdx.x & 63;
+    if (lane < 8) dma16_s(src, lane * 16, stage + QdoStage<D>::kLse + which * (kQueryTile * 4));
   }
 }
 
@@ -217,6 +218,35 @@ CT_DEVICE f32x16 rows_times_frags(int tile_off, const DkvRowFrags<D>& ro, const 
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) c = mfma32(ro.load(tile_off, 0, ks), frags[ks], c);
   return c;
+}
+
+// Hand-scheduled MFMA sequences of the dK/dV kernel for D = 128 (gen_attn_asm.py): the
+// compiler's own schedule issues each LDS fragment read directly in front of the MFMA that
+// consumes it, so with two wavefronts per SIMD every MFMA pays most of the LDS latency.
+// STAGE_OFF is the byte offset of the stage (Q tile, then dO tile) from the LDS base the
+// pointers were built on; v_off the byte offset of this wavefront's V rows.
+template <int STAGE_OFF>
+CT_DEVICE void dkv_sdp_sequence_128(const RowFragOffsets<16>& ro, const bf16x8* kf, unsigned v_off,
+                                    f32x16& s, f32x16& dp) {
+  asm volatile(CT_DKV_SDP_SEQUENCE
+               : "=&v"(s), "=&v"(dp)
+               : "v"(ro.ptr[0]), "v"(ro.ptr[1]), "v"(ro.ptr[2]), "v"(ro.ptr[3]), "v"(ro.ptr[4]),
+                 "v"(ro.ptr[5]), "v"(ro.ptr[6]), "v"(ro.ptr[7]), "v"(kf[0]), "v"(kf[1]), "v"(kf[2]),
+                 "v"(kf[3]), "v"(kf[4]), "v"(kf[5]), "v"(kf[6]), "v"(kf[7]), "s"(v_off), "i"(STAGE_OFF)
+               : "memory", CT_DKV_ASM_SCRATCH);
+}
+template <int STAGE_OFF>
+CT_DEVICE void dkv_acc_sequence_128(const TrFragOffsets<16, KSlots::kAccum>& to, const f32x16& prob,
+                                    const f32x16& ds, f32x16* dvacc, f32x16* dkacc) {
+  const bf16x8 p0 = pack_acc8(prob, 0), p1 = pack_acc8(prob, 1);
+  const bf16x8 d0 = pack_acc8(ds, 0), d1 = pack_acc8(ds, 1);
+  asm volatile(CT_DKV_ACC_SEQUENCE
+               : "+v"(dvacc[0]), "+v"(dvacc[1]), "+v"(dvacc[2]), "+v"(dvacc[3]), "+v"(dkacc[0]),
+                 "+v"(dkacc[1]), "+v"(dkacc[2]), "+v"(dkacc[3])
+               : "v"(to.ptr[0][0]), "v"(to.ptr[0][1]), "v"(to.ptr[0][2]), "v"(to.ptr[0][3]),
+                 "v"(to.ptr[1][0]), "v"(to.ptr[1][1]), "v"(to.ptr[1][2]), "v"(to.ptr[1][3]), "v"(p0),
+                 "v"(p1), "v"(d0), "v"(d1), "i"(STAGE_OFF)
+               : "memory", CT_DKV_ASM_SCRATCH);
 }
 
 // acc (32 keys x D) += W^T X, W in accumulator layout (rows = the 32 tile rows,
@@ -488,7 +518,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   // K fragments stay in registers; V fragments are parked in LDS (this wavefront's
   // private 32-row patch) and re-read per block, which keeps the kernel under 256
   // registers so that two workgroups share a CU.
-  const int vpatch_off = QdoStage<D>::kVResident + w * 32 * D * 2;
+  const int vpatch_off = QdoStage<D>::kVResident + uniform(w) * 32 * D * 2;
   const lds_addr vpatch = lds0 + vpatch_off;
   bf16x8 kf[D / 16];
 #pragma unroll
@@ -502,6 +532,12 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
     dkacc[db] = zero16();
     dvacc[db] = zero16();
   }
+
+  // Make the K fragment loads complete here. Left pending, their first use inside the item
+  // loop gets an `s_waitcnt vmcnt(n)` whose count fits the first item only; on every later item
+  // the same wait stalls until the asynchronous copies of the next stage have landed.
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) asm volatile("" : "+v"(kf[ks]));
 
   // The Q tiles stay unscaled in LDS: the softmax scale enters the exponent in f32
   // (S = scale * (Q K^T); the forward rounded scale * Q to bf16 first, a difference of one
@@ -525,6 +561,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   }
   __syncthreads();
 
+  QueryBlockBounds qb_bounds = query_block_bounds(meta_b, min(qb, nrb - 1));
   auto step = [&](auto stage_tag) {
     constexpr int CUR = decltype(stage_tag)::value;
     const lds_addr stage = lds0 + CUR * kStage;
@@ -536,16 +573,25 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
     }
     if (more) qdo_fetch<D>(dma, p, b, head_next, qb_next, lds0 + (CUR ^ 1) * kStage);
 
-    const MetaPtr qm = meta_const(meta_b + qb * kMetaW);
-    const int q_min = uniform(qm[kMinNz]), q_max = uniform(qm[kMaxId]),
-              q_end_max = uniform(qm[kEndMax]), q_end_min = uniform(qm[kEndMin]),
-              q_uni = uniform(qm[kUniform]);
+    // bounds of this query block (read one item ahead: the scalar loads are long done when
+    // the next item needs them)
+    const int q_min = qb_bounds.min_nz, q_max = qb_bounds.max_id, q_end_max = qb_bounds.end_max,
+              q_end_min = qb_bounds.end_min, q_uni = qb_bounds.uniform;
+    if (more) qb_bounds = query_block_bounds(meta_b, qb_next);
     if (blocks_interact(q_min, q_max, q_end_max, my_min, my_max, my_rb * 32)) {
-      f32x16 s = rows_times_frags<D>(CUR * kStage + QdoStage<D>::kQ, ro, kf);
-      f32x16 dp = zero16();
+      f32x16 s, dp;
+      if constexpr (D == 128) {
+        // (fragment pointers built here from the lane id: held across the loop they would
+        // push the kernel over its register budget)
+        const RowFragOffsets<16> rp(lds0, lane_id_here());
+        dkv_sdp_sequence_128<CUR * kStage>(rp, kf, (unsigned)vpatch_off, s, dp);
+      } else {
+        s = rows_times_frags<D>(CUR * kStage + QdoStage<D>::kQ, ro, kf);
+        dp = zero16();
 #pragma unroll
-      for (int ks = 0; ks < D / 16; ++ks)
-        dp = mfma32(ro.load(CUR * kStage + QdoStage<D>::kDo, 0, ks), ro.load(vpatch_off, 0, ks), dp);
+        for (int ks = 0; ks < D / 16; ++ks)
+          dp = mfma32(ro.load(CUR * kStage + QdoStage<D>::kDo, 0, ks), ro.load(vpatch_off, 0, ks), dp);
+      }
       const bool interior = tile_is_interior(q_uni, q_end_min, my_uni, my_rb * 32 + 31);
       f32x16 prob;
       // The row offsets below depend on the lane only; hoisted out of the loop they become
@@ -587,8 +633,13 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
           dp[r] = pr * (dp[r] - del4[e]);
         }
       }
-      accumulate_keys<D>(CUR * kStage + QdoStage<D>::kDo, to, prob, dvacc);
-      accumulate_keys<D>(CUR * kStage + QdoStage<D>::kQ, to, dp, dkacc);
+      if constexpr (D == 128) {
+        const TrFragOffsets<16, KSlots::kAccum> tp(lds0, lane_id_here());
+        dkv_acc_sequence_128<CUR * kStage>(tp, prob, dp, dvacc, dkacc);
+      } else {
+        accumulate_keys<D>(CUR * kStage + QdoStage<D>::kDo, to, prob, dvacc);
+        accumulate_keys<D>(CUR * kStage + QdoStage<D>::kQ, to, dp, dkacc);
+      }
     }
     dma_wait_all();
     __syncthreads();

@@ -207,8 +207,9 @@ struct RowFragOffsets {
   static constexpr int kSteps = CPR / 2;
   static constexpr int kRowBlockBytes = 32 * CPR * 16;
   lds_addr ptr[kSteps];
-  CT_DEVICE explicit RowFragOffsets(lds_addr base) {
-    const int l = lane_id(), row = l & 31, half = l >> 5;
+  CT_DEVICE explicit RowFragOffsets(lds_addr base) : RowFragOffsets(base, lane_id()) {}
+  CT_DEVICE RowFragOffsets(lds_addr base, int l) {
+    const int row = l & 31, half = l >> 5;
 #pragma unroll
     for (int ks = 0; ks < kSteps; ++ks) ptr[ks] = base + tile_byte_offset<CPR>(row, 2 * ks + half);
   }
@@ -237,8 +238,9 @@ template <int CPR, KSlots MAP>
 struct TrFragOffsets {
   static constexpr int kStepBytes = 16 * CPR * 16;
   lds_addr ptr[2][4];
-  CT_DEVICE explicit TrFragOffsets(lds_addr base) {
-    const int l = lane_id(), p = l & 15, q16 = (l >> 4) & 1, half = l >> 5;
+  CT_DEVICE explicit TrFragOffsets(lds_addr base) : TrFragOffsets(base, lane_id()) {}
+  CT_DEVICE TrFragOffsets(lds_addr base, int l) {
+    const int p = l & 15, q16 = (l >> 4) & 1, half = l >> 5;
 #pragma unroll
     for (int second = 0; second < 2; ++second) {
       const int row = (MAP == KSlots::kNatural ? 8 * half + 4 * second : 4 * half + 8 * second) +

@@ -83,13 +83,105 @@ def qk_sequence(ahead, slots):
     return lines + TAIL
 
 
+DKV_SLOTS = 5
+DKV_SCRATCH0 = 256 - 4 * DKV_SLOTS - 1  # one address temporary, then the fragment slots
+
+
+def dkv_slot(slot):
+    lo = DKV_SCRATCH0 + 1 + 4 * slot
+    return lo, lo + 3
+
+
+def dkv_sdp_sequence():
+    """S = Q K^T and dP = dO V^T of one (32 query rows x 32 keys) block, interleaved: per k-step
+    one MFMA of each chain. The fragment reads (Q, dO, V per k-step) run through a ring of
+    DKV_SLOTS registers quads: a read is issued as soon as the MFMA that used its slot has been
+    issued, so reads stay DKV_SLOTS fragments in front of their MFMAs.
+
+    operands: %0 S, %1 dP (written), %2-%9 row-fragment pointers (k-step), %10-%17 K fragments
+    (registers), %18 byte offset of this wavefront's V rows (scalar), %19 byte offset of the
+    stage (Q tile; the dO tile follows 8192 bytes later).
+    """
+    steps = 8
+    total = 3 * steps  # read r = 3 ks + which; which: 0 Q, 1 dO, 2 V
+    lines = ["s_waitcnt lgkmcnt(0)"]
+    state = {"issued": 0}
+
+    def load_next():
+        r = state["issued"]
+        if r >= total:
+            return []
+        state["issued"] += 1
+        ks, which = divmod(r, 3)
+        lo, hi = dkv_slot(r % DKV_SLOTS)
+        if which == 2:
+            return ["v_add_u32_e32 v%d, %%18, %%%d" % (DKV_SCRATCH0, 2 + ks),
+                    "ds_read_b128 v[%d:%d], v%d" % (lo, hi, DKV_SCRATCH0)]
+        return ["ds_read_b128 v[%d:%d], %%%d offset:%%19+%d" % (lo, hi, 2 + ks, which * 8192)]
+
+    for _ in range(DKV_SLOTS):
+        lines += load_next()
+    for ks in range(steps):
+        q_slot = dkv_slot((3 * ks) % DKV_SLOTS)
+        do_slot = dkv_slot((3 * ks + 1) % DKV_SLOTS)
+        v_slot = dkv_slot((3 * ks + 2) % DKV_SLOTS)
+        lines.append("s_waitcnt lgkmcnt(%d)" % (state["issued"] - (3 * ks + 1)))
+        lines.append("v_mfma_f32_32x32x16_bf16 %%0, v[%d:%d], %%%d, %s" % (q_slot[0], q_slot[1], 10 + ks,
+                                                                        "0" if ks == 0 else "%0"))
+        lines += load_next()
+        lines.append("s_waitcnt lgkmcnt(%d)" % (state["issued"] - (3 * ks + 3)))
+        lines.append("v_mfma_f32_32x32x16_bf16 %%1, v[%d:%d], v[%d:%d], %s" % (do_slot[0], do_slot[1], v_slot[0],
+                                                                              v_slot[1], "0" if ks == 0 else "%1"))
+        lines += load_next()
+        lines += load_next()
+    return lines + TAIL
+
+
+def dkv_acc_sequence(ahead=DKV_SLOTS, slots=DKV_SLOTS):
+    """dV[db] += P^T[step] dO(step, db) and dK[db] += dS^T[step] Q(step, db), interleaved: 16
+    MFMAs, each with one transposed fragment (2 ds_read_b64_tr_b16) read `ahead` fragments in
+    front of it.
+
+    operands: %0-%3 dV accumulators, %4-%7 dK accumulators, %8-%11 lo pointers (column block db),
+    %12-%15 hi pointers, %16-%17 P^T (k-step), %18-%19 dS^T (k-step), %20 byte offset of the
+    stage (Q tile; the dO tile follows 8192 bytes later).
+    """
+    order = [(step, db, which) for step in range(2) for db in range(4) for which in range(2)]  # which: 0 dV, 1 dK
+    n = len(order)
+    lines = ["s_waitcnt lgkmcnt(0)"]
+
+    def load(i):
+        step, db, which = order[i]
+        lo, _ = dkv_slot(i % slots)
+        off = "%%20+%d" % (step * 4096 + (8192 if which == 0 else 0))
+        return ["ds_read_b64_tr_b16 v[%d:%d], %%%d offset:%s" % (lo, lo + 1, 8 + db, off),
+                "ds_read_b64_tr_b16 v[%d:%d], %%%d offset:%s" % (lo + 2, lo + 3, 12 + db, off)]
+
+    for i in range(min(ahead, n)):
+        lines += load(i)
+    for i in range(n):
+        later = min(ahead - 1, n - 1 - i)
+        lines.append("s_waitcnt lgkmcnt(%d)" % (2 * later))
+        step, db, which = order[i]
+        lo, hi = dkv_slot(i % slots)
+        acc = db if which == 0 else 4 + db
+        aop = (16 if which == 0 else 18) + step
+        lines.append("v_mfma_f32_32x32x16_bf16 %%%d, %%%d, v[%d:%d], %%%d" % (acc, aop, lo, hi, acc))
+        if i + ahead < n:
+            lines += load(i + ahead)
+    return lines + TAIL
+
+
 def clobbers():
     regs = ", ".join('"v%d"' % r for r in range(SCRATCH0, SCRATCH0 + 16))
-    return "#define CT_ATTN_ASM_SCRATCH %s\n" % regs
+    dkv = ", ".join('"v%d"' % r for r in range(DKV_SCRATCH0, 256))
+    return "#define CT_ATTN_ASM_SCRATCH %s\n\n#define CT_DKV_ASM_SCRATCH %s\n" % (regs, dkv)
 
 
 if __name__ == "__main__":
     print("// Generated by gen_attn_asm.py -- do not edit by hand.")
     print(emit(pv_sequence(4, 4), "CT_ATTN_PV_SEQUENCE"))
     print(emit(qk_sequence(4, 4), "CT_ATTN_QK_SEQUENCE"))
+    print(emit(dkv_sdp_sequence(), "CT_DKV_SDP_SEQUENCE"))
+    print(emit(dkv_acc_sequence(), "CT_DKV_ACC_SEQUENCE"))
     print(clobbers())
