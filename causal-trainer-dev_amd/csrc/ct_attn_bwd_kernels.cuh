@@ -583,7 +583,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
       if constexpr (D == 128) {
         // (fragment pointers built here from the lane id: held across the loop they would
         // push the kernel over its register budget)
-        const RowFragOffsets<16> rp(lds0, lane_id_here());
+        const RowFragOffsets<16> rp = RowFragOffsets<16>::expand(RowFragCompact<16>(lds0, lane_id_here()));
         dkv_sdp_sequence_128<CUR * kStage>(rp, kf, (unsigned)vpatch_off, s, dp);
       } else {
         s = rows_times_frags<D>(CUR * kStage + QdoStage<D>::kQ, ro, kf);
@@ -634,7 +634,8 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
         }
       }
       if constexpr (D == 128) {
-        const TrFragOffsets<16, KSlots::kAccum> tp(lds0, lane_id_here());
+        const TrFragOffsets<16, KSlots::kAccum> tp =
+            TrFragOffsets<16, KSlots::kAccum>::expand(TrFragCompact<16, KSlots::kAccum>(lds0, lane_id_here()));
         dkv_acc_sequence_128<CUR * kStage>(tp, prob, dp, dvacc, dkacc);
       } else {
         accumulate_keys<D>(CUR * kStage + QdoStage<D>::kDo, to, prob, dvacc);

@@ -213,6 +213,16 @@ struct RowFragOffsets {
 #pragma unroll
     for (int ks = 0; ks < kSteps; ++ks) ptr[ks] = base + tile_byte_offset<CPR>(row, 2 * ks + half);
   }
+  // The same table from the compact form of the addresses (RowFragCompact): one xor-add per
+  // pointer instead of the three operations per pointer of the constructor above.
+  template <class Compact>
+  CT_DEVICE static RowFragOffsets expand(const Compact& c) {
+    RowFragOffsets out;
+#pragma unroll
+    for (int ks = 0; ks < kSteps; ++ks) out.ptr[ks] = c.row_base + (((unsigned)(2 * ks) << 4) ^ c.x16);
+    return out;
+  }
+  RowFragOffsets() = default;
   CT_DEVICE lds_addr addr(int tile_off, int rb, int ks) const {
     return ptr[ks] + (tile_off + rb * kRowBlockBytes);
   }
@@ -253,6 +263,18 @@ struct TrFragOffsets {
     }
   }
   CT_DEVICE static TrFragOffsets fresh(lds_addr base) { return TrFragOffsets(base); }
+  // The same table from the compact form (TrFragCompact): one xor-add per pointer.
+  template <class Compact>
+  CT_DEVICE static TrFragOffsets expand(const Compact& c) {
+    TrFragOffsets out;
+#pragma unroll
+    for (int second = 0; second < 2; ++second)
+#pragma unroll
+      for (int cb = 0; cb < 4; ++cb)
+        out.ptr[second][cb] = c.row_base[second] + (((unsigned)(cb * 4) << 4) ^ c.y16[second]);
+    return out;
+  }
+  TrFragOffsets() = default;
   CT_DEVICE bf16x8 load(int tile_off, int ks, int cb) const {
     const int off = tile_off + ks * kStepBytes + (cb >> 2) * 256;
     const bf16x4_vs lo = lds_load_tr(ptr[0][cb & 3] + off);
@@ -275,8 +297,9 @@ struct RowFragCompact {
   static constexpr int kRowBlockBytes = 32 * CPR * 16;
   lds_addr row_base;  // start of this lane's row
   unsigned x16;       // (half ^ swizzle(row)) * 16
-  CT_DEVICE explicit RowFragCompact(lds_addr base) {
-    const int l = lane_id(), row = l & 31, half = l >> 5;
+  CT_DEVICE explicit RowFragCompact(lds_addr base) : RowFragCompact(base, lane_id()) {}
+  CT_DEVICE RowFragCompact(lds_addr base, int l) {
+    const int row = l & 31, half = l >> 5;
     row_base = base + row * CPR * 16;
     x16 = (unsigned)((half ^ swizzle<CPR>(row)) << 4);
   }
