@@ -333,7 +333,7 @@ __global__ __launch_bounds__(1024) void attn_dkv_schedule_kernel(const int* meta
   long long local = 0;
   for (int t = tid; t < ntiles; t += 1024) local += dkv_tile_items(meta, nrb, t, g);
   const long long total = block_sum(local);
-  long long want = (total * Hkv + 2 * kDkvSlots - 1) / (2 * kDkvSlots);
+  long long want = (total * Hkv + kDkvSlots - 1) / kDkvSlots;  // one compute slot's fair share
   int target = (int)min((long long)INT_MAX / 2, max((long long)kDkvMinChunk, want));
 
   // Entry and partial-slot counts for this target; coarsen the target if they overflow the

@@ -92,12 +92,13 @@ __host__ __device__ inline size_t meta_total_ints(int B, int nrb) {
 // A 128-key tile's work is the list of (query head of the group, visiting
 // 32-row query block) items. Tiles at the start of a long segment carry many
 // times the mean, so the list of a heavy tile is cut into up to kDkvMaxSplit
-// chunks of about half a compute slot's fair share; every chunk is one
+// chunks of about one compute slot's fair share (measured: finer chunks shorten the
+// tail of the launch by less than their partial sums cost); every chunk is one
 // workgroup, chunks are dispatched heaviest first, and the chunks of a split
-// tile leave f32 partial sums that the last one to finish adds up in chunk
-// order (fixed order: results do not depend on timing).
-// Workspace: header (entry count, chunk target), one arrival counter per
-// (tile, KV head), the sorted entries, the partial sums.
+// tile leave f32 partial sums that a small kernel adds up in chunk order
+// (fixed order: results do not depend on timing).
+// Workspace: header (entry count, chunk target), the sorted entries, lse * log2 e,
+// the partial sums.
 // ---------------------------------------------------------------------------
 constexpr int kDkvSlots = 512;     // workgroups resident at once on the device (2 per CU)
 constexpr int kDkvMinChunk = 16;   // items
@@ -110,11 +111,11 @@ struct DkvLayout {
 };
 
 // Sum over tiles of the chunk count is at most tiles + total_items / target and the
-// target is at least total_items * kv_heads / (2 * kDkvSlots).
+// target is at least total_items * kv_heads / kDkvSlots.
 __host__ inline DkvLayout dkv_layout(int B, int S, int Hq, int Hkv, int D) {
   DkvLayout L;
   const int tiles = B * (S / kDkvKeys);
-  const int extra = (2 * kDkvSlots + Hkv - 1) / Hkv + 1;
+  const int extra = (kDkvSlots + Hkv - 1) / Hkv + 1;
   L.max_entries = tiles + extra;
   L.max_partials = min(2 * extra, L.max_entries);
   auto up = [](size_t v) { return (v + 255) / 256 * 256; };
