@@ -91,15 +91,21 @@ __device__ __forceinline__ bf16 scaled(bf16 v, float s, bool on) {
 // forward: out = bf16(bf16(R x) * s); inverse: out = bf16(R^T bf16(x * s)). The rotation is
 // evaluated in f32 from the bf16 operands and rounded once.
 template <bool ADJACENT>
-__global__ __launch_bounds__(256) void apply_rotary_kernel(ct_rotary_args a, long total_chunks) {
-  const long gid = (long)blockIdx.x * 256 + threadIdx.x;
-  if (gid >= total_chunks) return;
+__device__ __forceinline__ void apply_rotary_chunk(const ct_rotary_args& a, long t, int h, int c);
+
+// One workgroup per token walks the (head, chunk) pairs of that token: no 64-bit index
+// arithmetic per chunk, and the token's cos / sin row is shared by the whole workgroup.
+template <bool ADJACENT>
+__global__ __launch_bounds__(256) void apply_rotary_kernel(ct_rotary_args a) {
   const int cpr = a.head_dim / 8;  // chunks per head row
   const int heads = a.q_heads + a.kv_heads;
-  const int c = (int)(gid % cpr);
-  const long th = gid / cpr;
-  const int h = (int)(th % heads);
-  const long t = th / heads;
+  const long t = blockIdx.x;
+  for (unsigned item = threadIdx.x; item < (unsigned)(heads * cpr); item += 256)
+    apply_rotary_chunk<ADJACENT>(a, t, (int)(item / (unsigned)cpr), (int)(item % (unsigned)cpr));
+}
+
+template <bool ADJACENT>
+__device__ __forceinline__ void apply_rotary_chunk(const ct_rotary_args& a, long t, int h, int c) {
   const bool is_q = h < a.q_heads;
   const uint16_t* in = is_q ? a.q_in : a.k_in;
   uint16_t* out = is_q ? a.q_out : a.k_out;
@@ -204,6 +210,39 @@ __global__ __launch_bounds__(256) void rms_norm_fwd_kernel(const uint16_t* x, co
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = (bf16)((float)(bf16)((float)v[e] * r) * (float)w[e]);
     *reinterpret_cast<u32x4*>(yr + c * 8) = as_u32x4(o);
+  }
+}
+
+// The same for d = 512 NCH with the row held in registers: every load of the row is in flight
+// at once and x is read from memory exactly once.
+template <int NCH>
+__global__ __launch_bounds__(256) void rms_norm_fwd_rows_kernel(const uint16_t* x, const uint16_t* scale,
+                                                                float eps, long rows, uint16_t* y,
+                                                                float* rstd) {
+  constexpr int d = 512 * NCH;
+  const long row = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int lane = threadIdx.x & 63;
+  const uint16_t* xr = x + (size_t)row * d;
+  bf16x8 v[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) v[i] = as_bf16x8(*reinterpret_cast<const u32x4*>(xr + (lane + 64 * i) * 8));
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) ss += (float)v[i][e] * (float)v[i][e];
+  ss = wave_sum(ss);
+  const float r = 1.0f / sqrtf(ss / (float)d + eps);
+  if (rstd && lane == 0) rstd[row] = r;
+  uint16_t* yr = y + (size_t)row * d;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const bf16x8 w = as_bf16x8(*reinterpret_cast<const u32x4*>(scale + (lane + 64 * i) * 8));
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (bf16)((float)(bf16)((float)v[i][e] * r) * (float)w[e]);
+    *reinterpret_cast<u32x4*>(yr + (lane + 64 * i) * 8) = as_u32x4(o);
   }
 }
 
@@ -355,14 +394,14 @@ extern "C" int32_t ct_apply_rotary(void* stream, const ct_rotary_args* a) {
   CT_REQUIRE(aligned16(a->q_in) && aligned16(a->k_in) && aligned16(a->q_out) && aligned16(a->k_out) &&
                  aligned16(a->cosine) && aligned16(a->sine),
              "ct_apply_rotary: pointers must be 16-byte aligned");
-  const long total = (long)a->tokens * (a->q_heads + a->kv_heads) * (a->head_dim / 8);
+  CT_REQUIRE(a->tokens <= 0x7fffffffll, "ct_apply_rotary: at most 2^31 - 1 tokens per call");
   LaunchScope scope("apply_rotary_kernel", (hipStream_t)stream);
   if (a->rope_style == CT_ROPE_GPT_J)
-    hipLaunchKernelGGL((apply_rotary_kernel<true>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, *a, total);
+    hipLaunchKernelGGL((apply_rotary_kernel<true>), dim3((unsigned)a->tokens), dim3(256), 0,
+                       (hipStream_t)stream, *a);
   else
-    hipLaunchKernelGGL((apply_rotary_kernel<false>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0,
-                       (hipStream_t)stream, *a, total);
+    hipLaunchKernelGGL((apply_rotary_kernel<false>), dim3((unsigned)a->tokens), dim3(256), 0,
+                       (hipStream_t)stream, *a);
   return scope.done();
 }
 
@@ -375,8 +414,16 @@ extern "C" int32_t ct_rms_norm_fwd(void* stream, const uint16_t* x, const uint16
   CT_REQUIRE(aligned16(x) && aligned16(scale) && aligned16(y),
              "ct_rms_norm_fwd: pointers must be 16-byte aligned");
   LaunchScope scope("rms_norm_fwd_kernel", (hipStream_t)stream);
-  hipLaunchKernelGGL(rms_norm_fwd_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                     (hipStream_t)stream, x, scale, eps, (long)rows, hidden, y, rstd);
+  const dim3 grid((unsigned)((rows + 3) / 4)), block(256);
+  hipStream_t st = (hipStream_t)stream;
+  switch (hidden % 512 == 0 ? hidden / 512 : 0) {
+    case 1: hipLaunchKernelGGL((rms_norm_fwd_rows_kernel<1>), grid, block, 0, st, x, scale, eps, (long)rows, y, rstd); break;
+    case 2: hipLaunchKernelGGL((rms_norm_fwd_rows_kernel<2>), grid, block, 0, st, x, scale, eps, (long)rows, y, rstd); break;
+    case 4: hipLaunchKernelGGL((rms_norm_fwd_rows_kernel<4>), grid, block, 0, st, x, scale, eps, (long)rows, y, rstd); break;
+    case 8: hipLaunchKernelGGL((rms_norm_fwd_rows_kernel<8>), grid, block, 0, st, x, scale, eps, (long)rows, y, rstd); break;
+    case 16: hipLaunchKernelGGL((rms_norm_fwd_rows_kernel<16>), grid, block, 0, st, x, scale, eps, (long)rows, y, rstd); break;
+    default: hipLaunchKernelGGL(rms_norm_fwd_kernel, grid, block, 0, st, x, scale, eps, (long)rows, hidden, y, rstd);
+  }
   return scope.done();
 }
 
