@@ -456,38 +456,46 @@ __global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, Cutce
     }
 }
 
-// Same G^T from the f32 logits the forward left in its cache: one pass over memory, 8 slots
-// per thread. grid = (slab rows, ceil(n_pad / 2048)).
+// Same G^T from the f32 logits the forward left in its cache: one pass over memory. A thread
+// owns 8 slots and walks kDlogitsRows vocabulary rows with them, so the per-slot constants
+// (factor, lse, target: 96 bytes per thread) are loaded once per kDlogitsRows * 32 bytes of
+// logits and all of a thread's logits loads are in flight together.
+// grid = (slab rows / kDlogitsRows, ceil(n_pad / 2048)).
+constexpr int kDlogitsRows = 8;
 __global__ __launch_bounds__(256) void cutce_dlogits_cached_kernel(CutceParams p, CutceRowParams rp,
                                                                    const float* cache, int slab0,
                                                                    bf16* G) {
-  const int vrel = blockIdx.x, v = slab0 + vrel;
+  const int vrel0 = blockIdx.x * kDlogitsRows;
   const int slot0 = (blockIdx.y * 256 + threadIdx.x) * 8;
   // the two GEMM kernels that follow start from fresh work counters
   if (blockIdx.x == 0 && blockIdx.y == 0) reset_unit_counters(p.header);
   const int n_act = p.header->n_act;
   if (slot0 >= (n_act + kGemmTile - 1) / kGemmTile * kGemmTile) return;
-  bf16x8 out;
-  if (v < p.V) {
-    const float* src = cache + (size_t)v * p.n_pad + slot0;
-    const f32x4 a = *reinterpret_cast<const f32x4*>(src);
-    const f32x4 b = *reinterpret_cast<const f32x4*>(src + 4);
-    const f32x4 f0 = *reinterpret_cast<const f32x4*>(rp.fac + slot0);
-    const f32x4 f1 = *reinterpret_cast<const f32x4*>(rp.fac + slot0 + 4);
-    const f32x4 l0 = *reinterpret_cast<const f32x4*>(rp.lse2 + slot0);
-    const f32x4 l1 = *reinterpret_cast<const f32x4*>(rp.lse2 + slot0 + 4);
-    const i32x4 t0 = *reinterpret_cast<const i32x4*>(rp.tgt + slot0);
-    const i32x4 t1 = *reinterpret_cast<const i32x4*>(rp.tgt + slot0 + 4);
+  const f32x4 f0 = *reinterpret_cast<const f32x4*>(rp.fac + slot0);
+  const f32x4 f1 = *reinterpret_cast<const f32x4*>(rp.fac + slot0 + 4);
+  const f32x4 l0 = *reinterpret_cast<const f32x4*>(rp.lse2 + slot0);
+  const f32x4 l1 = *reinterpret_cast<const f32x4*>(rp.lse2 + slot0 + 4);
+  const i32x4 t0 = *reinterpret_cast<const i32x4*>(rp.tgt + slot0);
+  const i32x4 t1 = *reinterpret_cast<const i32x4*>(rp.tgt + slot0 + 4);
+  f32x4 a[kDlogitsRows], b[kDlogitsRows];
+#pragma unroll
+  for (int r = 0; r < kDlogitsRows; ++r) {
+    // rows past the vocabulary read the last row (the value is not used)
+    const float* src = cache + (size_t)min(slab0 + vrel0 + r, p.V - 1) * p.n_pad + slot0;
+    a[r] = *reinterpret_cast<const f32x4*>(src);
+    b[r] = *reinterpret_cast<const f32x4*>(src + 4);
+  }
+#pragma unroll
+  for (int r = 0; r < kDlogitsRows; ++r) {
+    const int v = slab0 + vrel0 + r;
+    bf16x8 out;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      out[e] = (bf16)(f0[e] != 0.f ? dlogit(a[e], f0[e], l0[e], t0[e], v) : 0.f);
-      out[4 + e] = (bf16)(f1[e] != 0.f ? dlogit(b[e], f1[e], l1[e], t1[e], v) : 0.f);
+      out[e] = (bf16)((f0[e] != 0.f && v < p.V) ? dlogit(a[r][e], f0[e], l0[e], t0[e], v) : 0.f);
+      out[4 + e] = (bf16)((f1[e] != 0.f && v < p.V) ? dlogit(b[r][e], f1[e], l1[e], t1[e], v) : 0.f);
     }
-  } else {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) out[e] = (bf16)0.f;
+    store_global16(G + (size_t)(vrel0 + r) * p.n_pad + slot0, as_u32x4(out));
   }
-  store_global16(G + (size_t)vrel * p.n_pad + slot0, as_u32x4(out));
 }
 
 // dHidden[idx[slot], n] (+)= sum_v G^T[v, slot] head[n, slab0 + v]
@@ -839,7 +847,7 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
     const int slab_width = slab_tiles * kGemmTile;
     if (cache) {
       LaunchScope scope11("cutce_dlogits_cached_kernel", stream);
-      hipLaunchKernelGGL(cutce_dlogits_cached_kernel, dim3(slab_width, (p.n_pad + 2047) / 2048),
+      hipLaunchKernelGGL(cutce_dlogits_cached_kernel, dim3(slab_width / kDlogitsRows, (p.n_pad + 2047) / 2048),
                          dim3(256), 0, stream, p, rp, cache, slab0, G);
       if ((rc = scope11.done())) return rc;
     } else {
