@@ -322,7 +322,8 @@ static int launch_dq(hipStream_t stream, const AttnParams& p) {
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
   }
   (void)PB;
-  const int grid = (p.Hq / HS) * kBins * 2;  // (head slice, KV head) groups x work bins x tile halves
+  // (head slice, KV head) groups x 64 workgroups: two per compute unit when there are 8 groups
+  const int grid = (p.Hq / HS) * kBins * 2;
   LaunchScope scope2("attn_dq_kernel", stream);
   hipLaunchKernelGGL((attn_dq_kernel<D, HS>), dim3(grid), dim3(256), smem, stream, p);
   return scope2.done();
@@ -356,13 +357,13 @@ static int launch_dkv(hipStream_t stream, const AttnParams& p) {
 template <int D>
 static int launch_delta(hipStream_t stream, const bf16* out, const bf16* dout, float* delta,
                         long rows, const float* lse = nullptr, float* lse2 = nullptr, int S = 0,
-                        int Hq = 0) {
+                        int Hq = 0, int* zeroed = nullptr, int zeroed_count = 0) {
   const long threads = rows * (D / 8);
   const dim3 grid((unsigned)((threads + 255) / 256));
   LaunchScope scope4("attn_delta_kernel", stream);
   if (lse2)
     hipLaunchKernelGGL((attn_delta_kernel<D, true>), grid, dim3(256), 0, stream, out, dout, delta,
-                       rows, lse, lse2, S, Hq);
+                       rows, lse, lse2, S, Hq, zeroed, zeroed_count);
   else
     hipLaunchKernelGGL((attn_delta_kernel<D, false>), grid, dim3(256), 0, stream, out, dout, delta,
                        rows, lse, lse2, S, Hq);
@@ -372,7 +373,7 @@ static int launch_delta(hipStream_t stream, const bf16* out, const bf16* dout, f
 template <int D>
 static int dispatch_bwd(hipStream_t stream, const AttnParams& p) {
   int rc = launch_delta<D>(stream, p.out, p.dout, p.delta, (long)p.B * p.S * p.Hq, p.lse, p.lse2,
-                           p.S, p.Hq);
+                           p.S, p.Hq, p.dq_counters, kDqCounters);
   if (rc) return rc;
   switch (heads_per_group(p.Hq, p.Hkv)) {
     case 4: rc = launch_dq<D, 4>(stream, p); break;
@@ -528,6 +529,7 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
                 L.total);
   char* ws = static_cast<char*>(a->workspace);
   p.dkv_header = reinterpret_cast<int*>(ws + L.header);
+  p.dq_counters = p.dkv_header + 64;
   p.dkv_entries = reinterpret_cast<int2*>(ws + L.entries);
   p.dkv_partials = reinterpret_cast<float*>(ws + L.partials);
   p.lse2 = reinterpret_cast<float*>(ws + L.lse2);

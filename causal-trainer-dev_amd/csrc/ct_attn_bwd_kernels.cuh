@@ -128,30 +128,39 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
   __syncthreads();
 }
 
-// Workgroup (group, bin, parity): walks the query tiles of one work bin for one (head slice, KV
-// head) group. The bins are those of the forward for tiles twice as tall; of each such tile
-// this workgroup takes the upper or the lower half, so that two workgroups share a compute
-// unit with near equal work. The group is the fast index: a group stays on one XCD and its
-// K / V rows in that XCD's L2.
+// Workgroups of one (head slice, KV head) group share a work counter and pull query tiles of PB
+// row blocks from the work-sorted schedules of the batch rows (tile `rank` of row b at pull
+// B * rank + b: heaviest tiles first), so a workgroup that drew light tiles simply draws more of
+// them. (Static bins left 15 % of the workgroup slots idle at the end of the launch: the time
+// of a tile depends on its mix of masked and unmasked key tiles, not just on their number.)
+// The group is the fast index of blockIdx: a group stays on one XCD and its K / V rows in that
+// XCD's L2. With more groups than counters (kDqCounters) the tiles are dealt round robin.
 template <int D, int HS>
 __global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr lds0 = lds_address_of(smem_raw);
+  __shared__ int next_pull;
   constexpr int PB = 4 / HS;
   const int nrb = p.S / 32;
   const int slices = (p.Hq / p.Hkv) / HS;
   const int groups = slices * p.Hkv;
-  const int group = blockIdx.x % groups, rest = blockIdx.x / groups;
-  const int bin = rest % kBins, parity = rest / kBins;
+  const int group = blockIdx.x % groups, member = blockIdx.x / groups, members = gridDim.x / groups;
   const int kvh = group % p.Hkv, slice = group / p.Hkv;
-  const MetaPtr region = meta_const(p.meta + bin_region_offset(p.B, nrb, 2 * PB));
-  const int tpr = bin_tiles_per_row(nrb, 2 * PB);
-  const int it_end = uniform(region[bin + 1]);
-  for (int it = uniform(region[bin]); it < it_end; ++it) {
-    const int item = uniform(region[kBins + 1 + it]);
-    const int qt = 2 * (item % tpr) + parity;
-    if (qt * PB >= nrb) continue;  // the lower half of a partial last tile
-    attn_dq_item<D, HS>(p, item / tpr, kvh, slice, qt, lds0);
+  const int tpr = bin_tiles_per_row(nrb, PB);
+  const int total = p.B * tpr;
+  const MetaPtr sched = meta_const(p.sched + query_schedule_offset(nrb, PB));
+  const bool dynamic = groups <= kDqCounters;
+  for (int pull = member;; pull += members) {
+    if (dynamic) {
+      if (threadIdx.x == 0) next_pull = atomicAdd(&p.dq_counters[group], 1);
+      __syncthreads();
+      pull = uniform(next_pull);
+      __syncthreads();
+    }
+    if (pull >= total) break;
+    const int b = pull % p.B, rank = pull / p.B;
+    const int qt = uniform(sched[(size_t)b * schedule_ints(nrb) + rank]);
+    attn_dq_item<D, HS>(p, b, kvh, slice, qt, lds0);
   }
 }
 

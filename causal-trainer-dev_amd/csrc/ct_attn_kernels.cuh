@@ -54,6 +54,7 @@ struct AttnParams {
   // dK/dV work list (backward only)
   int* dkv_header;
   int2* dkv_entries;
+  int* dq_counters;  // kDqCounters ints, zeroed by the delta pass of the same call
   float* dkv_partials;
   int dkv_max_entries, dkv_max_partials;
 };
@@ -572,9 +573,11 @@ attn_fwd_kernel(AttnParams p) {
 template <int D, bool HEAD_MAJOR>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* out, const bf16* dout,
                                                          float* delta, long rows, const float* lse,
-                                                         float* lse2, int S, int Hq) {
+                                                         float* lse2, int S, int Hq, int* zeroed = nullptr,
+                                                         int zeroed_count = 0) {
   constexpr int LPR = D / 8;  // lanes per row
   const long gid = (long)blockIdx.x * 256 + threadIdx.x;
+  if (zeroed && gid < zeroed_count) zeroed[gid] = 0;  // work counters of the kernel that follows
   const long row = gid / LPR;
   const int c = gid % LPR;
   float acc = 0.f;

@@ -105,6 +105,8 @@ constexpr int kDkvMinChunk = 16;   // items
 constexpr int kDkvMaxSplit = 32;
 constexpr int kDkvKeys = 128;      // keys per dK/dV tile
 
+constexpr int kDqCounters = 448;  // one per (head slice, KV head) group of the dQ kernel
+
 struct DkvLayout {
   int max_entries, max_partials;
   size_t header, entries, lse2, partials, total;
@@ -119,8 +121,8 @@ __host__ inline DkvLayout dkv_layout(int B, int S, int Hq, int Hkv, int D) {
   L.max_entries = tiles + extra;
   L.max_partials = min(2 * extra, L.max_entries);
   auto up = [](size_t v) { return (v + 255) / 256 * 256; };
-  L.header = 0;
-  L.entries = 256;
+  L.header = 0;  // 64 ints of dK/dV list header, then kDqCounters work counters of the dQ kernel
+  L.entries = (64 + kDqCounters) * sizeof(int);
   // lse * log2(e), head-major [B, Hq, S] (the caller's delta scratch holds delta the same way)
   L.lse2 = L.entries + up((size_t)L.max_entries * 2 * sizeof(int));
   L.partials = L.lse2 + up((size_t)B * S * Hq * sizeof(float));
