@@ -30,9 +30,12 @@ PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 def parse_args():
     parser = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     parser.add_argument("--gpus", type=int, default=1)
-    parser.add_argument("--steps", type=int, default=20)
-    parser.add_argument("--warmup", type=int, default=5)
-    parser.add_argument("--cutce-steps", type=int, default=None, help="default: min(steps, 5)")
+    # A step takes about 1.2 ms: short runs measure a GPU whose clocks are still ramping (20 timed
+    # steps after 5 read 6-7 % slower than the steady rate, which 200 after 50 reach and 2000
+    # after 1000 confirm), so the defaults are long enough for the steady rate.
+    parser.add_argument("--steps", type=int, default=200)
+    parser.add_argument("--warmup", type=int, default=50)
+    parser.add_argument("--cutce-steps", type=int, default=None, help="default: min(steps, 10)")
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-cutce", action="store_true")
     parser.add_argument("--no-layer-ops", action="store_true")
@@ -358,11 +361,11 @@ def main():
     if args.calibration_copy_bytes:
         calibration_copy(ct, torch, args.calibration_copy_bytes)
     if not args.no_cutce:
-        cut_steps = args.cutce_steps or min(args.steps, 5)
-        result["cutce"] = bench_cutce(ct, torch, cut_steps, min(args.warmup, 2),
+        cut_steps = args.cutce_steps or min(args.steps, 10)
+        result["cutce"] = bench_cutce(ct, torch, cut_steps, min(args.warmup, 3),
                                       logits_cache=not args.cutce_recompute)
     if not args.no_layer_ops:
-        result["layer_ops"] = bench_layer_ops(ct, torch, args.steps, args.warmup)
+        result["layer_ops"] = bench_layer_ops(ct, torch, min(args.steps, 50), min(args.warmup, 10))
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(ct, torch, attention)
     print(json.dumps(result))
