@@ -35,12 +35,11 @@ the reference and otherwise changes nothing.
 
 from __future__ import annotations
 
-import operator
 
 import torch
 
 from . import _lib
-from .efficient_attention import _mesh_sizes
+from .efficient_attention import _Axes, _integer
 
 _HIDDEN_ALIGN = 128
 # Largest logits cache the operator allocates by itself (f32 [vocab, rows], both padded to 256).
@@ -162,44 +161,38 @@ def pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weig
     targets int32 ``[B, S]``, weights f32 ``[B, S]``; a row is ignored iff its weight is 0.
     """
 
-    if isinstance(local_chunk_size, bool):
-        raise TypeError("local_chunk_size must be a static non-negative integer")
-    try:
-        local_chunk_size = operator.index(local_chunk_size)
-    except TypeError as error:
-        raise TypeError("local_chunk_size must be a static non-negative integer") from error
+    local_chunk_size = _integer(local_chunk_size, "local_chunk_size must be a static non-negative integer")
     if local_chunk_size < 0:
         raise ValueError("local_chunk_size must be non-negative")
-    if hidden_states.ndim != 3:
+    layout_ok = hidden_states.ndim == 3
+    if not layout_ok:
         raise ValueError("Cut cross-entropy expects hidden_states [batch, sequence, hidden]")
-    if lm_head_kernel.ndim != 2 or lm_head_kernel.shape[0] != hidden_states.shape[-1]:
+    batch, sequence, hidden = hidden_states.shape
+    if tuple(lm_head_kernel.shape[:1]) != (hidden,) or lm_head_kernel.ndim != 2:
         raise ValueError("lm_head_kernel must have shape [hidden, vocab]")
     targets = torch.as_tensor(targets, device=hidden_states.device).to(torch.int32)
     weights = torch.as_tensor(weights, device=hidden_states.device).to(torch.float32)
-    if targets.shape != hidden_states.shape[:-1] or weights.shape != targets.shape:
-        raise ValueError("targets and weights must match hidden_states.shape[:-1]")
-    if hidden_states.shape[0] == 0 or hidden_states.shape[1] == 0:
-        raise ValueError("Cut cross-entropy requires at least one token row")
-    if hidden_states.shape[-1] == 0 or hidden_states.shape[-1] % _HIDDEN_ALIGN:
-        raise ValueError("Cut cross-entropy hidden size must be divisible by 128")
-    if lm_head_kernel.shape[1] == 0:
-        raise ValueError("Cut cross-entropy requires a non-empty vocabulary")
-    if hidden_states.dtype != lm_head_kernel.dtype:
-        raise TypeError("hidden_states and lm_head_kernel must use the same compute dtype")
-    if not hidden_states.dtype.is_floating_point:
-        raise TypeError("Cut cross-entropy inputs must have a floating dtype")
-    if hidden_states.dtype != torch.bfloat16:
-        raise TypeError("this build computes Cut cross-entropy in bfloat16 only")
-    if not hidden_states.is_cuda:
-        raise RuntimeError("Cut cross-entropy is available only on a ROCm GPU")
-    sizes = _mesh_sizes(mesh)
-    unsupported = tuple(axis for axis in ("fsdp", "ep") if int(sizes.get(axis, 1)) != 1)
-    if unsupported:
-        raise ValueError(
-            "Cut cross-entropy currently requires fsdp=ep=1; active unsupported axes: "
-            + ", ".join(unsupported)
-        )
-    active = {axis: int(size) for axis, size in sizes.items() if int(size) != 1}
+    for broken, error in (
+        (not (targets.shape == weights.shape == (batch, sequence)),
+         ValueError("targets and weights must match hidden_states.shape[:-1]")),
+        (batch * sequence == 0, ValueError("Cut cross-entropy requires at least one token row")),
+        (hidden == 0 or hidden % _HIDDEN_ALIGN != 0,
+         ValueError("Cut cross-entropy hidden size must be divisible by 128")),
+        (lm_head_kernel.shape[1] == 0, ValueError("Cut cross-entropy requires a non-empty vocabulary")),
+        (lm_head_kernel.dtype != hidden_states.dtype,
+         TypeError("hidden_states and lm_head_kernel must use the same compute dtype")),
+        (not hidden_states.dtype.is_floating_point, TypeError("Cut cross-entropy inputs must have a floating dtype")),
+        (hidden_states.dtype != torch.bfloat16,
+         TypeError("this build computes Cut cross-entropy in bfloat16 only")),
+        (not hidden_states.is_cuda, RuntimeError("Cut cross-entropy is available only on a ROCm GPU")),
+    ):
+        if broken:
+            raise error
+    active = _Axes(mesh).beyond_one_device()
+    sharded_rows = [axis for axis in ("fsdp", "ep") if axis in active]
+    if sharded_rows:
+        raise ValueError("Cut cross-entropy currently requires fsdp=ep=1; active unsupported axes: "
+                         + ", ".join(sharded_rows))
     if active:
         raise ValueError(f"this build runs on one GPU; mesh axes larger than 1: {active}")
     width = hidden_states.shape[-1]

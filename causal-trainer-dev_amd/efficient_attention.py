@@ -67,84 +67,88 @@ class AttentionMetadata(NamedTuple):
     tile_bounds: torch.Tensor | None = None
 
 
-def _shape_tuple(shape: Sequence[int], name: str) -> tuple[int, ...]:
+def _integer(value, complaint: str) -> int:
+    """``value`` as a plain int; anything that is not an integer raises ``TypeError(complaint)``."""
+
+    if isinstance(value, bool):
+        raise TypeError(complaint)
     try:
-        result = tuple(operator.index(dimension) for dimension in shape)
-    except TypeError as error:
-        raise TypeError(f"{name} must be a static integer shape") from error
-    if any(dimension <= 0 for dimension in result):
-        raise ValueError(f"{name} dimensions must be positive, got {result}")
-    return result
+        return operator.index(value)
+    except TypeError:
+        raise TypeError(complaint) from None
 
 
-def _mesh_sizes(mesh) -> Mapping[str, int]:
-    if mesh is None:
-        return {}
-    sizes = getattr(mesh, "shape", mesh)
-    if not isinstance(sizes, Mapping):
-        raise TypeError("mesh_shape must be a Mesh or a mapping of named axis sizes")
-    return sizes
+def _positive(value, name: str) -> int:
+    number = _integer(value, f"{name} must be a static positive integer")
+    if number < 1:
+        raise ValueError(f"{name} must be positive, got {number}")
+    return number
 
 
-def _mesh_size(mesh, axis: str) -> int:
+def _dims(shape: Sequence[int], name: str) -> tuple[int, ...]:
+    complaint = f"{name} must be a static integer shape"
     try:
-        size = operator.index(_mesh_sizes(mesh).get(axis, 1))
-    except TypeError as error:
-        raise TypeError(f"mesh axis {axis!r} must have a static integer size") from error
-    if size <= 0:
-        raise ValueError(f"mesh axis {axis!r} must have a positive size, got {size}")
-    return size
+        entries = list(shape)
+    except TypeError:
+        raise TypeError(complaint) from None
+    dims = tuple(operator.index(entry) if isinstance(entry, bool) else _integer(entry, complaint)
+                 for entry in entries)
+    if any(extent < 1 for extent in dims):
+        raise ValueError(f"{name} dimensions must be positive, got {dims}")
+    return dims
+
+
+class _Axes:
+    """Named axis sizes of a ``mesh`` argument: ``None``, a mapping, or an object whose
+    ``.shape`` is one (the reference passes a jax Mesh, :88-104)."""
+
+    def __init__(self, mesh):
+        table = {} if mesh is None else getattr(mesh, "shape", mesh)
+        if not isinstance(table, Mapping):
+            raise TypeError("mesh_shape must be a Mesh or a mapping of named axis sizes")
+        self.table = table
+
+    def size(self, axis: str) -> int:
+        extent = _integer(self.table.get(axis, 1), f"mesh axis {axis!r} must have a static integer size")
+        if extent < 1:
+            raise ValueError(f"mesh axis {axis!r} must have a positive size, got {extent}")
+        return extent
+
+    def beyond_one_device(self) -> dict[str, int]:
+        return {axis: int(extent) for axis, extent in self.table.items() if int(extent) != 1}
 
 
 def _require_single_device(mesh) -> None:
-    active = {axis: int(size) for axis, size in _mesh_sizes(mesh).items() if int(size) != 1}
+    active = _Axes(mesh).beyond_one_device()
     if active:
         raise ValueError(f"this build runs on one GPU; mesh axes larger than 1: {active}")
 
 
-def _static_positive_int(value, name: str) -> int:
-    if isinstance(value, bool):
-        raise TypeError(f"{name} must be a static positive integer")
-    try:
-        result = operator.index(value)
-    except TypeError as error:
-        raise TypeError(f"{name} must be a static positive integer") from error
-    if result <= 0:
-        raise ValueError(f"{name} must be positive, got {result}")
-    return result
-
-
 def _validate_qkv_shapes(q_shape, kv_shape, mesh):
-    query_shape = _shape_tuple(q_shape, "q_shape")
-    key_value_shape = _shape_tuple(kv_shape, "kv_shape")
-    if len(query_shape) != 4 or len(key_value_shape) != 4:
-        raise ValueError(
-            "attention shapes must be [batch, sequence, heads, dim], got "
-            f"q={query_shape}, kv={key_value_shape}"
-        )
-    if query_shape[:2] != key_value_shape[:2]:
-        raise ValueError(
-            f"Q and KV batch/sequence dimensions must match, got q={query_shape}, kv={key_value_shape}"
-        )
-    if query_shape[-1] != key_value_shape[-1]:
-        raise ValueError(
-            f"Q and KV head dimensions must match, got q={query_shape[-1]}, kv={key_value_shape[-1]}"
-        )
-    if query_shape[2] % key_value_shape[2]:
-        raise ValueError(
-            "query head count must be divisible by the KV head count, got "
-            f"Hq={query_shape[2]}, Hkv={key_value_shape[2]}"
-        )
-    tp_size = _mesh_size(mesh, "tp")
-    sp_size = _mesh_size(mesh, "sp")
-    data_size = _mesh_size(mesh, "dp") * _mesh_size(mesh, "fsdp")
-    if query_shape[0] % data_size:
-        raise ValueError(f"global batch {query_shape[0]} must be divisible by dp*fsdp={data_size}")
-    if query_shape[2] % tp_size:
-        raise ValueError(f"Hq={query_shape[2]} must be divisible by TP={tp_size}")
-    if query_shape[1] % sp_size:
-        raise ValueError(f"sequence={query_shape[1]} must be divisible by SP={sp_size}")
-    return query_shape, key_value_shape, tp_size, sp_size
+    """``(q dims, kv dims, tp, sp)`` after the layout checks of the reference (:107-145)."""
+
+    q, kv = _dims(q_shape, "q_shape"), _dims(kv_shape, "kv_shape")
+    if not (len(q) == len(kv) == 4):
+        raise ValueError(f"attention shapes must be [batch, sequence, heads, dim], got q={q}, kv={kv}")
+    axes = _Axes(mesh)
+    tp, sp = axes.size("tp"), axes.size("sp")
+    replicas = axes.size("dp") * axes.size("fsdp")
+    batch, sequence, heads, width = q
+    for broken, text in (
+        (kv[:2] != (batch, sequence), f"Q and KV batch/sequence dimensions must match, got q={q}, kv={kv}"),
+        (kv[3] != width, f"Q and KV head dimensions must match, got q={width}, kv={kv[3]}"),
+        (heads % kv[2] != 0,
+         f"query head count must be divisible by the KV head count, got Hq={heads}, Hkv={kv[2]}"),
+        (batch % replicas != 0, f"global batch {batch} must be divisible by dp*fsdp={replicas}"),
+        (heads % tp != 0, f"Hq={heads} must be divisible by TP={tp}"),
+        (sequence % sp != 0, f"sequence={sequence} must be divisible by SP={sp}"),
+    ):
+        if broken:
+            raise ValueError(text)
+    return q, kv, tp, sp
+
+
+_PROFILE_TILES = ("block_h", "block_q", "block_kv_outer", "block_kv_compute")
 
 
 def validate_attention_profile(profile, q_shape, kv_shape, mesh_shape) -> None:
@@ -152,83 +156,64 @@ def validate_attention_profile(profile, q_shape, kv_shape, mesh_shape) -> None:
 
     if not isinstance(profile, AttentionKernelProfile):
         raise TypeError(f"profile must be AttentionKernelProfile, got {type(profile).__name__}")
-    if not isinstance(profile.compact_statistics, bool):
+    if type(profile.compact_statistics) is not bool:
         raise TypeError("profile.compact_statistics must be a static bool")
-    query_shape, _, tp_size, sp_size = _validate_qkv_shapes(q_shape, kv_shape, mesh_shape)
-    block_h = _static_positive_int(profile.block_h, "block_h")
-    block_q = _static_positive_int(profile.block_q, "block_q")
-    outer = _static_positive_int(profile.block_kv_outer, "block_kv_outer")
-    compute = _static_positive_int(profile.block_kv_compute, "block_kv_compute")
-    local_heads = query_shape[2] // tp_size
-    local_query = query_shape[1] // sp_size
-    details = (
-        f"q_shape={query_shape}, kv_shape={tuple(kv_shape)}, TP={tp_size}, SP={sp_size}, "
-        f"local_heads={local_heads}, local_query={local_query}, profile={profile}"
-    )
-    if block_h != local_heads:
-        raise ValueError(f"the efficient kernel requires block_h=local_heads; {details}")
-    if block_q % _TILE_ALIGN or local_query % block_q:
-        raise ValueError(f"block_q must be a 128-aligned divisor of local_query; {details}")
-    if outer % _TILE_ALIGN or query_shape[1] % outer:
-        raise ValueError(f"block_kv_outer must be a 128-aligned divisor of sequence; {details}")
-    if compute % _TILE_ALIGN or query_shape[1] % compute:
-        raise ValueError(f"block_kv_compute must be a 128-aligned divisor of sequence; {details}")
-    if compute > outer or outer % compute:
-        raise ValueError(f"block_kv_compute must divide block_kv_outer; {details}")
+    q, kv, tp, sp = _validate_qkv_shapes(q_shape, kv_shape, mesh_shape)
+    heads_h, tile_q, outer, compute = (_positive(getattr(profile, name), name) for name in _PROFILE_TILES)
+    sequence, local_heads, local_query = q[1], q[2] // tp, q[1] // sp
+
+    def tiles(length: int, tile: int) -> bool:
+        return tile % _TILE_ALIGN == 0 and length % tile == 0
+
+    for broken, text in (
+        (heads_h != local_heads, "the efficient kernel requires block_h=local_heads"),
+        (not tiles(local_query, tile_q), "block_q must be a 128-aligned divisor of local_query"),
+        (not tiles(sequence, outer), "block_kv_outer must be a 128-aligned divisor of sequence"),
+        (not tiles(sequence, compute), "block_kv_compute must be a 128-aligned divisor of sequence"),
+        (outer % compute != 0, "block_kv_compute must divide block_kv_outer"),
+    ):
+        if broken:
+            raise ValueError(f"{text}; q_shape={q}, kv_shape={kv}, TP={tp}, SP={sp}, local_heads={local_heads}, "
+                             f"local_query={local_query}, profile={profile}")
 
 
-def _aligned_divisors(length: int, limit: int) -> list[int]:
-    return [b for b in range(_TILE_ALIGN, min(length, limit) + 1, _TILE_ALIGN) if length % b == 0]
+def _pick_tile(length: int, cap: int, complaint: str, nearest_to: float | None = None) -> int:
+    """A 128-aligned divisor of ``length`` not above ``cap``: the largest, or the one nearest to
+    ``nearest_to`` (ties to the smaller)."""
+
+    options = [tile for tile in range(_TILE_ALIGN, min(length, cap) + 1, _TILE_ALIGN) if length % tile == 0]
+    if not options:
+        raise ValueError(complaint)
+    if nearest_to is None:
+        return options[-1]
+    return min(options, key=lambda tile: (abs(tile - nearest_to), tile))
 
 
-def _nearest_query_tile(local_query, local_heads, preferred_rows, max_query_tokens):
-    candidates = _aligned_divisors(local_query, max_query_tokens)
-    if not candidates:
-        raise ValueError(
-            "SP-local query length has no 128-aligned static divisor: "
-            f"local_query={local_query}, local_heads={local_heads}"
-        )
-    target = preferred_rows / local_heads
-    return min(candidates, key=lambda block: (abs(block - target), block))
-
-
-def _largest_aligned_divisor(length: int, preferred: int) -> int:
-    candidates = _aligned_divisors(length, preferred)
-    if not candidates:
-        raise ValueError(
-            f"length has no 128-aligned static divisor: length={length}, preferred={preferred}"
-        )
-    return max(candidates)
+# (longest sequence of the tier, query rows per tile summed over heads, outer KV tile, compute KV tile)
+_TIERS = ((16_384, _ROWS_COMMON, 512, 256), (262_144, _ROWS_LONG, 1024, 256), (None, _ROWS_LONG, 2048, 512))
 
 
 def resolve_attention_profile(q_shape, kv_shape, mesh_shape, *, compact_statistics=False,
                               has_attention_end=False) -> AttentionKernelProfile:
     """Resolve the static profile from global shapes (reference tiers, :251-276)."""
 
-    query_shape, _, tp_size, sp_size = _validate_qkv_shapes(q_shape, kv_shape, mesh_shape)
-    if not isinstance(has_attention_end, bool):
+    q, _, tp, sp = _validate_qkv_shapes(q_shape, kv_shape, mesh_shape)
+    if type(has_attention_end) is not bool:
         raise TypeError("has_attention_end must be a static bool")
-    local_heads = query_shape[2] // tp_size
-    local_query = query_shape[1] // sp_size
-    sequence = query_shape[1]
-    if sequence <= 16_384:
-        rows, outer_pref, compute_pref = _ROWS_COMMON, 512, 256
-    elif sequence <= 262_144:
-        rows, outer_pref, compute_pref = _ROWS_LONG, 1024, 256
-    else:
-        rows, outer_pref, compute_pref = _ROWS_LONG, 2048, 512
+    sequence, local_heads, local_query = q[1], q[2] // tp, q[1] // sp
+    _, rows, outer_cap, compute_cap = next(tier for tier in _TIERS if tier[0] is None or sequence <= tier[0])
     if has_attention_end:
         rows = min(rows, _ROWS_HYBRID)
-    outer = _largest_aligned_divisor(sequence, outer_pref)
-    compute = _largest_aligned_divisor(outer, compute_pref)
-    max_query_tokens = min(_MAX_QUERY_TOKENS, _MAX_QUERY_COMPUTE_ELEMENTS // compute)
-    profile = AttentionKernelProfile(
-        block_h=local_heads,
-        block_q=_nearest_query_tile(local_query, local_heads, rows, max_query_tokens),
-        block_kv_outer=outer,
-        block_kv_compute=compute,
-        compact_statistics=compact_statistics,
-    )
+    outer = _pick_tile(sequence, outer_cap,
+                       f"length has no 128-aligned static divisor: length={sequence}, preferred={outer_cap}")
+    compute = _pick_tile(outer, compute_cap,
+                         f"length has no 128-aligned static divisor: length={outer}, preferred={compute_cap}")
+    tile_q = _pick_tile(local_query, min(_MAX_QUERY_TOKENS, _MAX_QUERY_COMPUTE_ELEMENTS // compute),
+                        "SP-local query length has no 128-aligned static divisor: "
+                        f"local_query={local_query}, local_heads={local_heads}",
+                        nearest_to=rows / local_heads)
+    profile = AttentionKernelProfile(block_h=local_heads, block_q=tile_q, block_kv_outer=outer,
+                                     block_kv_compute=compute, compact_statistics=compact_statistics)
     validate_attention_profile(profile, q_shape, kv_shape, mesh_shape)
     return profile
 
@@ -236,7 +221,7 @@ def resolve_attention_profile(q_shape, kv_shape, mesh_shape, *, compact_statisti
 def default_attention_scale(head_dim: int) -> float:
     """``head_dim ** -0.5`` (reference :282-286)."""
 
-    return _static_positive_int(head_dim, "head_dim") ** -0.5
+    return _positive(head_dim, "head_dim") ** -0.5
 
 
 def _as_device_int32(value, name: str) -> torch.Tensor:
@@ -271,8 +256,8 @@ def prepare_attention_metadata(canonical_segment_ids, *, mesh, profile,
         raise ValueError(f"canonical_segment_ids must be [batch, sequence], got {tuple(segments.shape)}")
     if segments.shape[0] == 0 or segments.shape[1] == 0:
         raise ValueError("canonical_segment_ids must have non-empty batch and sequence dimensions")
-    block_q = _static_positive_int(profile.block_q, "profile.block_q")
-    outer = _static_positive_int(profile.block_kv_outer, "profile.block_kv_outer")
+    block_q = _positive(profile.block_q, "profile.block_q")
+    outer = _positive(profile.block_kv_outer, "profile.block_kv_outer")
     batch, sequence = segments.shape
     if sequence % block_q or sequence % outer:
         raise ValueError(
@@ -317,24 +302,36 @@ def _validate_metadata(metadata, query_shape, profile) -> None:
     if not isinstance(metadata, AttentionMetadata):
         raise TypeError("metadata must be AttentionMetadata")
     batch, sequence = query_shape[:2]
-    expected = {
-        "query_segment_ids": (batch, sequence),
-        "kv_segment_ids": (batch, sequence),
-        "q_block_segments": (batch, sequence // profile.block_q,
-                             3 if metadata.attention_end is not None else 2),
-        "kv_block_segments": (batch, sequence // profile.block_kv_outer, 2),
-    }
-    if metadata.attention_end is not None:
-        expected["attention_end"] = (batch, sequence)
-    for name, shape in expected.items():
-        value = getattr(metadata, name)
-        if tuple(value.shape) != shape:
-            raise ValueError(f"metadata.{name} must have shape {shape}, got {tuple(value.shape)}")
-        if value.dtype != torch.int32:
-            raise TypeError(f"metadata.{name} must have dtype int32, got {value.dtype}")
-    expected_bytes = _lib.load().ct_attn_meta_bytes(batch, sequence)
-    if metadata.tile_bounds is None or metadata.tile_bounds.numel() * 4 != expected_bytes:
+    hybrid = metadata.attention_end is not None
+    layout = [("query_segment_ids", (batch, sequence)), ("kv_segment_ids", (batch, sequence)),
+              ("q_block_segments", (batch, sequence // profile.block_q, 3 if hybrid else 2)),
+              ("kv_block_segments", (batch, sequence // profile.block_kv_outer, 2))]
+    if hybrid:
+        layout.append(("attention_end", (batch, sequence)))
+    for name, shape in layout:
+        tensor = getattr(metadata, name)
+        if tuple(tensor.shape) != shape:
+            raise ValueError(f"metadata.{name} must have shape {shape}, got {tuple(tensor.shape)}")
+        if tensor.dtype != torch.int32:
+            raise TypeError(f"metadata.{name} must have dtype int32, got {tensor.dtype}")
+    table = metadata.tile_bounds
+    if table is None or table.numel() * 4 != _lib.load().ct_attn_meta_bytes(batch, sequence):
         raise ValueError("metadata.tile_bounds is missing; build it with prepare_attention_metadata")
+
+
+def _python_scalar(scale) -> float:
+    """A static softmax scale as a finite float (the reference rejects traced values, :1950-1957)."""
+
+    complaint = "scale must be a compile-time Python scalar"
+    if isinstance(scale, torch.Tensor):
+        raise TypeError(complaint)
+    try:
+        number = float(scale)
+    except (TypeError, ValueError):
+        raise TypeError(complaint) from None
+    if math.isinf(number) or math.isnan(number):
+        raise ValueError(f"scale must be finite, got {number}")
+    return number
 
 
 def _attn_forward(query, key, value, metadata, scale):
@@ -433,17 +430,7 @@ def efficient_attention(query, key, value, metadata, *, mesh=None, profile=None,
     )
     validate_attention_profile(resolved_profile, query_shape, key_shape, mesh)
     _validate_metadata(metadata, query_shape, resolved_profile)
-    if scale is None:
-        resolved_scale = default_attention_scale(query_shape[-1])
-    else:
-        if isinstance(scale, torch.Tensor):
-            raise TypeError("scale must be a compile-time Python scalar")
-        try:
-            resolved_scale = float(scale)
-        except (TypeError, ValueError) as error:
-            raise TypeError("scale must be a compile-time Python scalar") from error
-        if not math.isfinite(resolved_scale):
-            raise ValueError(f"scale must be finite, got {resolved_scale}")
+    resolved_scale = default_attention_scale(query_shape[-1]) if scale is None else _python_scalar(scale)
     return _EfficientAttention.apply(
         query.contiguous(), key.contiguous(), value.contiguous(), metadata, resolved_scale
     )
