@@ -104,6 +104,20 @@ def bench_attention(ct, torch, steps, warmup):
 
     elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
     ms_per_step = elapsed / steps * 1e3
+
+    # The delta pass (HBM bound) is part of the dQ kernel in the backward; its rate as a pass of
+    # its own is measured here through its own entry point, outside the timed step.
+    out, _ = ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
+    rows = out.numel() // config.head_dim
+    delta = torch.empty(rows, dtype=torch.float32, device="cuda")
+
+    def delta_pass():
+        ct._lib.check(ct._lib.load().ct_attn_delta(ct._lib.current_stream(), out.data_ptr(), dout.data_ptr(),
+                                                   delta.data_ptr(), rows, config.head_dim))
+
+    _, delta_kernels = timed_region(torch, delta_pass, min(steps, 50), min(warmup, 10), ct.profiling.KernelTimer)
+    kernels = dict(kernels)
+    kernels["attn_delta_kernel"] = delta_kernels["attn_delta_kernel"]
     per_kernel_flops = {
         "attn_fwd_kernel": flops["fwd"],
         # backward = 5 GEMMs: dQ owns S recompute share + dP share + dQ; counted as executed-free
@@ -118,6 +132,7 @@ def bench_attention(ct, torch, steps, warmup):
             entry["algorithmic_tflops"] = per_kernel_flops[name] / (entry["avg_ms"] * 1e-3) / 1e12
         if name == "attn_delta_kernel":
             entry["algorithmic_gbps"] = W.attention_delta_bytes(config) / (entry["avg_ms"] * 1e-3) / 1e9
+            entry["note"] = "pass on its own (ct_attn_delta), not a launch of the timed step"
         table.append(entry)
     return {
         "config": config, "pairs": pairs, "flops": flops, "ms_per_step": ms_per_step,
@@ -152,6 +167,7 @@ def bench_cutce(ct, torch, steps, warmup, logits_cache=True):
 
     elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
     ms_per_step = elapsed / steps * 1e3
+
     gemm = 2 * active * config.hidden * config.vocab
     per_kernel_flops = {"cutce_stats_kernel": gemm, "cutce_dhidden_kernel": gemm, "cutce_dhead_kernel": gemm}
     table = []

@@ -337,12 +337,7 @@ static int launch_dkv(hipStream_t stream, const AttnParams& p) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
   }
-  LaunchScope scope7("attn_dkv_schedule_kernel", stream);
-  hipLaunchKernelGGL(attn_dkv_schedule_kernel, dim3(1), dim3(1024), 0, stream, p.meta, p.B, p.S,
-                     p.Hkv, p.Hq / p.Hkv, p.dkv_max_entries, p.dkv_max_partials, p.dkv_header,
-                     p.dkv_entries);
-  int rc = scope7.done();
-  if (rc) return rc;
+  int rc = 0;
   const int grid = p.dkv_max_entries * p.Hkv;  // entries beyond the list's length exit at once
   LaunchScope scope3("attn_dkv_kernel", stream);
   hipLaunchKernelGGL((attn_dkv_kernel<D>), dim3(grid), dim3(256), smem, stream, p);
@@ -353,27 +348,25 @@ static int launch_dkv(hipStream_t stream, const AttnParams& p) {
   return scope9.done();
 }
 
-// lse2 == nullptr: delta in row order (b, s, h); otherwise delta and lse * log2(e) head-major.
+// The delta pass on its own: delta in row order (b, s, h).
 template <int D>
-static int launch_delta(hipStream_t stream, const bf16* out, const bf16* dout, float* delta,
-                        long rows, const float* lse = nullptr, float* lse2 = nullptr, int S = 0,
-                        int Hq = 0, int* zeroed = nullptr, int zeroed_count = 0) {
+static int launch_delta(hipStream_t stream, const bf16* out, const bf16* dout, float* delta, long rows) {
   const long threads = rows * (D / 8);
   const dim3 grid((unsigned)((threads + 255) / 256));
   LaunchScope scope4("attn_delta_kernel", stream);
-  if (lse2)
-    hipLaunchKernelGGL((attn_delta_kernel<D, true>), grid, dim3(256), 0, stream, out, dout, delta,
-                       rows, lse, lse2, S, Hq, zeroed, zeroed_count);
-  else
-    hipLaunchKernelGGL((attn_delta_kernel<D, false>), grid, dim3(256), 0, stream, out, dout, delta,
-                       rows, lse, lse2, S, Hq);
+  hipLaunchKernelGGL((attn_delta_kernel<D>), grid, dim3(256), 0, stream, out, dout, delta, rows);
   return scope4.done();
 }
 
 template <int D>
 static int dispatch_bwd(hipStream_t stream, const AttnParams& p) {
-  int rc = launch_delta<D>(stream, p.out, p.dout, p.delta, (long)p.B * p.S * p.Hq, p.lse, p.lse2,
-                           p.S, p.Hq, p.dq_counters, kDqCounters);
+  // The work list of dK/dV depends on the metadata only: built first, by the launch that also
+  // clears dQ's work counters. dQ computes delta and lse * log2(e) for its rows on the way.
+  LaunchScope scope7("attn_dkv_schedule_kernel", stream);
+  hipLaunchKernelGGL(attn_dkv_schedule_kernel, dim3(1), dim3(1024), 0, stream, p.meta, p.B, p.S,
+                     p.Hkv, p.Hq / p.Hkv, p.dkv_max_entries, p.dkv_max_partials, p.dkv_header,
+                     p.dkv_entries, p.dq_counters, kDqCounters);
+  int rc = scope7.done();
   if (rc) return rc;
   switch (heads_per_group(p.Hq, p.Hkv)) {
     case 4: rc = launch_dq<D, 4>(stream, p); break;

@@ -44,14 +44,15 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
   const size_t stat_t = ((size_t)ctx.work.b * p.Hq + ctx.work.h) * p.S + ctx.pos;  // head-major
-  const float lse2 = p.lse2[stat_t];
-  const float delta_q = p.delta[stat_t];
+  const float lse2 = p.lse[ctx.stat_off] * kLog2e;
 
   bf16x8 qf[D / 16], dof[D / 16];
+  u32x4 of[D / 16];  // this row's half of `out`, for delta
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) {
     qf[ks] = scale_bf16x8(as_bf16x8(load_global16(p.q + ctx.q_off + 16 * ks + 8 * half)), p.scale);
     dof[ks] = as_bf16x8(load_global16(p.dout + ctx.q_off + 16 * ks + 8 * half));
+    of[ks] = load_global16(p.out + ctx.q_off + 16 * ks + 8 * half);
   }
   f32x16 dqacc[D / 32];
 #pragma unroll
@@ -66,6 +67,28 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
   }
   dma_wait_all();
   __syncthreads();
+
+  // delta = sum_d out[row, d] * dout[row, d], after the wait above so that the first key tile's
+  // copies are not held back behind these loads; the dK/dV kernel, launched after this one, reads
+  // delta and lse * log2(e) head-major
+  float delta_part = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) {
+    u32x4 o_bits = of[ks];
+    asm volatile("" : "+v"(o_bits));
+    const u32x4 do_bits = __builtin_bit_cast(u32x4, dof[ks]);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      delta_part = fmaf(__uint_as_float(o_bits[e] << 16), __uint_as_float(do_bits[e] << 16), delta_part);
+      delta_part = fmaf(__uint_as_float(o_bits[e] & 0xffff0000u), __uint_as_float(do_bits[e] & 0xffff0000u),
+                        delta_part);
+    }
+  }
+  const float delta_q = pair_sum(delta_part);
+  if (ctx.active && half == 0) {
+    p.delta[stat_t] = delta_q;
+    p.lse2[stat_t] = lse2;
+  }
 
   auto step = [&](auto stage_tag) {
     constexpr int CUR = decltype(stage_tag)::value;
@@ -319,7 +342,9 @@ CT_DEVICE int dkv_split_count(int items, int target) {
 __global__ __launch_bounds__(1024) void attn_dkv_schedule_kernel(const int* meta, int B, int S,
                                                                  int Hkv, int g, int max_entries,
                                                                  int max_partials, int* header,
-                                                                 int2* entries) {
+                                                                 int2* entries, int* zeroed,
+                                                                 int zeroed_count) {
+  for (int i = threadIdx.x; i < zeroed_count; i += 1024) zeroed[i] = 0;  // dQ's work counters
   __shared__ long long red[1024];
   __shared__ int hist[256];
   __shared__ int fill[256];

@@ -44,8 +44,8 @@ struct AttnParams {
   bf16* out;        // forward: written; backward: forward output
   float* lse;
   const bf16* dout;
-  float* delta;     // backward: rowsum(out * dout), head-major [B, Hq, S]
-  float* lse2;      // backward: lse * log2(e), head-major [B, Hq, S]
+  float* delta;     // backward: rowsum(out * dout), head-major [B, Hq, S] (written by dQ, read by dK/dV)
+  float* lse2;      // backward: lse * log2(e), head-major [B, Hq, S] (written by dQ, read by dK/dV)
   bf16* dq;
   bf16* dk;
   bf16* dv;
@@ -54,7 +54,7 @@ struct AttnParams {
   // dK/dV work list (backward only)
   int* dkv_header;
   int2* dkv_entries;
-  int* dq_counters;  // kDqCounters ints, zeroed by the delta pass of the same call
+  int* dq_counters;  // kDqCounters ints, zeroed by the work-list kernel of the same call
   float* dkv_partials;
   int dkv_max_entries, dkv_max_partials;
 };
@@ -565,19 +565,16 @@ attn_fwd_kernel(AttnParams p) {
 
 // ---------------------------------------------------------------------------
 // delta[row] = sum_d f32(out[row, d]) * f32(dout[row, d])      (HBM bound)
-// One 16-byte load per lane per tensor; D/8 lanes share a row.
-// HEAD_MAJOR: rows are (b, s, h) flattened; the result goes to [B, Hq, S] order together
-// with lse * log2(e), so that the backward kernels read the 32 rows of a query block of one
-// head as 128 contiguous bytes.
+// One 16-byte load per lane per tensor; D/8 lanes share a row; rows are (b, s, h) flattened.
+// The backward does not launch this kernel: its dQ kernel computes delta for the rows of each
+// query tile from the dO fragments it loads anyway (one read of `out` instead of a pass over
+// `out` and `dout`). This is the pass on its own, behind ct_attn_delta.
 // ---------------------------------------------------------------------------
-template <int D, bool HEAD_MAJOR>
+template <int D>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* out, const bf16* dout,
-                                                         float* delta, long rows, const float* lse,
-                                                         float* lse2, int S, int Hq, int* zeroed = nullptr,
-                                                         int zeroed_count = 0) {
+                                                         float* delta, long rows) {
   constexpr int LPR = D / 8;  // lanes per row
   const long gid = (long)blockIdx.x * 256 + threadIdx.x;
-  if (zeroed && gid < zeroed_count) zeroed[gid] = 0;  // work counters of the kernel that follows
   const long row = gid / LPR;
   const int c = gid % LPR;
   float acc = 0.f;
@@ -589,18 +586,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* out, const 
   }
 #pragma unroll
   for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-  if (row < rows && c == 0) {
-    if constexpr (HEAD_MAJOR) {
-      const long bs = row / Hq;
-      const int h = (int)(row % Hq);
-      const long b = bs / S, pos = bs % S;
-      const long dst = (b * Hq + h) * S + pos;
-      delta[dst] = acc;
-      lse2[dst] = lse[row] * kLog2e;
-    } else {
-      delta[row] = acc;
-    }
-  }
+  if (row < rows && c == 0) delta[row] = acc;
 }
 
 }  // namespace ct

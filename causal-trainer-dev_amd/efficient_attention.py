@@ -352,7 +352,7 @@ def _attn_forward(query, key, value, metadata, scale):
     return out, lse
 
 
-def _attn_backward(query, key, value, metadata, out, lse, dout, scale):
+def _attn_backward(query, key, value, metadata, out, lse, dout, scale, with_delta=False):
     batch, sequence, q_heads, head_dim = query.shape
     dq = torch.empty_like(query)
     dk = torch.empty_like(key)
@@ -373,6 +373,8 @@ def _attn_backward(query, key, value, metadata, out, lse, dout, scale):
     )
     with torch.cuda.device(query.device):
         _lib.check(_lib.load().ct_attn_bwd(_lib.current_stream(), args))
+    if with_delta:
+        return dq, dk, dv, delta.view(batch, q_heads, sequence)
     return dq, dk, dv
 
 
@@ -443,11 +445,12 @@ def attention_forward_with_lse(query, key, value, metadata, *, scale=None):
     return _attn_forward(query.contiguous(), key.contiguous(), value.contiguous(), metadata, resolved)
 
 
-def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=None):
-    """Backward only, from the saved residuals: returns ``(dq, dk, dv)``."""
+def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=None, with_delta=False):
+    """Backward only, from the saved residuals: returns ``(dq, dk, dv)``; with ``with_delta`` also the
+    scratch ``delta = rowsum(out * dout)`` as the kernels leave it, head-major ``[B, Hq, S]``."""
 
     resolved = default_attention_scale(query.shape[-1]) if scale is None else float(scale)
-    return _attn_backward(query, key, value, metadata, out, lse, dout.contiguous(), resolved)
+    return _attn_backward(query, key, value, metadata, out, lse, dout.contiguous(), resolved, with_delta)
 
 
 __all__ = [

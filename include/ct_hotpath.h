@@ -157,16 +157,18 @@ size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t q_heads, 
 
 /*
  * dq, dk, dv from the saved (q, k, v, out, lse) and dout. Four launches:
- * delta = rowsum(out * dout); dq per query tile; the dK/dV work list; dk/dv
- * per key tile (chunks of a split tile are summed in a fixed order, so the
- * result is deterministic).
+ * the dK/dV work list; dq per query tile, which also computes
+ * delta = rowsum(out * dout) for its rows; dk/dv per key tile; the sum of the
+ * chunks of split key tiles (in a fixed order, so the result is
+ * deterministic).
  * Replaces: delta at src/kernels/efficient_attention.py:1735-1738,
  * _local_attention_dq (:985-1267), _local_attention_dkv (:1270-1602) and the
  * f32 -> bf16 cast at :1774.
  */
 int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* args);
 
-/* The delta pass alone (exposed so it can be measured by itself). */
+/* The delta pass as a pass of its own (ct_attn_bwd computes delta inside its dQ kernel; this
+ * entry exists so that the HBM-bound pass can be measured and tested by itself). */
 int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16_t* dout,
                       float* delta, int64_t rows, int32_t head_dim);
 

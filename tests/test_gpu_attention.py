@@ -295,6 +295,30 @@ def test_delta_pass_matches_torch(ct, gpu):
         torch.testing.assert_close(delta, expected, atol=1e-4, rtol=1e-5)
 
 
+def test_backward_leaves_delta_and_matches_the_pass_on_its_own(ct, gpu):
+    """The backward forms delta = rowsum(out * dout) inside its dQ kernel (head-major scratch);
+    it has to agree with the closed form on every row, padding rows and hybrid ends included."""
+
+    rng = np.random.default_rng(67)
+    for (batch, seq, hq, hkv, dim, hybrid) in ((2, 256, 4, 1, 128, False), (1, 384, 8, 2, 64, True),
+                                                (2, 128, 2, 2, 128, False)):
+        ids = _layout(rng, batch, seq, holes=True)
+        ends = _random_ends(rng, ids) if hybrid else None
+        q = _bf16(rng.standard_normal((batch, seq, hq, dim)))
+        k = _bf16(rng.standard_normal((batch, seq, hkv, dim)))
+        v = _bf16(rng.standard_normal((batch, seq, hkv, dim)))
+        dout = _bf16(rng.standard_normal((batch, seq, hq, dim)))
+        profile = ct.resolve_attention_profile(q.shape, k.shape, None, has_attention_end=hybrid)
+        metadata = ct.prepare_attention_metadata(
+            torch.from_numpy(ids).to(gpu), mesh=None, profile=profile,
+            attention_end=None if ends is None else torch.from_numpy(ends).to(gpu))
+        qd, kd, vd, dod = (t.to(gpu) for t in (q, k, v, dout))
+        out, lse = ct.attention_forward_with_lse(qd, kd, vd, metadata, scale=dim ** -0.5)
+        *_, delta = ct.attention_backward(qd, kd, vd, metadata, out, lse, dod, scale=dim ** -0.5, with_delta=True)
+        expected = (out.float() * dod.float()).sum(-1).permute(0, 2, 1)  # [B, Hq, S]
+        torch.testing.assert_close(delta, expected, atol=1e-4, rtol=1e-5)
+
+
 def _self_contained_window(ids_row, limit):
     """Largest run of whole segments (and padding) of at most `limit` positions: (start, stop)."""
 
