@@ -345,27 +345,58 @@ __global__ __launch_bounds__(1024) void attn_dkv_schedule_kernel(const int* meta
                                                                  int2* entries, int* zeroed,
                                                                  int zeroed_count) {
   for (int i = threadIdx.x; i < zeroed_count; i += 1024) zeroed[i] = 0;  // dQ's work counters
-  __shared__ long long red[1024];
+  __shared__ long long red[16];  // one value per wavefront
   __shared__ int hist[256];
   __shared__ int fill[256];
   __shared__ int carry;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int nrb = S / 32, ntiles = B * (nrb / 4);
 
+  // Reductions and scans run inside the wavefronts (lane shuffles) and meet once in LDS: the
+  // kernel is one workgroup on an otherwise idle GPU, so its time is its chain of barriers.
   auto block_sum = [&](long long v) {
-    red[tid] = v;
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    if (lane == 0) red[wave] = v;
     __syncthreads();
-    for (int s = 512; s > 0; s >>= 1) {
-      if (tid < s) red[tid] += red[tid + s];
-      __syncthreads();
-    }
-    const long long out = red[0];
+    long long out = 0;
+    for (int i = 0; i < 16; ++i) out += red[i];
     __syncthreads();
     return out;
   };
+  auto block_max = [&](int v) {
+    for (int off = 32; off > 0; off >>= 1) v = max(v, __shfl_xor(v, off, 64));
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    int out = (int)red[0];
+    for (int i = 1; i < 16; ++i) out = max(out, (int)red[i]);
+    __syncthreads();
+    return out;
+  };
+  // exclusive prefix of v over the workgroup's threads, and the total
+  auto block_scan = [&](int v, int* total) {
+    int inc = v;
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(inc, off, 64);
+      if (lane >= off) inc += up;
+    }
+    if (lane == 63) red[wave] = inc;
+    __syncthreads();
+    int before = 0, all = 0;
+    for (int i = 0; i < 16; ++i) {
+      const int part = (int)red[i];
+      if (i < wave) before += part;
+      all += part;
+    }
+    __syncthreads();
+    *total = all;
+    return before + inc - v;
+  };
+  // this thread's first tile is read once; further tiles (more than 1024) are re-read per pass
+  const int items_first = tid < ntiles ? dkv_tile_items(meta, nrb, tid, g) : 0;
+  auto items_of = [&](int t) { return t == tid ? items_first : dkv_tile_items(meta, nrb, t, g); };
 
   long long local = 0;
-  for (int t = tid; t < ntiles; t += 1024) local += dkv_tile_items(meta, nrb, t, g);
+  for (int t = tid; t < ntiles; t += 1024) local += items_of(t);
   const long long total = block_sum(local);
   long long want = (total * Hkv + kDkvSlots - 1) / kDkvSlots;  // one compute slot's fair share
   int target = (int)min((long long)INT_MAX / 2, max((long long)kDkvMinChunk, want));
@@ -377,20 +408,13 @@ __global__ __launch_bounds__(1024) void attn_dkv_schedule_kernel(const int* meta
     long long counts = 0;  // entries in the high half, partial slots in the low half
     int local_max = 1;
     for (int t = tid; t < ntiles; t += 1024) {
-      const int items = dkv_tile_items(meta, nrb, t, g);
+      const int items = items_of(t);
       const int ns = dkv_split_count(items, target);
       counts += ((long long)ns << 32) + (ns > 1 ? ns : 0);
       local_max = max(local_max, (items + ns - 1) / ns);
     }
     const long long both = block_sum(counts);
-    red[tid] = local_max;
-    __syncthreads();
-    for (int s = 512; s > 0; s >>= 1) {
-      if (tid < s) red[tid] = max(red[tid], red[tid + s]);
-      __syncthreads();
-    }
-    max_work = (int)red[0];
-    __syncthreads();
+    max_work = block_max(local_max);
     if ((both >> 32) <= max_entries && (both & 0xffffffffll) <= max_partials) break;
     target = target >= INT_MAX / 4 ? INT_MAX / 2 : target * 2;
   }
@@ -404,21 +428,20 @@ __global__ __launch_bounds__(1024) void attn_dkv_schedule_kernel(const int* meta
   __syncthreads();
   auto bucket_of = [&](int work) { return 255 - (int)((long long)work * 255 / max_work); };
   for (int t = tid; t < ntiles; t += 1024) {
-    const int items = dkv_tile_items(meta, nrb, t, g);
+    const int items = items_of(t);
     const int ns = dkv_split_count(items, target);
     const int per = (items + ns - 1) / ns;
     for (int c = 0; c < ns; ++c) atomicAdd(&hist[bucket_of(max(0, min(per, items - c * per)))], 1);
   }
   __syncthreads();
-  if (tid == 0) {
-    int run = 0;
-    for (int i = 0; i < 256; ++i) {
-      const int n = hist[i];
-      hist[i] = run;
-      run += n;
+  {
+    int entries_total = 0;
+    const int start = block_scan(tid < 256 ? hist[tid] : 0, &entries_total);
+    if (tid < 256) hist[tid] = start;  // bucket -> first position in the list
+    if (tid == 0) {
+      header[0] = entries_total;
+      header[1] = target;
     }
-    header[0] = run;
-    header[1] = target;
   }
   __syncthreads();
 
@@ -427,20 +450,12 @@ __global__ __launch_bounds__(1024) void attn_dkv_schedule_kernel(const int* meta
     const int t = base + tid;
     int items = 0, ns = 1;
     if (t < ntiles) {
-      items = dkv_tile_items(meta, nrb, t, g);
+      items = items_of(t);
       ns = dkv_split_count(items, target);
     }
     const int mine = (t < ntiles && ns > 1) ? ns : 0;
-    red[tid] = mine;
-    __syncthreads();
-    for (int s = 1; s < 1024; s <<= 1) {
-      const long long add = tid >= s ? red[tid - s] : 0;
-      __syncthreads();
-      red[tid] += add;
-      __syncthreads();
-    }
-    const int slot0 = carry + (int)red[tid] - mine;
-    const int chunk_total = (int)red[1023];
+    int chunk_total = 0;
+    const int slot0 = carry + block_scan(mine, &chunk_total);
     __syncthreads();
     if (tid == 0) carry += chunk_total;
     if (t < ntiles) {
