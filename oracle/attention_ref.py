@@ -27,6 +27,11 @@ Functions and what they follow:
   efficient_backward         src/kernels/efficient_attention.py:1015-1048, :1170-1173,
                              :1294-1343, :1735-1738, :1774
   attention_f64              float64 evaluation of the same mathematics, for error budgets
+  segment_sampled_rows       the same analytic forward/backward (:586-591, :746-760, :1015-1048,
+                             :1294-1343, :1735-1738) restricted to sampled rows of one long
+                             segment, evaluated in query chunks so that segments of tens of
+                             thousands of positions fit in memory; pinned against
+                             efficient_forward / efficient_backward on short segments
   attention_end_from_blocks  src/data/maskgit.py:106, :116
 """
 
@@ -315,6 +320,65 @@ def attention_f64(query, key, value, allowed, *, scale: float, dout=None):
     dk = dk.reshape(batch, seq, kv_heads, groups, dim).sum(dim=3)
     dv = dv.reshape(batch, seq, kv_heads, groups, dim).sum(dim=3)
     return out, lse, dq, dk, dv
+
+
+def segment_sampled_rows(query, key, value, dout, ends, *, scale: float, query_rows, key_rows,
+                         chunk: int = 2048):
+    """Sampled rows of one segment of length L that shares one KV head.
+
+    ``query`` / ``dout``: bf16 [L, G, D] (the G query heads of the KV head); ``key`` / ``value``:
+    bf16 [L, D]; ``ends``: int [L], last visible key of each query (``arange(L)`` for plain
+    causal), positions relative to the segment. Every position belongs to the segment.
+
+    Returns (out [Rq, G, D] f32, lse [Rq, G] f32, dq [Rq, G, D] f32, dk [Rk, D] f32,
+    dv [Rk, D] f32) for the query positions ``query_rows`` and key positions ``key_rows``,
+    following the reference kernel's analytic backward: delta from the bf16-rounded output,
+    f32 scores from bf16(q * bf16(scale)), natural-log LSE. dK / dV need every query of the
+    segment, so the whole forward is evaluated, chunk by chunk.
+    """
+
+    length, groups, dim = query.shape
+    qs = _scaled_query_f32(query, scale)                      # [L, G, D]
+    kf, vf, do = key.float(), value.float(), dout.float()
+    ends_t = torch.as_tensor(np.asarray(ends)).long()
+    query_rows = torch.as_tensor(np.asarray(query_rows)).long()
+    key_rows = torch.as_tensor(np.asarray(key_rows)).long()
+    scale_f32 = float(torch.tensor(scale, dtype=torch.bfloat16).float())
+    out_rows = torch.zeros((len(query_rows), groups, dim))
+    lse_rows = torch.zeros((len(query_rows), groups))
+    dq_rows = torch.zeros((len(query_rows), groups, dim))
+    dk_rows = torch.zeros((len(key_rows), dim))
+    dv_rows = torch.zeros((len(key_rows), dim))
+    k_sel, v_sel = kf[key_rows], vf[key_rows]
+    for start in range(0, length, chunk):
+        stop = min(length, start + chunk)
+        reach = int(ends_t[start:stop].max()) + 1             # keys any query of the chunk can see
+        visible = torch.arange(reach)[None, :] <= ends_t[start:stop, None]          # [c, reach]
+        in_chunk = (query_rows >= start) & (query_rows < stop)
+        local = query_rows[in_chunk] - start
+        sel_visible = key_rows[None, :] <= ends_t[start:stop, None]                  # [c, Rk]
+        for head in range(groups):
+            scores = qs[start:stop, head] @ kf[:reach].T                             # [c, reach]
+            masked = torch.where(visible, scores, float("-inf"))
+            row_max = masked.amax(dim=-1, keepdim=True)
+            total = torch.exp(masked - row_max).sum(dim=-1, keepdim=True)
+            lse = torch.log(total) + row_max                                          # [c, 1]
+            prob = torch.exp(masked - lse)                                            # 0 where masked
+            out = prob @ vf[:reach]                                                   # [c, D]
+            delta = (_bf16(out).float() * do[start:stop, head]).sum(dim=-1, keepdim=True)
+            if len(local):
+                p_rows = prob[local]
+                dprob = do[start:stop, head][local] @ vf[:reach].T
+                dscore = p_rows * (dprob - delta[local])
+                out_rows[in_chunk, head] = out[local]
+                lse_rows[in_chunk, head] = lse[local, 0]
+                dq_rows[in_chunk, head] = (dscore @ kf[:reach]) * scale_f32
+            # sampled key columns, every query of the chunk
+            p_cols = torch.where(sel_visible, torch.exp(qs[start:stop, head] @ k_sel.T - lse), 0.0)
+            ds_cols = p_cols * (do[start:stop, head] @ v_sel.T - delta)
+            dv_rows += p_cols.T @ do[start:stop, head]
+            dk_rows += ds_cols.T @ qs[start:stop, head]
+    return out_rows, lse_rows, dq_rows, dk_rows, dv_rows
 
 
 def relative_l2(actual, expected) -> float:

@@ -319,6 +319,42 @@ def test_backward_leaves_delta_and_matches_the_pass_on_its_own(ct, gpu):
         torch.testing.assert_close(delta, expected, atol=1e-4, rtol=1e-5)
 
 
+def test_split_key_tiles_match_oracle(ct, gpu):
+    """One 2048-position segment, one KV head, a small batch: the dK/dV work list is far below
+    one compute slot's share, so the chunk target sits at its minimum and the key tiles with the
+    longest query lists are split into several chunks whose f32 partial sums the reduce kernel
+    adds. Checked against the oracle like any other case, and for run-to-run equality."""
+
+    rng = np.random.default_rng(71)
+    batch, seq, q_heads, kv_heads, dim = 1, 2048, 2, 1, 128
+    ids = np.ones((batch, seq), np.int32)
+    ids[0, 2000:] = 0
+    q = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    k = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    v = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    dout = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    # 16 key tiles of 128; the first has (2048 / 32) * 2 = 128 (head, query block) items against
+    # a minimum chunk of 16: it is cut into 8 chunks
+    results = _run_gpu(ct, gpu, q, k, v, dout, ids, None, dim ** -0.5)
+    _check_against_oracle(results, q, k, v, dout, ids, None, dim ** -0.5)
+    again = _run_gpu(ct, gpu, q, k, v, dout, ids, None, dim ** -0.5)
+    for a, b in zip(results, again):
+        assert torch.equal(a, b)
+
+
+def _longest_segment(ids):
+    """(batch row, start, stop) of the longest run of one nonzero id."""
+
+    best = (0, 0, 0)
+    for row in range(ids.shape[0]):
+        cuts = np.flatnonzero(np.diff(ids[row])) + 1
+        edges = np.concatenate(([0], cuts, [ids.shape[1]]))
+        for a, c in zip(edges[:-1], edges[1:]):
+            if ids[row, a] != 0 and c - a > best[2] - best[1]:
+                best = (row, int(a), int(c))
+    return best
+
+
 def _self_contained_window(ids_row, limit):
     """Largest run of whole segments (and padding) of at most `limit` positions: (start, stop)."""
 
@@ -368,3 +404,28 @@ def test_benchmark_shapes(ct, gpu, name):
     got = (out[b:b + 1, window, heads], lse[b:b + 1, window, heads], dq[b:b + 1, window, heads],
            dk[b:b + 1, window, kvh:kvh + 1], dv[b:b + 1, window, kvh:kvh + 1])
     _check_against_oracle(got, q, k, v, dout, w_ids, w_ends, config.scale)
+
+    # The longest segment of the batch (up to the whole sequence): 64 sampled query rows with
+    # every head of the group for O, LSE and dQ; 64 sampled key rows for dK and dV, which sum
+    # over every query of the segment and every head of the group.
+    b, start, stop = _longest_segment(ids)
+    length = stop - start
+    assert length >= 256
+    pick = np.random.default_rng(config.seed + 1)
+    edge = np.array([0, 1, 31, 32, 63, 64, 127, 128, length - 129, length - 65, length - 33, length - 2,
+                     length - 1])
+    edge = edge[(edge >= 0) & (edge < length)]
+    query_rows = np.unique(np.concatenate((edge, pick.choice(length, 64 - len(edge), replace=False))))
+    key_rows = np.unique(np.concatenate((edge, pick.choice(length, 64 - len(edge), replace=False))))
+    seg_ends = (np.arange(length) if ends is None else ends[b, start:stop] - start)
+    want = ref.segment_sampled_rows(
+        inputs["q"][b, start:stop, heads], inputs["k"][b, start:stop, kvh], inputs["v"][b, start:stop, kvh],
+        inputs["dout"][b, start:stop, heads], seg_ends, scale=config.scale, query_rows=query_rows,
+        key_rows=key_rows)
+    print("longest segment", name, b, start, stop, flush=True)
+    rows, cols = start + query_rows, start + key_rows
+    assert float((out[b, rows][:, heads].float() - want[0]).abs().max()) <= O_ATOL
+    assert float((lse[b, rows][:, heads] - want[1]).abs().max()) <= LSE_ATOL
+    assert ref.relative_l2(dq[b, rows][:, heads], want[2]) <= GRAD_RTOL
+    assert ref.relative_l2(dk[b, cols, kvh], want[3]) <= GRAD_RTOL
+    assert ref.relative_l2(dv[b, cols, kvh], want[4]) <= GRAD_RTOL

@@ -226,8 +226,11 @@ def test_closed_form_uniform_logits(ct, gpu):
     assert float((lse[weights != 0] - np.log(vocab)).abs().max()) < 1e-5
 
 
-def test_benchmark_shape(ct, gpu):
-    """N=16384, d=4096, V=128256, 30% ignored: oracle on samples + size-independent properties."""
+@pytest.mark.parametrize("cache", [False, True], ids=["recompute", "logits_cache"])
+def test_benchmark_shape(ct, gpu, cache):
+    """N=16384, d=4096, V=128256, 30% ignored: oracle on samples + size-independent properties,
+    for the backward that recomputes the logits and for the one that reads the forward's f32
+    logits cache (8.4 GB here, poisoned before the forward: offsets beyond 2^32 bytes)."""
 
     W = ct.workloads
     config = W.CUTCE_CONFIGS["llama3_8b_head"]
@@ -236,7 +239,8 @@ def test_benchmark_shape(ct, gpu):
     active = int((weights != 0).sum())
     dy = 1.0 / active
     print("shape", config, "active", active, flush=True)
-    nll, weight_sum, lse, dhidden, dhead = _gpu(ct, gpu, hidden, head, targets, weights, dy, compaction=True)
+    nll, weight_sum, lse, dhidden, dhead = _gpu(ct, gpu, hidden, head, targets, weights, dy, compaction=True,
+                                                cache=cache)
     assert weight_sum == float(active)
     ignored = weights == 0
     assert (lse[ignored] == 0).all() and (lse[~ignored] != 0).all()

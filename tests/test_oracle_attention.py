@@ -312,3 +312,35 @@ def test_reference_seeded_fixture_regenerates(tmp_path):
         assert (grad[:, seg != 2] == 0).all()
         assert grad[0, 71:128].float().abs().sum() > 0
     assert (dq[:, seg != 2] == 0).all()
+
+
+def test_sampled_rows_of_a_segment_agree_with_the_full_restatement():
+    """segment_sampled_rows (chunked, sampled) against efficient_forward / efficient_backward
+    evaluated on the whole segment, for plain causal and for bidirectional blocks."""
+
+    rng = np.random.default_rng(77)
+    length, groups, dim = 300, 3, 64
+    for hybrid in (False, True):
+        q = _bf16(rng.standard_normal((1, length, groups, dim)))
+        k = _bf16(rng.standard_normal((1, length, 1, dim)))
+        v = _bf16(rng.standard_normal((1, length, 1, dim)))
+        dout = _bf16(rng.standard_normal((1, length, groups, dim)))
+        ends = np.arange(length, dtype=np.int32)
+        if hybrid:
+            ends[40:111] = 110
+            ends[200:290] = 289
+        ids = np.ones((1, length), np.int32)
+        allowed = ref.allowed_from_canonical(ids, ends[None])
+        scale = dim ** -0.5
+        out, lse = ref.efficient_forward(q, k, v, allowed, scale=scale)
+        dq, dk, dv = ref.efficient_backward(q, k, v, allowed, out, lse, dout, scale=scale)
+        query_rows = np.sort(rng.choice(length, 37, replace=False))
+        key_rows = np.sort(rng.choice(length, 29, replace=False))
+        got = ref.segment_sampled_rows(q[0], k[0, :, 0], v[0, :, 0], dout[0], ends, scale=scale,
+                                       query_rows=query_rows, key_rows=key_rows, chunk=64)
+        torch.testing.assert_close(got[1], lse[0, query_rows], atol=2e-5, rtol=0)
+        # the full restatement rounds its results to bf16: half an ulp (2^-9 relative) each
+        assert ref.relative_l2(got[0], out[0, query_rows].float()) < 3e-3
+        assert ref.relative_l2(got[2], dq[0, query_rows].float()) < 3e-3
+        assert ref.relative_l2(got[3], dk[0, key_rows, 0].float()) < 3e-3
+        assert ref.relative_l2(got[4], dv[0, key_rows, 0].float()) < 3e-3
