@@ -140,6 +140,8 @@ SYMBOLS = {
     "ct_cutce_logits_cache_bytes": (c_size_t, [POINTER(CutceShape)]),
     "ct_cutce_fwd": (c_int32, [c_void_p, POINTER(CutceFwdArgs)]),
     "ct_cutce_bwd": (c_int32, [c_void_p, POINTER(CutceBwdArgs)]),
+    "ct_cutce_fwd_noalloc_max_bytes": (c_size_t, []),
+    "ct_cutce_fwd_noalloc": (c_int32, [c_void_p, POINTER(CutceFwdArgs)]),
 }
 
 _library = None

@@ -21,6 +21,8 @@
 // The cache is vocabulary-major [vocab, rows] like G^T: in the transposed tile
 // the GEMMs produce, the lanes of a wavefront run along the rows, so both are
 // written with contiguous stores.
+#include <mutex>
+
 #include "ct_error.h"
 #include "ct_gemm.cuh"
 
@@ -726,26 +728,27 @@ static CutceParams make_params(const uint16_t* hidden, const uint16_t* head, con
   return p;
 }
 
-extern "C" int32_t ct_cutce_fwd(void* stream_, const ct_cutce_fwd_args* a) {
-  CT_REQUIRE(a, "ct_cutce_fwd: null args");
+// Shared body of ct_cutce_fwd and ct_cutce_fwd_noalloc: `ws` / `ws_bytes` is the workspace to use
+// (the caller's, or this device's static scratch array), `fn` the name for error texts.
+static int32_t cutce_fwd_on(void* stream_, const ct_cutce_fwd_args* a, void* ws_, size_t ws_bytes,
+                            const char* fn) {
   CT_REQUIRE(a->hidden && a->head && a->targets && a->weights && a->nll_sum && a->weight_sum &&
-                 a->lse && a->workspace,
-             "ct_cutce_fwd: null pointer");
-  int rc = validate_cutce("ct_cutce_fwd", a->shape);
+                 a->lse && ws_,
+             "%s: null pointer", fn);
+  int rc = validate_cutce(fn, a->shape);
   if (rc) return rc;
   const FwdLayout L = fwd_layout(a->shape);
-  if (a->workspace_bytes < L.total)
-    return fail(CT_WORKSPACE_TOO_SMALL, "ct_cutce_fwd: workspace %zu < %zu bytes",
-                a->workspace_bytes, L.total);
-  CT_REQUIRE(is_aligned16(a->workspace), "ct_cutce_fwd: workspace must be 16-byte aligned");
+  if (ws_bytes < L.total)
+    return fail(CT_WORKSPACE_TOO_SMALL, "%s: workspace %zu < %zu bytes", fn, ws_bytes, L.total);
+  CT_REQUIRE(is_aligned16(ws_), "%s: workspace must be 16-byte aligned", fn);
   if (a->logits_cache) {
-    CT_REQUIRE(is_aligned16(a->logits_cache), "ct_cutce_fwd: logits cache must be 16-byte aligned");
+    CT_REQUIRE(is_aligned16(a->logits_cache), "%s: logits cache must be 16-byte aligned", fn);
     if (a->logits_cache_bytes < ct_cutce_logits_cache_bytes(&a->shape))
-      return fail(CT_WORKSPACE_TOO_SMALL, "ct_cutce_fwd: logits cache %zu < %zu bytes",
+      return fail(CT_WORKSPACE_TOO_SMALL, "%s: logits cache %zu < %zu bytes", fn,
                   a->logits_cache_bytes, ct_cutce_logits_cache_bytes(&a->shape));
   }
   hipStream_t stream = (hipStream_t)stream_;
-  char* ws = static_cast<char*>(a->workspace);
+  char* ws = static_cast<char*>(ws_);
   CutceParams p = make_params(a->hidden, a->head, a->targets, a->weights, a->shape, ws);
   float* part = reinterpret_cast<float*>(ws + L.part);
   double* sums = reinterpret_cast<double*>(ws + L.sums);
@@ -758,8 +761,8 @@ extern "C" int32_t ct_cutce_fwd(void* stream_, const ct_cutce_fwd_args* a) {
   if ((rc = scope1.done())) return rc;
 
   const size_t smem = GemmSmem::kBytes;
-  if ((rc = set_smem(cutce_stats_kernel<false>, smem, "ct_cutce_fwd"))) return rc;
-  if ((rc = set_smem(cutce_stats_kernel<true>, smem, "ct_cutce_fwd"))) return rc;
+  if ((rc = set_smem(cutce_stats_kernel<false>, smem, fn))) return rc;
+  if ((rc = set_smem(cutce_stats_kernel<true>, smem, fn))) return rc;
   const int persistent = min(device_cu_count(), chunks * row_blocks);
   LaunchScope scope2("cutce_stats_kernel", stream);
   if (a->logits_cache)
@@ -778,6 +781,60 @@ extern "C" int32_t ct_cutce_fwd(void* stream_, const ct_cutce_fwd_args* a) {
   hipLaunchKernelGGL(cutce_finalize_kernel, dim3(1), dim3(64), 0, stream, sums, row_blocks,
                      a->nll_sum, a->weight_sum);
   return scope4.done();
+}
+
+extern "C" int32_t ct_cutce_fwd(void* stream, const ct_cutce_fwd_args* a) {
+  CT_REQUIRE(a, "ct_cutce_fwd: null args");
+  return cutce_fwd_on(stream, a, a->workspace, a->workspace_bytes, "ct_cutce_fwd");
+}
+
+// ---------------------------------------------------------------------------
+// The forward for callers that cannot allocate: its workspace (header, active-row
+// index list, per-chunk row statistics, per-block loss sums) lives in a static
+// device array instead of a caller buffer. Every GPU that loads the library holds
+// its own copy of the array at its own address, so the address is looked up once
+// per device, with that device current, and kept.
+// ---------------------------------------------------------------------------
+namespace ct {
+constexpr size_t kNoAllocScratchBytes = (size_t)32 << 20;
+constexpr int kNoAllocMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kNoAllocScratchBytes];
+static void* g_scratch_ptr[kNoAllocMaxDevices];  // device address of `scratch`, per device
+static std::mutex g_scratch_mutex;
+}  // namespace ct
+
+extern "C" size_t ct_cutce_fwd_noalloc_max_bytes(void) { return kNoAllocScratchBytes; }
+
+extern "C" int32_t ct_cutce_fwd_noalloc(void* stream, const ct_cutce_fwd_args* a) {
+  CT_REQUIRE(a, "ct_cutce_fwd_noalloc: null args");
+  int rc = validate_cutce("ct_cutce_fwd_noalloc", a->shape);
+  if (rc) return rc;
+  const size_t need = fwd_layout(a->shape).total;
+  if (need > kNoAllocScratchBytes)
+    return fail(CT_UNSUPPORTED,
+                "ct_cutce_fwd_noalloc: rows=%d, vocab=%d need %zu bytes of scratch, the static "
+                "array holds %zu; use ct_cutce_fwd with a caller workspace",
+                a->shape.rows, a->shape.vocab, need, kNoAllocScratchBytes);
+  int device = 0;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess)
+    return fail(CT_LAUNCH_FAILED, "ct_cutce_fwd_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  CT_REQUIRE(device >= 0 && device < kNoAllocMaxDevices, "ct_cutce_fwd_noalloc: device %d out of range",
+             device);
+  void* ws = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+      void* ptr = nullptr;
+      e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || !ptr)
+        return fail(CT_LAUNCH_FAILED, "ct_cutce_fwd_noalloc: hipGetSymbolAddress: %s",
+                    hipGetErrorString(e));
+      g_scratch_ptr[device] = ptr;
+    }
+    ws = g_scratch_ptr[device];
+  }
+  return cutce_fwd_on(stream, a, ws, kNoAllocScratchBytes, "ct_cutce_fwd_noalloc");
 }
 
 extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {

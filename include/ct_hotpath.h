@@ -384,6 +384,23 @@ typedef struct ct_cutce_fwd_args {
  */
 int32_t ct_cutce_fwd(void* stream, const ct_cutce_fwd_args* args);
 
+/*
+ * ct_cutce_fwd for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight evaluation or serving loops, harnesses that forbid
+ * hipMalloc). No counterpart in the reference. Same arguments, results and
+ * kernels as ct_cutce_fwd, but args->workspace / workspace_bytes are ignored:
+ * the workspace is a static device array inside the library,
+ * ct_cutce_fwd_noalloc_max_bytes() (32 MiB) per GPU, held until the process
+ * ends. Shapes whose ct_cutce_fwd_workspace_bytes() exceeds that are rejected
+ * with CT_UNSUPPORTED before any launch (N = 16384, V = 128256 needs 25 MB and
+ * fits). The call makes no hipMalloc / hipFree and no allocating library call.
+ * All calls on one GPU share the array: calls that overlap on one GPU (two
+ * streams, two threads) race; serialise them. Each call initialises what it
+ * reads, so nothing carries over from the previous call.
+ */
+size_t ct_cutce_fwd_noalloc_max_bytes(void);
+int32_t ct_cutce_fwd_noalloc(void* stream, const ct_cutce_fwd_args* args);
+
 typedef struct ct_cutce_bwd_args {
   const uint16_t* hidden;
   const uint16_t* head;
