@@ -135,7 +135,7 @@ CT_DEVICE void dma16_s(const void* uniform_base, unsigned lane_offset, lds_addr 
   const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
   const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
   const unsigned long long base = ((unsigned long long)hi << 32) | (unsigned long long)lo;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %0, %1"
                :
                : "v"(lane_offset), "s"(base), "s"(m0_value)
                : "memory", "m0");
@@ -358,7 +358,10 @@ CT_DEVICE u32x4 load_global16(const void* p) { return *reinterpret_cast<const u3
 CT_DEVICE void store_global16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 
 // 4-byte store to uniform_base + lane_offset + IMM bytes (scalar base, 32-bit lane offset): no
-// per-store vector address arithmetic.
+// per-store vector address arithmetic. The scalar base may have just been written by a vector
+// instruction (v_readfirstlane): a memory instruction that reads such a register needs 5 wait
+// states after the write, and the compiler does not add them in front of an asm statement, so
+// each of these stores carries them itself (s_nop 4).
 template <int IMM>
 CT_DEVICE void store_global4_s(void* uniform_base, unsigned lane_offset, float value) {
   static_assert(IMM >= 0 && IMM < 4096, "immediate offset out of range");
@@ -366,7 +369,29 @@ CT_DEVICE void store_global4_s(void* uniform_base, unsigned lane_offset, float v
   const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
   const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
   const unsigned long long base = ((unsigned long long)hi << 32) | (unsigned long long)lo;
-  asm volatile("global_store_dword %0, %1, %2 offset:%3" : : "v"(lane_offset), "v"(value), "s"(base), "n"(IMM) : "memory");
+  asm volatile("s_nop 4\n\tglobal_store_dword %0, %1, %2 offset:%3" : : "v"(lane_offset), "v"(value), "s"(base), "n"(IMM) : "memory");
+}
+
+// 16- and 8-byte stores of the same form.
+template <int IMM>
+CT_DEVICE void store_global16_s(void* uniform_base, unsigned lane_offset, f32x4 value) {
+  static_assert(IMM >= 0 && IMM < 4096, "immediate offset out of range");
+  const unsigned long long b = (unsigned long long)(uintptr_t)uniform_base;
+  const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
+  const unsigned long long base = ((unsigned long long)hi << 32) | (unsigned long long)lo;
+  asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 offset:%3" : : "v"(lane_offset), "v"(value), "s"(base), "n"(IMM) : "memory");
+}
+template <int IMM>
+CT_DEVICE void store_global8_s(void* uniform_base, unsigned lane_offset, bf16x4 value) {
+  static_assert(IMM >= 0 && IMM < 4096, "immediate offset out of range");
+  const unsigned long long b = (unsigned long long)(uintptr_t)uniform_base;
+  const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
+  const unsigned long long base = ((unsigned long long)hi << 32) | (unsigned long long)lo;
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  const u32x2 bits = __builtin_bit_cast(u32x2, value);
+  asm volatile("s_nop 4\n\tglobal_store_dwordx2 %0, %1, %2 offset:%3" : : "v"(lane_offset), "v"(bits), "s"(base), "n"(IMM) : "memory");
 }
 
 CT_DEVICE bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }

@@ -30,18 +30,28 @@ namespace ct {
 
 constexpr int kBK = kGemmBK;
 constexpr int kTilesPerChunk = 4;  // vocab tiles per stats work unit
+#ifndef CT_CUTCE_SWEEP
+#define CT_CUTCE_SWEEP 1
+#endif
+constexpr bool kSweepUnits = CT_CUTCE_SWEEP != 0;  // unit order of the two projection kernels
 constexpr float kNegInfF = -__builtin_inff();
 
 struct CutceHeader {
   int n_act;
   int counter;
-  // per-XCD work counters: set 0 statistics kernel / hidden gradient, set 1 head gradient
-  int xcd_counter[2][8];
-  int pad[14];
+  // per-XCD work counters: set 0 statistics kernel / hidden gradient, set 1 head gradient,
+  // set 2 the dlogits kernel that recomputes the projection
+  int xcd_counter[3][8];
+  int pad[6];
 };
 
+// Clears counter sets 0 and 1 (called by workgroup 0 of a kernel that runs before their users).
 CT_DEVICE void reset_unit_counters(CutceHeader* header) {
   if (threadIdx.x < 16) (&header->xcd_counter[0][0])[threadIdx.x] = 0;
+}
+// Clears counter set 2.
+CT_DEVICE void reset_dlogits_counters(CutceHeader* header) {
+  if (threadIdx.x < 8) header->xcd_counter[2][threadIdx.x] = 0;
 }
 
 // Work order of the persistent GEMM kernels. A unit is a pair (a, b) of operand tile indices,
@@ -52,12 +62,21 @@ CT_DEVICE void reset_unit_counters(CutceHeader* header) {
 // operand tiles feed 32 GEMM tiles), the sequence of blocks is cut into 8 equal ranges, and an
 // XCD takes the units of its range through its own counter. Indices that fall outside the
 // grid (ragged edges) are skipped. An XCD that runs dry helps the next one.
+//
+// Sweep mode (the two projection kernels, a = vocabulary chunk, b = row block): XCD x owns the
+// row blocks x, x + 8, ... and walks (a, its row blocks) with a as the slow index, so all eight
+// XCDs are on the same few vocabulary chunks at the same time. The head is the large operand
+// (1 GB against 0.1 GB of hidden rows): with every XCD on the same chunk it leaves HBM about once
+// per pass, and the other XCDs find it in the memory-side cache; in block mode each XCD streams
+// its own range of the vocabulary and the head is read from HBM once per 8 row blocks.
 struct XcdUnits {
   static constexpr int kA = 4, kB = 8, kXcds = 8;
   int* counters;
   int a_count, b_count, b_groups, padded_total, per_xcd, my_xcd;
   int helping;  // how many XCDs further the counter in use belongs to
-  CT_DEVICE void init(int* counters_, int a_count_, int b_count_) {
+  bool sweep;
+  CT_DEVICE void init(int* counters_, int a_count_, int b_count_, bool sweep_ = false) {
+    sweep = sweep_;
     counters = counters_;
     a_count = a_count_;
     b_count = b_count_;
@@ -70,14 +89,32 @@ struct XcdUnits {
     helping = 0;
   }
   // Called by all threads of the workgroup (contains barriers); false when nothing is left.
+  CT_DEVICE bool next_sweep(int& a, int& b, int* lds_slot) {
+    while (helping < kXcds) {
+      const int x = (my_xcd + helping) % kXcds;
+      const int mine = x < b_count ? (b_count - x + kXcds - 1) / kXcds : 0;  // row blocks of XCD x
+      if (threadIdx.x == 0) *lds_slot = mine ? atomicAdd(&counters[x], 1) : 0;
+      __syncthreads();
+      const int local = uniform(*lds_slot);  // scalar from here on: unit indices feed scalar address arithmetic
+      __syncthreads();
+      if (mine && local < a_count * mine) {
+        a = local / mine;
+        b = x + kXcds * (local % mine);
+        return true;
+      }
+      ++helping;
+    }
+    return false;
+  }
   CT_DEVICE bool next(int& a, int& b, int* lds_slot) {
+    if (sweep) return next_sweep(a, b, lds_slot);
     for (;;) {
       int index = -1;
       while (helping < kXcds) {
         const int x = (my_xcd + helping) % kXcds;
         if (threadIdx.x == 0) *lds_slot = atomicAdd(&counters[x], 1);
         __syncthreads();
-        const int local = *lds_slot;
+        const int local = uniform(*lds_slot);  // scalar from here on: unit indices feed scalar address arithmetic
         __syncthreads();
         if (local < per_xcd && x * per_xcd + local < padded_total) {
           index = x * per_xcd + local;
@@ -120,6 +157,7 @@ __global__ __launch_bounds__(1024) void cutce_index_kernel(const float* weights,
       header->counter = 0;
     }
     reset_unit_counters(header);
+    reset_dlogits_counters(header);
     return;
   }
   int carry = 0;
@@ -147,6 +185,7 @@ __global__ __launch_bounds__(1024) void cutce_index_kernel(const float* weights,
     header->counter = 0;
   }
   reset_unit_counters(header);
+  reset_dlogits_counters(header);
 }
 
 // ---------------------------------------------------------------------------
@@ -173,7 +212,7 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
   // units: (vocabulary chunk, row block)
   const int active_blocks = (n_act + kGemmTile - 1) / kGemmTile;
   XcdUnits units;
-  units.init(p.header->xcd_counter[0], chunks, active_blocks);
+  units.init(p.header->xcd_counter[0], chunks, active_blocks, kSweepUnits);
   int chunk, rb;
   while (units.next(chunk, rb, &unit_s)) {
     const int n0 = rb * kGemmTile;
@@ -181,10 +220,12 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
     const int active = my_slot < n_act && p.weights[p.idx[my_slot]] != 0.f;
     if (!__syncthreads_or(active)) continue;  // no row of this block carries weight
 
+    // Rows are interleaved in the tile (KcLoader): column block nb of lane j is row slot
+    // n0 + wn + 4 j + nb, so a lane owns 4 consecutive slots.
     int tgt[4];
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) {
-      const int slot = n0 + wn + 32 * nb + j;
+      const int slot = n0 + wn + 4 * j + nb;
       tgt[nb] = slot < n_act ? p.targets[p.idx[slot]] : -1;
     }
     float m2[4], sum[4], tl[4];
@@ -195,7 +236,7 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
       tl[nb] = 0.f;
     }
     KcLoader B;
-    B.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true);
+    B.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true, true);
 
     const int vt_end = min((chunk + 1) * kTilesPerChunk, vocab_tiles);
     for (int vt = chunk * kTilesPerChunk; vt < vt_end; ++vt) {
@@ -209,20 +250,18 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
       const int vbase = v0 + wm + 4 * half;  // vocab id of (i, r) = vbase + 32 i + 8 (r/4) + r%4
       const bool ragged = v0 + kGemmTile > p.V;
       if constexpr (CACHE) {
-        // cache^T[v][slot]: 32 lanes = 32 consecutive slots, 128 contiguous bytes per store.
-        // Address = wave-uniform tile origin + uniform (row, column block) offset + a 32-bit
-        // lane offset, so the stores need no per-store vector address arithmetic.
+        // cache^T[v][slot]: a lane stores its 4 consecutive slots with one 16-byte access, 32
+        // lanes = 512 contiguous bytes. Address = wave-uniform tile origin + uniform row offset +
+        // a 32-bit lane offset, so the stores need no per-store vector address arithmetic.
         float* origin = cache + (size_t)(v0 + uniform(wm)) * p.n_pad + n0 + uniform(wn);
-        const unsigned lane_off = (unsigned)(4 * half * p.n_pad + j) * 4u;  // bytes
+        const unsigned lane_off = (unsigned)(4 * half * p.n_pad + 4 * j) * 4u;  // bytes
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             float* row = origin + (size_t)(32 * i + 8 * (r >> 2) + (r & 3)) * p.n_pad;
-            store_global4_s<0>(row, lane_off, acc.c[i][0][r]);
-            store_global4_s<128>(row, lane_off, acc.c[i][1][r]);
-            store_global4_s<256>(row, lane_off, acc.c[i][2][r]);
-            store_global4_s<384>(row, lane_off, acc.c[i][3][r]);
+            const f32x4 quad = {acc.c[i][0][r], acc.c[i][1][r], acc.c[i][2][r], acc.c[i][3][r]};
+            store_global16_s<0>(row, lane_off, quad);
           }
       }
 #pragma unroll
@@ -278,7 +317,7 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
         const float* e = exch + ((w & 1) * 128 + 32 * nb + j) * 3;
         merge_stats(m2[nb], sum[nb], e[0], e[1]);
         tl[nb] += e[2];
-        float* out = part + ((size_t)chunk * p.n_pad + n0 + wn + 32 * nb + j) * 3;
+        float* out = part + ((size_t)chunk * p.n_pad + n0 + wn + 4 * j + nb) * 3;
         out[0] = m2[nb];
         out[1] = sum[nb];
         out[2] = tl[nb];
@@ -407,55 +446,60 @@ CT_DEVICE float dlogit(float logit, float fac, float lse2, int tgt, int v) {
   return fac * (exp2_fast(logit * kLog2e - lse2) - (v == tgt ? 1.f : 0.f));
 }
 
-// G^T[v - slab0][slot] for one 256 x 256 tile, logits recomputed (transposed tile as in the
-// statistics kernel: rows = vocabulary, lanes = row slots).
+// G^T[v - slab0][slot], logits recomputed (transposed tile as in the statistics kernel: rows =
+// vocabulary, lanes = row slots). Persistent like the statistics kernel and with its unit order:
+// a unit is kTilesPerChunk vocabulary tiles of the slab times one block of 256 active rows.
 __global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, CutceRowParams rp,
                                                             int slab0, int slab_tiles, bf16* G) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr smem = lds_address_of(smem_raw);
+  __shared__ int unit_s;
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
-  const int row_blocks = p.n_pad / kGemmTile;
-  int id = xcd_remap(blockIdx.x, slab_tiles * row_blocks);
-  const int rb = id % row_blocks, vt = id / row_blocks;
-  const int n0 = rb * kGemmTile;
   const int n_act = p.header->n_act;
   // the two GEMM kernels that follow start from fresh work counters
   if (blockIdx.x == 0) reset_unit_counters(p.header);
-  if (n0 >= n_act) return;  // G^T columns past the active count's block are never read
-  const int v0 = slab0 + vt * kGemmTile;
+  const int active_blocks = (n_act + kGemmTile - 1) / kGemmTile;  // G^T columns past them are never read
+  const int chunks = (slab_tiles + kTilesPerChunk - 1) / kTilesPerChunk;
+  XcdUnits units;
+  units.init(p.header->xcd_counter[2], chunks, active_blocks, kSweepUnits);
+  int chunk, rb;
+  while (units.next(chunk, rb, &unit_s)) {
+    const int n0 = rb * kGemmTile;
+    // Rows are interleaved in the tile (KcLoader): column block nb of lane j is row slot
+    // n0 + wn + 4 j + nb, so a lane owns 4 consecutive slots of G^T and stores them together.
+    const int slot4 = n0 + wn + 4 * j;
+    const f32x4 fac = *reinterpret_cast<const f32x4*>(rp.fac + slot4);
+    const f32x4 lse2 = *reinterpret_cast<const f32x4*>(rp.lse2 + slot4);
+    const i32x4 tgt = *reinterpret_cast<const i32x4*>(rp.tgt + slot4);
+    KcLoader B;
+    B.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true, true);
+    const int vt_end = min((chunk + 1) * kTilesPerChunk, slab_tiles);
+    for (int vt = chunk * kTilesPerChunk; vt < vt_end; ++vt) {
+      const int v0 = slab0 + vt * kGemmTile;
+      McLoader A;
+      A.init(p.head, p.V, nullptr, v0, p.V, p.d, p.head_aligned);
+      GemmAcc acc;
+      acc.clear();
+      gemm_tile(A, B, 0, p.d, smem, acc);
 
-  McLoader A;
-  A.init(p.head, p.V, nullptr, v0, p.V, p.d, p.head_aligned);
-  KcLoader B;
-  B.init(p.hidden, p.d, p.idx, n0, n_act, p.d, p.hidden_aligned, true);
-  GemmAcc acc;
-  acc.clear();
-  gemm_tile(A, B, 0, p.d, smem, acc);
-
-  float fac[4], lse2[4];
-  int tgt[4];
+      bf16* origin = G + (size_t)(v0 - slab0 + uniform(wm)) * p.n_pad + n0 + uniform(wn);
+      const unsigned lane_off = (unsigned)(4 * half * p.n_pad + 4 * j) * 2u;  // bytes
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
-    const int slot = n0 + wn + 32 * nb + j;
-    fac[nb] = rp.fac[slot];
-    lse2[nb] = rp.lse2[slot];
-    tgt[nb] = rp.tgt[slot];
-  }
-  bf16* gbase = G + (size_t)(v0 - slab0 + wm + 4 * half) * p.n_pad + n0 + wn + j;
+      for (int i = 0; i < 4; ++i)
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+        for (int r = 0; r < 16; ++r) {
+          const int vrel = 32 * i + 8 * (r >> 2) + (r & 3);
+          const int v = v0 + wm + 4 * half + vrel;
+          bf16x4 quad;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int vrel = 32 * i + 8 * (r >> 2) + (r & 3);
-      const int v = v0 + wm + 4 * half + vrel;
-      bf16* dst = gbase + (size_t)vrel * p.n_pad;
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb) {
-        const float g = (fac[nb] != 0.f && v < p.V) ? dlogit(acc.c[i][nb][r], fac[nb], lse2[nb], tgt[nb], v) : 0.f;
-        dst[32 * nb] = (bf16)g;
-      }
+          for (int nb = 0; nb < 4; ++nb)
+            quad[nb] = (bf16)((fac[nb] != 0.f && v < p.V)
+                                  ? dlogit(acc.c[i][nb][r], fac[nb], lse2[nb], tgt[nb], v) : 0.f);
+          store_global8_s<0>(origin + (size_t)vrel * p.n_pad, lane_off, quad);
+        }
     }
+  }
 }
 
 // Same G^T from the f32 logits the forward left in its cache: one pass over memory. A thread
@@ -513,6 +557,8 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
   const int col_blocks = (p.d + kGemmTile - 1) / kGemmTile;
   const int n_act = p.header->n_act;
   __shared__ int unit_s;
+  // the dlogits kernel of the next vocabulary slab starts from fresh work counters
+  if (blockIdx.x == 0) reset_dlogits_counters(p.header);
   // units: (row block, column block) over the started row blocks
   XcdUnits units;
   units.init(p.header->xcd_counter[0], (n_act + kGemmTile - 1) / kGemmTile, col_blocks);
@@ -521,29 +567,31 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
     const int n0 = rb * kGemmTile, c0 = cb * kGemmTile;
     McLoader A;
     A.init(G, p.n_pad, nullptr, n0, p.n_pad, slab_width, true);
+    // (rows of B interleaved: lane j owns the 4 consecutive columns c0 + wn + 4 j + nb)
     KcLoader B;
     B.init(p.head + slab0, p.V, nullptr, c0, p.d, min(slab_width, p.V - slab0), p.head_aligned,
-           false);
+           false, true);
     GemmAcc acc;
     acc.clear();
     gemm_tile(A, B, 0, slab_width, smem, acc);
 
+    const int col = c0 + wn + 4 * j;  // hidden sizes are multiples of 128: col < d implies col + 3 < d
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int slot = n0 + wm + 32 * i + acc_row(r, half);
-        if (slot >= n_act) continue;
+        if (slot >= n_act || col >= p.d) continue;
         const long row = p.idx[slot];
+        f32x4 val = {acc.c[i][0][r], acc.c[i][1][r], acc.c[i][2][r], acc.c[i][3][r]};
+        f32x4* a = reinterpret_cast<f32x4*>(dh_acc + (size_t)slot * p.d + col);
+        if (mode >= 2) val += *a;
+        if (mode == 1 || mode == 2) *a = val;
+        if (mode == 0 || mode == 3) {
+          bf16x4 out;
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-          const int col = c0 + wn + 32 * nb + j;
-          if (col >= p.d) continue;
-          float val = acc.c[i][nb][r];
-          float* a = dh_acc + (size_t)slot * p.d + col;
-          if (mode >= 2) val += *a;
-          if (mode == 1 || mode == 2) *a = val;
-          if (mode == 0 || mode == 3) dhidden[row * p.d + col] = (bf16)val;
+          for (int nb = 0; nb < 4; ++nb) out[nb] = (bf16)val[nb];
+          *reinterpret_cast<bf16x4*>(dhidden + row * p.d + col) = out;
         }
       }
   }
@@ -571,22 +619,31 @@ __global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const b
     const int m0 = mb * kGemmTile, v0 = vt * kGemmTile;  // v0 relative to the slab
     McLoader A;
     A.init(packed, p.d, nullptr, m0, p.d, k_end, true);
+    // (rows of B interleaved: lane j owns the 4 consecutive vocabulary ids v .. v + 3)
     KcLoader B;
-    B.init(G, p.n_pad, nullptr, v0, slab_tiles * kGemmTile, k_end, true, false);
+    B.init(G, p.n_pad, nullptr, v0, slab_tiles * kGemmTile, k_end, true, false, true);
     GemmAcc acc;
     acc.clear();
     gemm_tile(A, B, 0, k_end, smem, acc);
 
+    const int v = slab0 + v0 + wn + 4 * j;
+    const bool vector_store = (p.V % 4 == 0) && ((reinterpret_cast<uintptr_t>(dhead) & 7u) == 0);
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm + 32 * i + acc_row(r, half);
         if (m >= p.d) continue;
+        bf16* dst = dhead + (size_t)m * p.V + v;
+        if (vector_store && v + 3 < p.V) {
+          bf16x4 out;
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-          const int v = slab0 + v0 + wn + 32 * nb + j;
-          if (v < p.V) dhead[(size_t)m * p.V + v] = (bf16)acc.c[i][nb][r];
+          for (int nb = 0; nb < 4; ++nb) out[nb] = (bf16)acc.c[i][nb][r];
+          *reinterpret_cast<bf16x4*>(dst) = out;
+        } else {
+#pragma unroll
+          for (int nb = 0; nb < 4; ++nb)
+            if (v + nb < p.V) dst[nb] = (bf16)acc.c[i][nb][r];
         }
       }
   }
@@ -909,7 +966,8 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
       if ((rc = scope11.done())) return rc;
     } else {
       LaunchScope scope7("cutce_dlogits_kernel", stream);
-      hipLaunchKernelGGL(cutce_dlogits_kernel, dim3(slab_tiles * row_blocks), dim3(256), smem, stream,
+      const int dl_units = ((slab_tiles + kTilesPerChunk - 1) / kTilesPerChunk) * row_blocks;
+      hipLaunchKernelGGL(cutce_dlogits_kernel, dim3(min(cus, dl_units)), dim3(256), smem, stream,
                          p, rp, slab0, slab_tiles, G);
       if ((rc = scope7.done())) return rc;
     }

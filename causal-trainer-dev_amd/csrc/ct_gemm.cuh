@@ -67,8 +67,12 @@ struct KcLoader {
   // gathered through row_index. Rows >= rows_valid read as zero, or, with
   // alias_invalid_rows, as a copy of the first row (for callers that discard
   // those rows); k >= k_valid reads as zero.
+  // With interleave_rows, tile row 128 w + 32 nb + j holds matrix row m0 + 128 w + 4 j + nb:
+  // in the accumulator layout lane j of a wavefront then owns 4 consecutive matrix rows (its
+  // column blocks nb = 0..3), which an epilogue can store with one 8- or 16-byte access.
   CT_DEVICE void init(const bf16* base_, long ld, const int* row_index, int m0, int rows_valid,
-                      int k_valid_, bool aligned, bool alias_invalid_rows) {
+                      int k_valid_, bool aligned, bool alias_invalid_rows,
+                      bool interleave_rows = false) {
     const int t = threadIdx.x;
     k_valid = k_valid_;
     const bool gathered = row_index != nullptr;
@@ -78,7 +82,9 @@ struct KcLoader {
     chunk = (t % CPR) ^ swizzle<CPR>(r0);  // rows r0 + 64 n share the swizzle
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
-      const int r = r0 + 64 * n;
+      const int tile_row = r0 + 64 * n;
+      const int r = interleave_rows ? ((tile_row & 128) | ((tile_row & 31) << 2) | ((tile_row >> 5) & 3))
+                                    : tile_row;
       const bool ok = m0 + r < rows_valid;
       if (ok || alias_invalid_rows) row_mask |= 1 << n;
       const long src = gathered ? row_index[ok ? m0 + r : 0] : (ok ? r : 0);

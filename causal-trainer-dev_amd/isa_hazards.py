@@ -1,0 +1,109 @@
+"""Static check of the compiled kernels for one hazard the compiler does not cover.
+
+On gfx9-family hardware a memory instruction that reads a scalar register needs 5 wait states
+after a vector instruction wrote that register (v_readfirstlane, v_readlane, carries, compares).
+hipcc inserts those wait states in its own code but not in front of an ``asm`` statement, so a
+scalar base that the compiler materialises with v_readfirstlane directly before an inline-asm
+load, store or global->LDS copy is read stale: the access goes to whatever address the register
+pair held before. ``scan`` walks device assembly (``hipcc -S --cuda-device-only``) and reports
+every memory instruction whose scalar operands were written by a vector instruction fewer than
+5 wait states earlier. ``python -m causal_trainer_dev_amd.isa_hazards`` compiles every source of
+the library and scans it; tests/test_isa_hazards.py runs the same on the CPU.
+"""
+
+from __future__ import annotations
+
+import re
+import subprocess
+import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+WAIT_STATES = 5
+_MEMORY = re.compile(r"^\s*(global_|buffer_|flat_|scratch_)")
+_VECTOR_WRITES_SCALAR = re.compile(
+    r"^\s*(v_readfirstlane_b32|v_readlane_b32|v_cmp\w*|v_add_co\w*|v_sub_co\w*|v_subrev_co\w*|v_addc\w*|"
+    r"v_subb\w*|v_div_scale\w*|v_mad_u64_u32|v_mad_i64_i32)\s+(.*)")
+_LABEL = re.compile(r"^([A-Za-z_.$][\w.$]*):")
+
+
+def _scalar_registers(text: str) -> set:
+    found = set()
+    for match in re.finditer(r"s\[(\d+):(\d+)\]", text):
+        found.update(range(int(match.group(1)), int(match.group(2)) + 1))
+    for match in re.finditer(r"(?<![\w\[])s(\d+)\b", text):
+        found.add(int(match.group(1)))
+    if "vcc" in text:
+        found.add("vcc")
+    return found
+
+
+def _wait_states(line: str) -> int:
+    match = re.match(r"\s*s_nop\s+(\d+)", line)
+    return int(match.group(1)) + 1 if match else 1
+
+
+def scan(assembly: str) -> list[str]:
+    """One message per memory instruction that reads a freshly vector-written scalar register."""
+
+    problems, window, kernel = [], [], "?"
+    for number, line in enumerate(assembly.splitlines(), start=1):
+        text = line.strip()
+        label = _LABEL.match(text)
+        if label:
+            if not text.startswith(".L"):
+                kernel, window = label.group(1), []
+            continue
+        if not text or text.startswith((";", ".")):
+            continue
+        if _MEMORY.match(line):
+            operands = text.split(None, 1)[1] if " " in text else ""
+            used = _scalar_registers(operands)
+            elapsed = 0
+            for earlier_number, earlier in reversed(window):
+                write = _VECTOR_WRITES_SCALAR.match(earlier)
+                if write and _scalar_registers(write.group(2).split(",")[0]) & used:
+                    problems.append(f"{kernel}: line {number} '{text}' reads a scalar register that line "
+                                    f"{earlier_number} '{earlier.strip()}' wrote {elapsed} wait states earlier")
+                    break
+                elapsed += _wait_states(earlier)
+                if elapsed >= WAIT_STATES:
+                    break
+        window.append((number, line))
+        if len(window) > 16:
+            del window[0]
+    return problems
+
+
+def device_assembly(source: Path, flags) -> str:
+    from . import build as recipe
+
+    with tempfile.TemporaryDirectory() as scratch:
+        target = Path(scratch) / (source.stem + ".s")
+        command = [recipe.hipcc(), *[f for f in flags if f != "-fPIC"], "--cuda-device-only", "-S", str(source),
+                   "-o", str(target)]
+        done = subprocess.run(command, capture_output=True, text=True)
+        if done.returncode != 0:
+            raise RuntimeError(done.stderr)
+        return target.read_text()
+
+
+def scan_library() -> dict[str, list[str]]:
+    """Compiles every source of the library to device assembly and scans it."""
+
+    from . import build as recipe
+
+    sources = [recipe.CSRC / name for name in recipe.SOURCES]
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        texts = list(pool.map(lambda path: device_assembly(path, recipe.HIP_FLAGS), sources))
+    return {path.name: scan(text) for path, text in zip(sources, texts)}
+
+
+if __name__ == "__main__":
+    findings = scan_library()
+    for name, problems in findings.items():
+        print(f"{name}: {len(problems)} hazard(s)")
+        for problem in problems:
+            print("  " + problem)
+    sys.exit(1 if any(findings.values()) else 0)

@@ -1,0 +1,48 @@
+"""The compiled kernels must not read a scalar register in a memory instruction fewer than
+5 wait states after a vector instruction wrote it (the compiler does not pad inline asm)."""
+
+import shutil
+
+import pytest
+
+
+def test_scanner_flags_the_pattern_and_accepts_padding(ct):
+    from causal_trainer_dev_amd import isa_hazards
+
+    bad = """
+kernel_a:
+	v_readfirstlane_b32 s9, v5
+	v_readfirstlane_b32 s8, v4
+	global_store_dwordx2 v120, v[18:19], s[8:9] offset:0
+"""
+    assert len(isa_hazards.scan(bad)) == 1
+    padded = bad.replace("\tglobal_store", "\ts_nop 4\n\tglobal_store")
+    assert isa_hazards.scan(padded) == []
+    scalar_alu = """
+kernel_b:
+	v_readfirstlane_b32 s0, v1
+	s_ashr_i32 s1, s0, 31
+	s_lshl_b64 s[0:1], s[0:1], 2
+	s_add_u32 s0, s2, s0
+	s_addc_u32 s1, s3, s1
+	s_nop 0
+	global_store_dwordx4 v252, v[2:5], s[0:1] offset:0
+"""
+    assert isa_hazards.scan(scalar_alu) == []
+    two_short = """
+kernel_c:
+	v_readfirstlane_b32 s16, v4
+	s_mov_b32 m0, s8
+	s_nop 0
+	global_load_lds_dwordx4 v52, s[16:17]
+"""
+    assert len(isa_hazards.scan(two_short)) == 1
+    assert isa_hazards.scan("kernel_d:\n\tv_readfirstlane_b32 s16, v4\n\tglobal_load_dword v1, v[2:3], off\n") == []
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_library_sources_have_no_scalar_base_hazard(ct):
+    from causal_trainer_dev_amd import isa_hazards
+
+    findings = isa_hazards.scan_library()
+    assert findings and all(not problems for problems in findings.values()), findings
