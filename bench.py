@@ -133,7 +133,7 @@ def kernel_table(config, pairs, kernels):
     return table
 
 
-def bench_delta_pass(ct, torch, config, q_like, launches=400, pairs_of_buffers=4):
+def bench_delta_pass(ct, torch, config, q_like, launches=400, pairs_of_buffers=8):
     """The delta pass (rowsum(O * dO), HBM bound) on its own, through ct_attn_delta. It rotates over
     `pairs_of_buffers` (O, dO) pairs, 268 MB each at the Llama-3-8B shape, so that no launch can
     find its operands in the 256 MB last-level cache, and has its own launch count, independent of
@@ -154,13 +154,25 @@ def bench_delta_pass(ct, torch, config, q_like, launches=400, pairs_of_buffers=4
         ct._lib.check(lib.ct_attn_delta(ct._lib.current_stream(), out.data_ptr(), dout.data_ptr(),
                                         delta.data_ptr(), rows, config.head_dim))
 
-    _, kernels = timed_region(torch, delta_pass, launches, 40, ct.profiling.KernelTimer)
-    avg_ms = mean(kernels["attn_delta_kernel"])
+    # One pair of events around all launches (recorded on the stream the launches go to): with
+    # an event pair per launch, taken from a Python callback, the GPU drains its queue between
+    # two launches of a 40 us kernel and the bracket mostly measures the host.
+    for _ in range(40):
+        delta_pass()
+    torch.cuda.synchronize()
+    begin, finish = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    begin.record()
+    for _ in range(launches):
+        delta_pass()
+    finish.record()
+    torch.cuda.synchronize()
+    avg_ms = begin.elapsed_time(finish) / launches
     gbps = W.attention_delta_bytes(config) / (avg_ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": gbps, "peak": PEAK_HBM_GBPS, "unit": "GB/s", "frac": gbps / PEAK_HBM_GBPS,
             "avg_launch_ms": avg_ms, "launches": launches,
             "note": (f"pass on its own (ct_attn_delta), not a launch of the timed step: the backward forms delta "
-                     f"inside its dQ kernel; rotates over {pairs_of_buffers} (O, dO) pairs of "
+                     f"inside its dQ kernel; {launches} back-to-back launches between one pair of stream events, "
+                     f"rotating over {pairs_of_buffers} (O, dO) pairs of "
                      f"{W.attention_delta_bytes(config) / 1e6:.0f} MB so operands come from HBM")}
 
 

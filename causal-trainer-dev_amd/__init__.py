@@ -30,4 +30,4 @@ from .layer_ops import (  # noqa: F401,E402
 )
 from . import maskgit, packing  # noqa: F401,E402
 from .maskgit import MaskGITBatchTransform  # noqa: F401,E402
-from .packing import best_fit_decreasing, collate, pack_dataset, pack_examples, pad_example, pad_examples  # noqa: F401,E402
+from .packing import best_fit_decreasing, collate, pack_examples, pad_example, pad_examples  # noqa: F401,E402

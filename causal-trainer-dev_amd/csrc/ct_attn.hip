@@ -14,9 +14,13 @@ namespace ct {
 // 32-position block, phase 2 turns the summaries into visit ranges.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, const int* end, int S,
-                                                            int* meta, int* sched_all) {
-  extern __shared__ int lds_meta[];  // [nrb][3]: min_nz, max_id, end_max; later schedule_ints(nrb) work counts
+                                                            int* meta, int* sched_all,
+                                                            int* global_scratch) {
+  // [nrb][3]: min_nz, max_id, end_max; later schedule_ints(nrb) work counts. In LDS when the
+  // row fits, else this batch row's part of the scratch region (3 * nrb ints per row).
+  extern __shared__ int lds_meta_shared[];
   const int b = blockIdx.x;
+  int* lds_meta = global_scratch ? global_scratch + (size_t)b * 3 * (S / 32) : lds_meta_shared;
   const int nrb = S / 32, nt = S / kKeyTile;
   const int* segb = seg + (size_t)b * S;
   const int* endb = end ? end + (size_t)b * S : nullptr;
@@ -53,6 +57,7 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, cons
     lds_meta[rb * 3 + 1] = max_id;
     lds_meta[rb * 3 + 2] = end_max;
   }
+  __threadfence();
   __syncthreads();
 
   for (int rb = threadIdx.x; rb < nrb; rb += blockDim.x) {
@@ -89,7 +94,7 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, cons
     m[kQFirst] = q_first;
     m[kQLast] = q_last;
   }
-  __threadfence_block();
+  __threadfence();  // the table and (for long rows) the scratch arrays are re-read through global memory
   __syncthreads();
 
   // Phase 3: amount of work per tile, for the four schedules, into LDS (the
@@ -132,6 +137,7 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, cons
     }
     work[off8 + i] = last >= first ? last - first + 1 : 0;
   }
+  __threadfence();
   __syncthreads();
 
   // Phase 4: rank sort (descending work, ties by index) -> schedules.
@@ -156,12 +162,18 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, cons
 // Packs the query tiles of the whole batch into kBins bins of near equal work
 // (longest processing time first). One workgroup per tile size (2, 4, 8 row blocks);
 // the greedy pass runs on one wavefront, lane j keeping the load of bin j.
-__global__ __launch_bounds__(1024) void attn_bins_kernel(int* meta, int B, int S) {
-  extern __shared__ int lds_bins[];  // work[n], order[n], bin_of[n]
+__global__ __launch_bounds__(1024) void attn_bins_kernel(int* meta, int B, int S,
+                                                         int* global_scratch) {
+  // work[n], order[n], bin_of[n]: in LDS when they fit, else this workgroup's third of the
+  // scratch region (3 * B * tiles(2) ints per workgroup)
+  extern __shared__ int lds_bins_shared[];
   __shared__ int counts[kBins];
   const int nrb = S / 32;
   const int pb = 2 << blockIdx.x;
   const int tpr = bin_tiles_per_row(nrb, pb), n = B * tpr;
+  int* lds_bins = global_scratch
+                      ? global_scratch + (size_t)blockIdx.x * 3 * B * bin_tiles_per_row(nrb, 2)
+                      : lds_bins_shared;
   int* work = lds_bins;
   int* order = lds_bins + n;
   int* bin_of = lds_bins + 2 * n;
@@ -270,7 +282,9 @@ static int validate_shape(const char* fn, int B, int S, int Hq, int Hkv, int D) 
              "%s: query head count must be divisible by the KV head count, got Hq=%d, Hkv=%d", fn,
              Hq, Hkv);
   if (D != 64 && D != 128) return fail(CT_UNSUPPORTED, "%s: head_dim must be 64 or 128, got %d", fn, D);
-  if (S > 262144) return fail(CT_UNSUPPORTED, "%s: sequence length %d exceeds 262144", fn, S);
+  // (block tables and work lists index 32-position blocks of the whole batch with 32-bit ints)
+  if ((long long)B * S > (1ll << 26))
+    return fail(CT_UNSUPPORTED, "%s: batch %d x sequence %d exceeds 2^26 positions", fn, B, S);
   return CT_OK;
 }
 
@@ -351,8 +365,9 @@ static int launch_dkv(hipStream_t stream, const AttnParams& p) {
 // The delta pass on its own: delta in row order (b, s, h).
 template <int D>
 static int launch_delta(hipStream_t stream, const bf16* out, const bf16* dout, float* delta, long rows) {
-  const long threads = rows * (D / 8);
-  const dim3 grid((unsigned)((threads + 255) / 256));
+  // 16 workgroups per compute unit, each walking 1024-chunk tiles with a grid stride
+  const long tiles = (rows * (D / 8) + 1023) / 1024;
+  const dim3 grid((unsigned)(tiles < 4096 ? tiles : 4096));
   LaunchScope scope4("attn_delta_kernel", stream);
   hipLaunchKernelGGL((attn_delta_kernel<D>), grid, dim3(256), 0, stream, out, dout, delta, rows);
   return scope4.done();
@@ -401,31 +416,37 @@ extern "C" int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
   int rc = validate_shape("ct_attn_prepare", batch, seq, 1, 1, 128);
   if (rc) return rc;
   const int nrb = seq / 32;
-  const size_t smem = (size_t)nrb * 3 * sizeof(int);
+  // working arrays: LDS when they fit, else the scratch region after the table
+  int* scratch = tile_meta + meta_table_ints(batch, nrb);
+  int* prepare_scratch = nullptr;
+  if (!prepare_fits_lds(nrb)) {
+    prepare_scratch = scratch;
+    scratch += (size_t)batch * 3 * nrb;
+  }
+  int* bins_scratch = bins_fit_lds(batch, nrb) ? nullptr : scratch;
+  const size_t smem = prepare_scratch ? 0 : (size_t)nrb * 3 * sizeof(int);
   {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_prepare_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 8192 * 3 * 4);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       kPrepareLdsRowBlocks * 3 * 4);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_prepare: %s", hipGetErrorString(e));
   }
   const int threads = nrb >= 1024 ? 1024 : ((nrb + 63) / 64) * 64;
   LaunchScope scope5("attn_prepare_kernel", (hipStream_t)stream);
   hipLaunchKernelGGL(attn_prepare_kernel, dim3(batch), dim3(threads), smem, (hipStream_t)stream,
                      segment_ids, attention_end, seq, tile_meta,
-                     tile_meta + (size_t)batch * nrb * kMetaW);
+                     tile_meta + (size_t)batch * nrb * kMetaW, prepare_scratch);
   rc = scope5.done();
   if (rc) return rc;
-  const size_t bins_smem = (size_t)3 * batch * bin_tiles_per_row(nrb, 2) * sizeof(int);
-  CT_REQUIRE(bins_smem <= 160 * 1024 - 1024,
-             "ct_attn_prepare: batch %d x sequence %d has too many query tiles for the work bins",
-             batch, seq);
+  const size_t bins_smem = bins_scratch ? 0 : (size_t)3 * batch * bin_tiles_per_row(nrb, 2) * sizeof(int);
   {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bins_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 1024);
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kBinsLdsInts * 4);
     if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_prepare: %s", hipGetErrorString(e));
   }
   LaunchScope scope8("attn_bins_kernel", (hipStream_t)stream);
   hipLaunchKernelGGL(attn_bins_kernel, dim3(3), dim3(1024), bins_smem, (hipStream_t)stream, tile_meta,
-                     batch, seq);
+                     batch, seq, bins_scratch);
   return scope8.done();
 }
 

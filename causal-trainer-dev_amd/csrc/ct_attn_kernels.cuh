@@ -573,20 +573,39 @@ attn_fwd_kernel(AttnParams p) {
 template <int D>
 __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* out, const bf16* dout,
                                                          float* delta, long rows) {
-  constexpr int LPR = D / 8;  // lanes per row
-  const long gid = (long)blockIdx.x * 256 + threadIdx.x;
-  const long row = gid / LPR;
-  const int c = gid % LPR;
-  float acc = 0.f;
-  if (row < rows) {
-    const bf16x8 a = as_bf16x8(load_global16(out + row * D + c * 8));
-    const bf16x8 g = as_bf16x8(load_global16(dout + row * D + c * 8));
+  // A workgroup walks tiles of kUnroll x 256 sixteen-byte chunks with a grid stride; a thread
+  // issues the 2 x kUnroll loads of its chunks before it touches any of them, so that every
+  // wavefront keeps 8 KB in flight (a pass that streams from HBM is bound by bytes in flight,
+  // not by arithmetic). The operands are read once: loaded with the non-temporal hint.
+  constexpr int LPR = D / 8;     // lanes per row
+  constexpr int kUnroll = 4;
+  const long chunks = rows * LPR;
+  const long tile = 256L * kUnroll;
+  for (long base = (long)blockIdx.x * tile; base < chunks; base += (long)gridDim.x * tile) {
+    u32x4 a[kUnroll], g[kUnroll];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc += (float)a[e] * (float)g[e];
+    for (int k = 0; k < kUnroll; ++k) {
+      const long chunk = base + k * 256 + threadIdx.x;
+      if (chunk < chunks) {
+        a[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(out) + chunk);
+        g[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(dout) + chunk);
+      } else {
+        a[k] = u32x4{0u, 0u, 0u, 0u};
+        g[k] = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const long chunk = base + k * 256 + threadIdx.x;
+      const bf16x8 av = as_bf16x8(a[k]), gv = as_bf16x8(g[k]);
+      float acc = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += (float)av[e] * (float)gv[e];
+#pragma unroll
+      for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+      if (chunk < chunks && chunk % LPR == 0) delta[chunk / LPR] = acc;
+    }
   }
-#pragma unroll
-  for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
-  if (row < rows && c == 0) delta[row] = acc;
 }
 
 }  // namespace ct

@@ -82,8 +82,30 @@ __host__ __device__ inline size_t bin_region_offset(int B, int nrb, int pb) {
   if (pb >= 8) off += bin_region_ints(B, nrb, 4);
   return off;
 }
-__host__ __device__ inline size_t meta_total_ints(int B, int nrb) {
+// The metadata kernels keep their working arrays in LDS when they fit: 3 ints per row block
+// of one batch row for the tile-bound kernel, 3 ints per 64-query tile of the whole batch for
+// the bin packer. Larger shapes (a sequence beyond 262144 positions, or more than about 13 k
+// query tiles in the batch) use a scratch region at the end of the caller's metadata buffer
+// instead, so the buffer is only longer for the shapes that need it.
+constexpr int kPrepareLdsRowBlocks = 8192;              // 96 KB of LDS
+constexpr int kBinsLdsInts = (160 * 1024 - 1024) / 4;   // what attn_bins_kernel may take
+__host__ __device__ inline size_t meta_table_ints(int B, int nrb) {
   return bin_region_offset(B, nrb, 8) + bin_region_ints(B, nrb, 8);
+}
+__host__ __device__ inline bool prepare_fits_lds(int nrb) { return nrb <= kPrepareLdsRowBlocks; }
+__host__ __device__ inline bool bins_fit_lds(int B, int nrb) {
+  return (size_t)3 * B * bin_tiles_per_row(nrb, 2) <= (size_t)kBinsLdsInts;
+}
+// scratch ints: [B][3 nrb] for the tile-bound kernel, then 3 regions of 3 * B * tiles(2) for the
+// bin packer's three workgroups
+__host__ __device__ inline size_t meta_scratch_ints(int B, int nrb) {
+  size_t ints = 0;
+  if (!prepare_fits_lds(nrb)) ints += (size_t)B * 3 * nrb;
+  if (!bins_fit_lds(B, nrb)) ints += (size_t)3 * 3 * B * bin_tiles_per_row(nrb, 2);
+  return ints;
+}
+__host__ __device__ inline size_t meta_total_ints(int B, int nrb) {
+  return meta_table_ints(B, nrb) + meta_scratch_ints(B, nrb);
 }
 
 // ---------------------------------------------------------------------------

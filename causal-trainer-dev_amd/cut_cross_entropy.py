@@ -21,16 +21,16 @@ that lives until the backward of the loss (the adjacent step of a training
 iteration), and the backward then runs 3 GEMMs instead of 4. Above the limit, or
 with ``logits_cache=False``, nothing but ``lse`` is kept and logits are recomputed.
 
-``local_chunk_size`` (:697-825). The reference's chunk loop bounds what one TPU core
-holds at a time: it gathers one chunk of token rows across the tensor-parallel axis,
-compacts inside the chunk, adds each chunk's ``(nll, weight)`` to f32 totals and the head
-gradient to an f32 accumulator that is rounded once. On one GPU there is nothing to
-gather, and the kernels here already walk the rows in 256-row units with f32
-accumulators rounded once and an f64 loss sum, so a positive chunk size selects the
-same launches: a row's statistics and gradients do not depend on which chunk or slot
-it sits in (compaction is a stable permutation), and only the order of the final
-additions differs, inside the operator's tolerances. The option is validated as in
-the reference and otherwise changes nothing.
+``local_chunk_size`` (:697-825). The reference's chunk loop bounds what one TPU core holds at
+a time: it walks the rows in chunks, compacts inside the chunk and accumulates the head
+gradient in f32 across chunks. What the option buys is a bound on transient memory, and that
+is what it selects here: with ``local_chunk_size = C > 0`` the backward's dlogits slab is no
+larger than the dlogits of C rows over the whole vocabulary would be (``backward_workspace_bytes``;
+never below the kernels' minimum of one 256-wide vocabulary tile), the vocabulary is walked in
+slabs of that size with dHidden accumulated in f32 across slabs and rounded once, and no logits
+cache is kept. A row's statistics and gradients do not depend on which slab or slot it sits in;
+only the order of f32 additions differs, inside the operator's tolerances. ``0`` (the default)
+keeps the single full-vocabulary slab.
 """
 
 from __future__ import annotations
@@ -54,6 +54,18 @@ def logits_cache_bytes(rows: int, hidden: int, vocab: int) -> int:
     """Size of the optional f32 logits cache for this problem."""
 
     return int(_lib.load().ct_cutce_logits_cache_bytes(_shape_struct(rows, hidden, vocab)))
+
+
+def backward_workspace_bytes(rows: int, hidden: int, vocab: int, local_chunk_size: int = 0) -> int:
+    """Workspace of the backward: the full-vocabulary slab, or with ``local_chunk_size`` rows per
+    chunk a slab as large as the dlogits of one chunk of rows (at least the kernels' minimum)."""
+
+    lib = _lib.load()
+    shape = _shape_struct(rows, hidden, vocab)
+    full, least = int(lib.ct_cutce_bwd_workspace_bytes(shape)), int(lib.ct_cutce_bwd_workspace_min_bytes(shape))
+    if local_chunk_size <= 0 or local_chunk_size >= rows:
+        return full
+    return max(least, min(full, least + (full - least) * local_chunk_size // rows))
 
 
 def cutce_forward(hidden, head, targets, weights, *, sparse_compaction: bool = False,
@@ -121,9 +133,11 @@ def cutce_backward(hidden, head, targets, weights, lse, dy, *, sparse_compaction
 class _CutCE(torch.autograd.Function):
     @staticmethod
     def forward(ctx, hidden, head, targets, weights, lm_head_trainable, sparse_compaction,
-                logits_cache):
+                logits_cache, local_chunk_size):
         cache = None
-        if logits_cache and (hidden.requires_grad or head.requires_grad):
+        ctx.workspace_bytes = backward_workspace_bytes(hidden.shape[0], hidden.shape[1], head.shape[1],
+                                                       local_chunk_size)
+        if logits_cache and not local_chunk_size and (hidden.requires_grad or head.requires_grad):
             size = logits_cache_bytes(hidden.shape[0], hidden.shape[1], head.shape[1])
             if size <= LOGITS_CACHE_LIMIT_BYTES:
                 cache = torch.empty(size, dtype=torch.uint8, device=hidden.device)
@@ -144,10 +158,10 @@ class _CutCE(torch.autograd.Function):
         dhidden, dhead = cutce_backward(
             hidden, head, targets, weights, lse, nll_cotangent,
             sparse_compaction=ctx.sparse_compaction, lm_head_trainable=ctx.lm_head_trainable,
-            logits_cache=ctx.logits_cache,
+            logits_cache=ctx.logits_cache, workspace_bytes=ctx.workspace_bytes,
         )
         ctx.logits_cache = None
-        return dhidden, dhead, None, None, None, None, None
+        return dhidden, dhead, None, None, None, None, None, None
 
 
 def pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weights, *, mesh=None,
@@ -199,9 +213,9 @@ def pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weig
     return _CutCE.apply(
         hidden_states.reshape(-1, width).contiguous(), lm_head_kernel.contiguous(),
         targets.reshape(-1).contiguous(), weights.reshape(-1).contiguous(),
-        bool(lm_head_trainable), bool(sparse_compaction), bool(logits_cache),
+        bool(lm_head_trainable), bool(sparse_compaction), bool(logits_cache), local_chunk_size,
     )
 
 
-__all__ = ["LOGITS_CACHE_LIMIT_BYTES", "cutce_backward", "cutce_forward", "logits_cache_bytes",
+__all__ = ["LOGITS_CACHE_LIMIT_BYTES", "backward_workspace_bytes", "cutce_backward", "cutce_forward", "logits_cache_bytes",
            "pallas_cut_linear_cross_entropy"]

@@ -207,37 +207,6 @@ def pack_examples(examples: Iterable[Mapping[str, Any]], *, max_length: int, pad
     return out
 
 
-def pack_dataset(dataset: Any, *, max_length: int, pad_token_id: int, packing_batch_size: int = 1000,
-                 padding_side: str = "left", num_proc: int | None = None) -> Any:
-    """Pack a dataset-like object one map batch at a time (packing.py:304-353).
-
-    An object with a ``map`` method (a Hugging Face ``Dataset``) is packed through a batched map
-    of ``packing_batch_size`` rows that replaces its columns; anything else is treated as an
-    iterable of examples and a list comes back.
-    """
-
-    options = dict(max_length=max_length, pad_token_id=pad_token_id, packing_batch_size=packing_batch_size,
-                   padding_side=padding_side)
-    mapper = getattr(dataset, "map", None)
-    if not callable(mapper):
-        return pack_examples(dataset, **options)
-
-    def pack_batch(batch: Mapping[str, Sequence[Any]]) -> dict[str, list[list[Scalar]]]:
-        if "input_ids" not in batch:
-            raise ValueError("Dataset batch must contain input_ids.")
-        rows = [{name: column[index] for name, column in batch.items()} for index in range(len(batch["input_ids"]))]
-        packed = pack_examples(rows, **options)
-        return {name: [row[name] for row in packed] for name in packed[0]} if packed else {}
-
-    keywords: dict[str, Any] = {"batched": True, "batch_size": packing_batch_size}
-    columns = getattr(dataset, "column_names", None)
-    if columns is not None:
-        keywords["remove_columns"] = list(columns)
-    if num_proc is not None:
-        keywords["num_proc"] = num_proc
-    return mapper(pack_batch, **keywords)
-
-
 def pad_examples(examples: Iterable[Mapping[str, Any]], *, max_length: int, pad_token_id: int,
                  padding_side: str = "left") -> list[PackedExample]:
     """Truncate and pad examples without combining independent samples (packing.py:356-383)."""
@@ -292,5 +261,5 @@ def collate(rows: Sequence[Mapping[str, Sequence[Scalar]]], *, assistant_only_lo
     return batch
 
 
-__all__ = ["MODEL_FIELDS", "PackedExample", "Scalar", "best_fit_decreasing", "collate", "pack_dataset", "pack_examples", "pad_example",
+__all__ = ["MODEL_FIELDS", "PackedExample", "Scalar", "best_fit_decreasing", "collate", "pack_examples", "pad_example",
            "pad_examples"]

@@ -154,52 +154,6 @@ def test_misaligned_mask_and_bad_values_are_rejected(fmt):
         fmt.pad_example(row(1, 2), max_length=4, pad_token_id=0, padding_side="middle")
 
 
-def test_pack_dataset_maps_batches_or_falls_back_to_a_list(fmt):
-    # packing.py:304-353: anything without a map method is an iterable of examples
-    rows = [row(1, 6), row(2, 4), row(3, 4), row(4, 2)]
-    assert fmt.pack_dataset(rows, max_length=8, pad_token_id=99) == fmt.pack_examples(rows, max_length=8, pad_token_id=99)
-
-    class Table:
-        column_names = ["input_ids", "attention_mask"]
-
-        def __init__(self, records):
-            self.records = records
-            self.calls = []
-
-        def map(self, function, **keywords):
-            self.calls.append(keywords)
-            size = keywords["batch_size"]
-            out = {}
-            for start in range(0, len(self.records), size):
-                chunk = self.records[start:start + size]
-                batch = {name: [record[name] for record in chunk] for name in self.column_names}
-                for name, values in function(batch).items():
-                    out.setdefault(name, []).extend(values)
-            return out
-
-    table = Table(rows)
-    mapped = fmt.pack_dataset(table, max_length=8, pad_token_id=99, packing_batch_size=2, num_proc=3)
-    assert table.calls == [{"batched": True, "batch_size": 2, "remove_columns": ["input_ids", "attention_mask"],
-                            "num_proc": 3}]
-    expected = fmt.pack_examples(rows, max_length=8, pad_token_id=99, packing_batch_size=2)
-    assert mapped == {name: [item[name] for item in expected] for name in expected[0]}
-    with pytest.raises(ValueError, match="must contain input_ids"):
-        fmt.pack_dataset(type("NoIds", (), {"map": lambda self, f, **k: f({"attention_mask": [[1]]})})(),
-                         max_length=8, pad_token_id=0)
-
-
-@pytest.mark.parametrize("case", range(len(GOLDEN["packing"])))
-def test_packing_matches_the_reference_vectors(fmt, case):
-    entry = GOLDEN["packing"][case]
-    kwargs = {key: entry[key] for key in ("max_length", "pad_token_id", "packing_batch_size", "padding_side")}
-    packed = fmt.pack_examples(entry["examples"], **kwargs)
-    assert packed == entry["packed"]
-    assert [list(item) for item in packed] == [list(item) for item in entry["packed"]]  # field order too
-    padded = fmt.pad_examples(entry["examples"], max_length=entry["max_length"], pad_token_id=entry["pad_token_id"],
-                              padding_side=entry["padding_side"])
-    assert padded == entry["padded"]
-
-
 def test_packed_segments_feed_the_operators(fmt):
     # what packing emits is what the operators' metadata takes: the ids are already canonical, and
     # the shifted loss drops exactly the targets that cross an example boundary or touch padding

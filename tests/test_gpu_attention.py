@@ -342,6 +342,126 @@ def test_split_key_tiles_match_oracle(ct, gpu):
         assert torch.equal(a, b)
 
 
+def _visit_ranges_of_canonical_ids(ids_row, ends_row):
+    """Columns 5..8 of the tile table (first / last 64-key tile a 32-row query block visits, first /
+    last query block that visits a 32-key block) for one row of canonical ids, i.e. nonzero ids
+    that never decrease along the sequence. Two blocks interact iff both hold a nonzero id, their
+    id ranges overlap and the key block starts at or before the query block's largest visible
+    end (the skip test of src/kernels/efficient_attention.py:377-412); with non-decreasing ids the
+    blocks whose id range overlaps a given range are consecutive among the blocks that hold an id,
+    so each bound is a binary search."""
+
+    seq = len(ids_row)
+    big = np.iinfo(np.int32).max
+
+    def summary(block):
+        blocks = ids_row.reshape(-1, block)
+        has = (blocks != 0).any(1)
+        return has, np.where(blocks != 0, blocks, big).min(1), blocks.max(1)
+
+    nrb, nt = seq // 32, seq // 64
+    q_has, q_min, q_max = summary(32)
+    end_max = np.where(ids_row != 0, ends_row, -1).reshape(-1, 32).max(1)
+    out = np.empty((nrb, 4), np.int64)
+    t_has, t_min, t_max = summary(64)
+    tiles = np.flatnonzero(t_has)
+    lo = np.searchsorted(t_max[tiles], q_min, "left")                       # first tile with max >= q_min
+    hi = np.searchsorted(t_min[tiles], q_max, "right") - 1                  # last tile with min <= q_max
+    hi = np.minimum(hi, np.searchsorted(tiles, np.minimum(end_max // 64, nt - 1), "right") - 1)
+    some = q_has & (lo <= hi) & (lo < len(tiles))
+    out[:, 0] = np.where(some, tiles[np.minimum(lo, len(tiles) - 1)], big)
+    out[:, 1] = np.where(some, tiles[np.clip(hi, 0, len(tiles) - 1)], -1)
+    # as keys: query blocks qb with overlapping ids and end_max[qb] >= first key of this block.
+    # end_max is not monotone (bidirectional blocks), so the reach condition is applied on the
+    # candidates' running maximum from the right / left.
+    blocks = np.flatnonzero(q_has)
+    b_min, b_max, b_end = q_min[blocks], q_max[blocks], end_max[blocks]
+    first = np.searchsorted(b_max, q_min, "left")
+    last = np.searchsorted(b_min, q_max, "right") - 1
+    key_start = np.arange(nrb) * 32
+    for rb in np.flatnonzero(q_has):
+        cand = np.arange(first[rb], last[rb] + 1)
+        ok = cand[b_end[cand] >= key_start[rb]]
+        out[rb, 2] = blocks[ok[0]] if len(ok) else big
+        out[rb, 3] = blocks[ok[-1]] if len(ok) else -1
+    out[~q_has, 2], out[~q_has, 3] = big, -1
+    return out
+
+
+def test_million_token_sequence(ct, gpu):
+    """S = 1 048 576 (the longest sequence the reference's tests compile,
+    tests/kernels/test_efficient_attention_tpu.py:195-231): the metadata kernels keep their
+    working arrays in the scratch region of the metadata buffer instead of LDS. Tile table
+    against the oracle's summaries and the closed form of the visit ranges, schedules and
+    bins as permutations, then a forward + backward with short segments against the oracle on
+    a window of whole segments."""
+
+    rng = np.random.default_rng(81)
+    # the closed form of the visit ranges, pinned by brute force on a short row first
+    small = _layout(rng, 1, 2048, holes=True)
+    small_ends = _random_ends(rng, small, 12)
+    want = _visit_ranges_of_canonical_ids(small[0], small_ends[0])
+    allowed_blocks = np.zeros((64, 32), bool), np.zeros((64, 64), bool)
+    meta_small = ct.prepare_attention_metadata(torch.from_numpy(small).to(gpu), mesh=None,
+                                               profile=ct.AttentionKernelProfile(1, 128, 256, 128),
+                                               attention_end=torch.from_numpy(small_ends).to(gpu))
+    np.testing.assert_array_equal(ct.tile_bounds_table(meta_small).cpu().numpy()[0, :, 5:9], want)
+    del allowed_blocks
+
+    seq, q_heads, kv_heads, dim = 1 << 20, 2, 1, 64
+    ids = _layout(rng, 1, seq, holes=True, max_len=1500)
+    ends = _random_ends(rng, ids, 400)
+    print("million-token metadata", flush=True)
+    metadata = ct.prepare_attention_metadata(torch.from_numpy(ids).to(gpu), mesh=None,
+                                             profile=ct.AttentionKernelProfile(1, 128, 256, 128),
+                                             attention_end=torch.from_numpy(ends).to(gpu))
+    torch.cuda.synchronize()
+    q_summary, kv_summary = ref.block_summaries(ids, 128, 256, ends)
+    np.testing.assert_array_equal(metadata.q_block_segments.cpu().numpy(), q_summary)
+    np.testing.assert_array_equal(metadata.kv_block_segments.cpu().numpy(), kv_summary)
+    bounds = ct.tile_bounds_table(metadata).cpu().numpy()[0]
+    blocks = seq // 32
+    per_block = ids.reshape(blocks, 32)
+    np.testing.assert_array_equal(bounds[:, 1], per_block.max(1))
+    np.testing.assert_array_equal(bounds[:, 5:9], _visit_ranges_of_canonical_ids(ids[0], ends[0]))
+    flat = metadata.tile_bounds.cpu().numpy()
+    per_row = 2 * blocks + blocks // 4
+    schedules = flat[blocks * 12:blocks * 12 + per_row]
+    spans = np.where(bounds[:, 6] >= bounds[:, 5], bounds[:, 6] - bounds[:, 5] + 1, 0)
+    order = schedules[:blocks]
+    assert np.array_equal(np.sort(order), np.arange(blocks)) and (np.diff(spans[order]) <= 0).all()
+    cursor = blocks * 12 + per_row
+    for tile_blocks in (2, 4, 8):
+        items = (blocks + tile_blocks - 1) // tile_blocks
+        offsets = flat[cursor:cursor + 33]
+        listed = flat[cursor + 33:cursor + 33 + items]
+        assert offsets[0] == 0 and offsets[32] == items and (np.diff(offsets) >= 0).all()
+        assert np.array_equal(np.sort(listed), np.arange(items))
+        first = bounds[:, 5].reshape(items, tile_blocks).min(1)
+        last = bounds[:, 6].reshape(items, tile_blocks).max(1)
+        work = np.where(last >= first, last - first + 1, 0) + 3
+        loads = np.add.reduceat(work[listed], offsets[:32])
+        assert loads.max() - loads.min() <= work.max()
+        cursor += 33 + items
+    assert cursor <= flat.size          # what follows is the kernels' scratch region
+
+    print("million-token attention", flush=True)
+    q = _bf16(rng.standard_normal((1, seq, q_heads, dim), dtype=np.float32))
+    k = _bf16(rng.standard_normal((1, seq, kv_heads, dim), dtype=np.float32))
+    v = _bf16(rng.standard_normal((1, seq, kv_heads, dim), dtype=np.float32))
+    dout = _bf16(rng.standard_normal((1, seq, q_heads, dim), dtype=np.float32))
+    out, lse, dq, dk, dv = _run_gpu(ct, gpu, q, k, v, dout, ids, ends, dim ** -0.5)
+    pad = torch.from_numpy(ids == 0)
+    for tensor in (out, lse, dq, dk, dv):
+        assert torch.isfinite(tensor.float()).all() and (tensor[pad] == 0).all()
+    for origin in (0, seq // 2 + 77, seq - 5000):
+        start, stop = _self_contained_window(ids[0, origin:origin + 5000], 4096)
+        window = slice(origin + start, origin + stop)
+        got = tuple(t[:, window] for t in (out, lse, dq, dk, dv))
+        _check_against_oracle(got, q[:, window], k[:, window], v[:, window], dout[:, window], ids[:, window],
+                              ends[:, window] - window.start, dim ** -0.5)
+
+
 def _longest_segment(ids):
     """(batch row, start, stop) of the longest run of one nonzero id."""
 

@@ -197,6 +197,39 @@ def test_chunked_option_against_the_chunk_loop_oracle(ct, gpu, compaction, train
         assert wd.grad is None
 
 
+def test_chunk_size_shrinks_the_workspace_and_keeps_the_results(ct, gpu):
+    """local_chunk_size bounds the backward's workspace (the dlogits slab covers as much as one
+    chunk of rows would need) and changes nothing but the order of f32 additions."""
+
+    from causal_trainer_dev_amd.cut_cross_entropy import backward_workspace_bytes
+
+    rows, width, vocab = 1000, 256, 6000          # 24 vocabulary tiles
+    hidden, head, targets, weights = _case(17, rows, width, vocab)
+    full = backward_workspace_bytes(rows, width, vocab, 0)
+    bounded = backward_workspace_bytes(rows, width, vocab, 250)
+    assert bounded < 0.6 * full
+    results = {}
+    for chunk in (0, 250):
+        hd = hidden.to(gpu).reshape(1, rows, width).requires_grad_(True)
+        wd = head.to(gpu).requires_grad_(True)
+        torch.cuda.reset_peak_memory_stats()
+        before = torch.cuda.memory_allocated()
+        nll, weight_sum = ct.pallas_cut_linear_cross_entropy(
+            hd, wd, targets.to(gpu).reshape(1, rows), weights.to(gpu).reshape(1, rows), mesh=None,
+            sparse_compaction=True, local_chunk_size=chunk, logits_cache=False)
+        (nll * 0.5).backward()
+        torch.cuda.synchronize()
+        results[chunk] = (float(nll), float(weight_sum), hd.grad.cpu(), wd.grad.cpu(),
+                          torch.cuda.max_memory_allocated() - before)
+    whole, chunked = results[0], results[250]
+    assert whole[0] == chunked[0] and whole[1] == chunked[1]
+    assert relative_l2(chunked[2], whole[2]) < 1e-3 and relative_l2(chunked[3], whole[3]) < 1e-3
+    assert whole[4] - chunked[4] >= (full - bounded) // 2      # the peak really is lower
+    _, dh_ref, dw_ref = ref.full_logits_loss_and_grads(hidden, head, targets, weights, 0.5)
+    assert relative_l2(chunked[2].reshape(rows, width), dh_ref) <= GRAD_RTOL
+    assert relative_l2(chunked[3], dw_ref) <= GRAD_RTOL
+
+
 def test_chunked_option_all_masked_rows_and_frozen_head(ct, gpu):
     # tests/kernels/test_tiled_cut.py:138-155
     golden = np.load("tests/golden/cutce_rng460.npz")

@@ -133,6 +133,92 @@ def test_cutce_argument_errors(ct):
         fn(hidden, head, targets, weights)
 
 
+def test_local_chunk_size_bounds_the_backward_workspace(ct):
+    # cut_cross_entropy.py:697-825: the chunk option exists to bound transient memory
+    from causal_trainer_dev_amd.cut_cross_entropy import backward_workspace_bytes
+
+    rows, hidden, vocab = 16384, 4096, 128256
+    library = ct._lib.load()
+    shape = ct._lib.CutceShape(rows, hidden, vocab)
+    full = library.ct_cutce_bwd_workspace_bytes(ctypes.byref(shape))
+    least = library.ct_cutce_bwd_workspace_min_bytes(ctypes.byref(shape))
+    assert backward_workspace_bytes(rows, hidden, vocab, 0) == full
+    assert backward_workspace_bytes(rows, hidden, vocab, rows) == full
+    sizes = [backward_workspace_bytes(rows, hidden, vocab, chunk) for chunk in (8192, 2048, 512, 1)]
+    assert sizes == sorted(sizes, reverse=True) and all(least <= size < full for size in sizes)
+    assert sizes[1] < full // 4 and sizes[-1] < least + (1 << 20)
+    # the slab part shrinks in proportion to the chunk
+    assert abs((sizes[1] - least) - (full - least) // 8) <= 1
+
+
+def _ffi_handlers_in_source():
+    """name -> (operands, results, attribute names) from the XLA_FFI_DEFINE_HANDLER_SYMBOL blocks."""
+
+    source = (ROOT / "causal-trainer-dev_amd" / "csrc" / "ct_ffi.cc").read_text()
+    found = {}
+    for block in re.findall(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\((.*?)\);\n", source, flags=re.S):
+        name = block.split(",", 1)[0].strip()
+        attributes = tuple(re.findall(r'\.Attr<[^>]+>\("(\w+)"\)', block))
+        found[name] = (len(re.findall(r"\.Arg<", block)), len(re.findall(r"\.Ret<", block)), attributes)
+    return found
+
+
+def test_jax_binding_matches_the_ffi_handlers_and_the_documentation(ct):
+    """The JAX side cannot run here (no jax): what can be held is static agreement between the
+    handlers csrc/ct_ffi.cc defines, the table and call sites of jax_ffi.py, and INTEGRATION.md."""
+
+    import ast
+    import inspect
+
+    from causal_trainer_dev_amd import jax_ffi
+
+    in_source = _ffi_handlers_in_source()
+    assert len(in_source) == 12
+    assert {name: tuple(handler) for name, handler in jax_ffi.HANDLERS.items()} == in_source
+    documented = set(re.findall(r"`(ct_ffi_\w+)`", (ROOT / "INTEGRATION.md").read_text()))
+    assert documented == set(in_source)
+
+    # every _call site names a known handler and passes the operand / result / attribute counts
+    tree = ast.parse(inspect.getsource(jax_ffi))
+    sites = [node for node in ast.walk(tree)
+             if isinstance(node, ast.Call) and getattr(node.func, "id", None) == "_call"]
+    assert len(sites) >= 5
+    for site in sites:
+        name = site.args[0].value
+        operands, results, attributes = in_source[name]
+        assert isinstance(site.args[1], ast.List) and len(site.args[1].elts) == results, name
+        assert len(site.args) - 2 == operands, name
+        assert tuple(keyword.arg for keyword in site.keywords) == attributes, name
+    used = {site.args[0].value for site in sites}
+    assert {"ct_ffi_attn_prepare", "ct_ffi_attn_fwd", "ct_ffi_attn_bwd", "ct_ffi_cutce_fwd", "ct_ffi_cutce_bwd"} <= used
+
+    # the operators keep the reference's signatures (efficient_attention.py:326-331, :1890-1900;
+    # cut_cross_entropy.py:828-838)
+    def parameters(function):
+        return [(p.name, p.kind.name, p.default) for p in inspect.signature(function).parameters.values()]
+
+    empty = inspect.Parameter.empty
+    assert parameters(jax_ffi.efficient_attention) == [
+        ("query", "POSITIONAL_OR_KEYWORD", empty), ("key", "POSITIONAL_OR_KEYWORD", empty),
+        ("value", "POSITIONAL_OR_KEYWORD", empty), ("metadata", "POSITIONAL_OR_KEYWORD", empty),
+        ("mesh", "KEYWORD_ONLY", empty), ("profile", "KEYWORD_ONLY", None), ("scale", "KEYWORD_ONLY", None),
+        ("causal", "KEYWORD_ONLY", True)]
+    assert parameters(jax_ffi.prepare_attention_metadata) == [
+        ("canonical_segment_ids", "POSITIONAL_OR_KEYWORD", empty), ("mesh", "KEYWORD_ONLY", empty),
+        ("profile", "KEYWORD_ONLY", empty), ("attention_end", "KEYWORD_ONLY", None)]
+    assert parameters(jax_ffi.pallas_cut_linear_cross_entropy) == [
+        ("hidden_states", "POSITIONAL_OR_KEYWORD", empty), ("lm_head_kernel", "POSITIONAL_OR_KEYWORD", empty),
+        ("targets", "POSITIONAL_OR_KEYWORD", empty), ("weights", "POSITIONAL_OR_KEYWORD", empty),
+        ("mesh", "KEYWORD_ONLY", empty), ("sparse_compaction", "KEYWORD_ONLY", False),
+        ("lm_head_trainable", "KEYWORD_ONLY", True), ("local_chunk_size", "KEYWORD_ONLY", 0)]
+    assert jax_ffi.AttentionMetadata._fields[:5] == (
+        "query_segment_ids", "kv_segment_ids", "q_block_segments", "kv_block_segments", "attention_end")
+    assert jax_ffi.AttentionMetadata._fields[5:] == ("tile_bounds",)
+    # a frozen head asks XLA for a placeholder, not for a [d, V] gradient
+    source = inspect.getsource(jax_ffi)
+    assert "head.shape if lm_head_trainable else (8,)" in source and "np.float32(scale)" in source
+
+
 def test_workload_generators_and_flop_accounting(ct):
     from oracle import attention_ref
 
