@@ -253,7 +253,7 @@ def bench_cutce(ct, torch, steps, warmup, logits_cache=True):
 
     gemm = 2 * active * config.hidden * config.vocab
     per_kernel_flops = {"cutce_stats_kernel": gemm, "cutce_dhidden_kernel": gemm, "cutce_dhead_kernel": gemm,
-                        "cutce_dlogits_kernel": gemm}
+                        "cutce_dlogits_kernel": gemm, "cutce_grads_kernel": 2 * gemm}  # dHidden + dHead in one launch
     table = []
     for name, durations in kernels.items():
         entry = {"kernel": name, "launches": len(durations), "avg_ms": mean(durations)}
@@ -269,9 +269,9 @@ def bench_cutce(ct, torch, steps, warmup, logits_cache=True):
         "roofline": {"bound": "mfma", "kernel": dominant["kernel"], "achieved": dominant["algorithmic_tflops"],
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": dominant["algorithmic_tflops"] / PEAK_BF16_TFLOPS,
-                     "avg_launch_ms": dominant["avg_ms"], "flops_per_launch": gemm,
+                     "avg_launch_ms": dominant["avg_ms"], "flops_per_launch": per_kernel_flops[dominant["kernel"]],
                      "traffic": measured_traffic(dominant["kernel"])},
-        "gemms_executed": len(gemms) + (0 if logits_cache else 1),
+        "gemms_executed": 3 if logits_cache else 4,
         "logits_cache": bool(logits_cache),
         "logits_cache_bytes": 0 if cache is None else cache.numel(),
         "active_rows": active,

@@ -361,7 +361,10 @@ CT_DEVICE void store_global16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) =
 // per-store vector address arithmetic. The scalar base may have just been written by a vector
 // instruction (v_readfirstlane): a memory instruction that reads such a register needs 5 wait
 // states after the write, and the compiler does not add them in front of an asm statement, so
-// each of these stores carries them itself (s_nop 4).
+// each of these stores carries them itself (s_nop 4). A store of more than 8 bytes has a second
+// hazard the compiler cannot see through an asm statement: a vector instruction must not write
+// the registers that hold the store's data for 2 wait states after it (the data is read late),
+// so the 16-byte form ends with s_nop 1.
 template <int IMM>
 CT_DEVICE void store_global4_s(void* uniform_base, unsigned lane_offset, float value) {
   static_assert(IMM >= 0 && IMM < 4096, "immediate offset out of range");
@@ -380,7 +383,7 @@ CT_DEVICE void store_global16_s(void* uniform_base, unsigned lane_offset, f32x4 
   const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
   const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
   const unsigned long long base = ((unsigned long long)hi << 32) | (unsigned long long)lo;
-  asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 offset:%3" : : "v"(lane_offset), "v"(value), "s"(base), "n"(IMM) : "memory");
+  asm volatile("s_nop 4\n\tglobal_store_dwordx4 %0, %1, %2 offset:%3\n\ts_nop 1" : : "v"(lane_offset), "v"(value), "s"(base), "n"(IMM) : "memory");
 }
 template <int IMM>
 CT_DEVICE void store_global8_s(void* uniform_base, unsigned lane_offset, bf16x4 value) {

@@ -426,7 +426,9 @@ __global__ __launch_bounds__(256) void cutce_rowparams_kernel(CutceParams p, con
                                                               const float* dy, CutceRowParams rp) {
   const int slot = blockIdx.x * 256 + threadIdx.x;
   if (slot >= p.n_pad) return;
-  float f = 0.f, l2 = 0.f;
+  // A slot without weight gets factor 0 and lse = +inf: exp2(x - inf) is exactly 0 for every finite
+  // logit, so the gradient formula gives 0 for it without a per-element test.
+  float f = 0.f, l2 = __builtin_inff();
   int t = -1;
   if (slot < p.header->n_act) {
     const int row = p.idx[slot];
@@ -485,6 +487,13 @@ __global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, Cutce
 
       bf16* origin = G + (size_t)(v0 - slab0 + uniform(wm)) * p.n_pad + n0 + uniform(wn);
       const unsigned lane_off = (unsigned)(4 * half * p.n_pad + 4 * j) * 2u;  // bytes
+      // Most tiles hold no target of the wavefront's rows and lie inside the vocabulary: there the
+      // gradient is factor * softmax, three instructions per element. (Slots without weight have
+      // factor 0 and lse = +inf.)
+      bool target_here = false;
+#pragma unroll
+      for (int nb = 0; nb < 4; ++nb) target_here |= (unsigned)(tgt[nb] - (v0 + wm)) < 128u;
+      const bool plain = v0 + kGemmTile <= p.V && !__any(target_here);
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
@@ -492,10 +501,16 @@ __global__ __launch_bounds__(256) void cutce_dlogits_kernel(CutceParams p, Cutce
           const int vrel = 32 * i + 8 * (r >> 2) + (r & 3);
           const int v = v0 + wm + 4 * half + vrel;
           bf16x4 quad;
+          if (plain) {
 #pragma unroll
-          for (int nb = 0; nb < 4; ++nb)
-            quad[nb] = (bf16)((fac[nb] != 0.f && v < p.V)
-                                  ? dlogit(acc.c[i][nb][r], fac[nb], lse2[nb], tgt[nb], v) : 0.f);
+            for (int nb = 0; nb < 4; ++nb)
+              quad[nb] = (bf16)(fac[nb] * exp2_fast(acc.c[i][nb][r] * kLog2e - lse2[nb]));
+          } else {
+#pragma unroll
+            for (int nb = 0; nb < 4; ++nb)
+              quad[nb] = (bf16)((fac[nb] != 0.f && v < p.V)
+                                    ? dlogit(acc.c[i][nb][r], fac[nb], lse2[nb], tgt[nb], v) : 0.f);
+          }
           store_global8_s<0>(origin + (size_t)vrel * p.n_pad, lane_off, quad);
         }
     }
@@ -544,14 +559,12 @@ __global__ __launch_bounds__(256) void cutce_dlogits_cached_kernel(CutceParams p
   }
 }
 
-// dHidden[idx[slot], n] (+)= sum_v G^T[v, slot] head[n, slab0 + v]
-__global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const bf16* G,
-                                                            int slab0, int slab_width, int mode,
-                                                            float* dh_acc, bf16* dhidden) {
+// dHidden[idx[slot], n] (+)= sum_v G^T[v, slot] head[n, slab0 + v]: the workgroup's share of the
+// units, pulled from counter set 0.
+CT_DEVICE void dhidden_units(const CutceParams& p, const bf16* G, int slab0, int slab_width, int mode,
+                             float* dh_acc, bf16* dhidden, const lds_addr smem) {
   // mode: 0 = single slab (store bf16), 1 = first slab (store f32), 2 = middle
   // slab (add f32), 3 = last slab (add, store bf16)
-  extern __shared__ __align__(16) char smem_raw[];
-  const lds_addr smem = lds_address_of(smem_raw);
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
   const int col_blocks = (p.d + kGemmTile - 1) / kGemmTile;
@@ -597,12 +610,17 @@ __global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const
   }
 }
 
-// dHead[m, slab0 + v] = sum_slot packed[slot, m] G^T[v, slot], packed[slot] = hidden[idx[slot]]
-__global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const bf16* packed,
-                                                          const bf16* G, int slab0, int slab_tiles,
-                                                          bf16* dhead) {
+__global__ __launch_bounds__(256) void cutce_dhidden_kernel(CutceParams p, const bf16* G,
+                                                            int slab0, int slab_width, int mode,
+                                                            float* dh_acc, bf16* dhidden) {
   extern __shared__ __align__(16) char smem_raw[];
-  const lds_addr smem = lds_address_of(smem_raw);
+  dhidden_units(p, G, slab0, slab_width, mode, dh_acc, dhidden, lds_address_of(smem_raw));
+}
+
+// dHead[m, slab0 + v] = sum_slot packed[slot, m] G^T[v, slot], packed[slot] = hidden[idx[slot]]:
+// the workgroup's share of the units, pulled from counter set 1.
+CT_DEVICE void dhead_units(const CutceParams& p, const bf16* packed, const bf16* G, int slab0,
+                           int slab_tiles, bf16* dhead, const lds_addr smem) {
   const int tid = threadIdx.x, l = tid & 63, j = l & 31, half = l >> 5, w = tid >> 6;
   const int wm = (w >> 1) * 128, wn = (w & 1) * 128;
   const int m_blocks = (p.d + kGemmTile - 1) / kGemmTile;
@@ -647,6 +665,28 @@ __global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const b
         }
       }
   }
+}
+
+__global__ __launch_bounds__(256) void cutce_dhead_kernel(CutceParams p, const bf16* packed,
+                                                          const bf16* G, int slab0, int slab_tiles,
+                                                          bf16* dhead) {
+  extern __shared__ __align__(16) char smem_raw[];
+  dhead_units(p, packed, G, slab0, slab_tiles, dhead, lds_address_of(smem_raw));
+}
+
+// Both gradients of a slab in one launch. The hidden gradient has few, long units (45 x 16 at
+// N = 16384, d = 4096: 2.8 per compute unit, so its last round leaves a sixth of the device idle);
+// a workgroup that finds no hidden-gradient unit left goes on to the head-gradient units, which
+// are many and short, and the idle tail of the first fills with work of the second. The two
+// read the same G^T and write different tensors: neither waits for the other.
+__global__ __launch_bounds__(256) void cutce_grads_kernel(CutceParams p, const bf16* packed,
+                                                         const bf16* G, int slab0, int slab_width,
+                                                         int slab_tiles, int mode, float* dh_acc,
+                                                         bf16* dhidden, bf16* dhead) {
+  extern __shared__ __align__(16) char smem_raw[];
+  const lds_addr smem = lds_address_of(smem_raw);
+  dhidden_units(p, G, slab0, slab_width, mode, dh_acc, dhidden, smem);
+  dhead_units(p, packed, G, slab0, slab_tiles, dhead, smem);
 }
 
 // ---------------------------------------------------------------------------
@@ -931,6 +971,7 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
   if ((rc = set_smem(cutce_dlogits_kernel, smem, "ct_cutce_bwd"))) return rc;
   if ((rc = set_smem(cutce_dhidden_kernel, smem, "ct_cutce_bwd"))) return rc;
   if ((rc = set_smem(cutce_dhead_kernel, smem, "ct_cutce_bwd"))) return rc;
+  if ((rc = set_smem(cutce_grads_kernel, smem, "ct_cutce_bwd"))) return rc;
 
   LaunchScope scope5("cutce_index_kernel", stream);
   hipLaunchKernelGGL(cutce_index_kernel, dim3(1), dim3(1024), 0, stream, p.weights, p.N, p.n_pad,
@@ -972,16 +1013,19 @@ extern "C" int32_t ct_cutce_bwd(void* stream_, const ct_cutce_bwd_args* a) {
       if ((rc = scope7.done())) return rc;
     }
     const int mode = L.slabs == 1 ? 0 : (s == 0 ? 1 : (s == L.slabs - 1 ? 3 : 2));
-    LaunchScope scope8("cutce_dhidden_kernel", stream);
     const int col_blocks = (p.d + kGemmTile - 1) / kGemmTile;
-    hipLaunchKernelGGL(cutce_dhidden_kernel, dim3(min(cus, row_blocks * col_blocks)), dim3(256), smem,
-                       stream, p, G, slab0, slab_width, mode, dh_acc, dhidden);
-    if ((rc = scope8.done())) return rc;
     if (dhead) {
-      LaunchScope scope9("cutce_dhead_kernel", stream);
-      hipLaunchKernelGGL(cutce_dhead_kernel, dim3(min(cus, col_blocks * slab_tiles)), dim3(256), smem,
-                         stream, p, packed, G, slab0, slab_tiles, dhead);
-      if ((rc = scope9.done())) return rc;
+      // both gradients in one launch: the head-gradient units fill the hidden gradient's tail
+      LaunchScope scope8("cutce_grads_kernel", stream);
+      const int units = max(row_blocks * col_blocks, col_blocks * slab_tiles);
+      hipLaunchKernelGGL(cutce_grads_kernel, dim3(min(cus, units)), dim3(256), smem, stream, p, packed, G,
+                         slab0, slab_width, slab_tiles, mode, dh_acc, dhidden, dhead);
+      if ((rc = scope8.done())) return rc;
+    } else {
+      LaunchScope scope8("cutce_dhidden_kernel", stream);
+      hipLaunchKernelGGL(cutce_dhidden_kernel, dim3(min(cus, row_blocks * col_blocks)), dim3(256), smem,
+                         stream, p, G, slab0, slab_width, mode, dh_acc, dhidden);
+      if ((rc = scope8.done())) return rc;
     }
   }
   return CT_OK;

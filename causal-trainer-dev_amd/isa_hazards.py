@@ -7,7 +7,9 @@ scalar base that the compiler materialises with v_readfirstlane directly before 
 load, store or global->LDS copy is read stale: the access goes to whatever address the register
 pair held before. ``scan`` walks device assembly (``hipcc -S --cuda-device-only``) and reports
 every memory instruction whose scalar operands were written by a vector instruction fewer than
-5 wait states earlier. ``python -m causal_trainer_dev_amd.isa_hazards`` compiles every source of
+5 wait states earlier. It also reports the second hazard of that kind: a store of more than 8 bytes
+reads its data registers late, and a vector instruction that writes one of them within 2 wait
+states of the store replaces the data on its way out. ``python -m causal_trainer_dev_amd.isa_hazards`` compiles every source of
 the library and scans it; tests/test_isa_hazards.py runs the same on the CPU.
 """
 
@@ -21,6 +23,9 @@ from concurrent.futures import ThreadPoolExecutor
 from pathlib import Path
 
 WAIT_STATES = 5
+STORE_DATA_WAIT_STATES = 2
+_WIDE_STORE = re.compile(r"^\s*(global|buffer|flat|scratch)_store_dwordx[34]\s+(.*)")
+_VECTOR_ALU = re.compile(r"^\s*v_\w+\s+(.*)")
 _MEMORY = re.compile(r"^\s*(global_|buffer_|flat_|scratch_)")
 _VECTOR_WRITES_SCALAR = re.compile(
     r"^\s*(v_readfirstlane_b32|v_readlane_b32|v_cmp\w*|v_add_co\w*|v_sub_co\w*|v_subrev_co\w*|v_addc\w*|"
@@ -36,6 +41,15 @@ def _scalar_registers(text: str) -> set:
         found.add(int(match.group(1)))
     if "vcc" in text:
         found.add("vcc")
+    return found
+
+
+def _vector_registers(text: str) -> set:
+    found = set()
+    for match in re.finditer(r"\bv\[(\d+):(\d+)\]", text):
+        found.update(range(int(match.group(1)), int(match.group(2)) + 1))
+    for match in re.finditer(r"(?<![\w\[])v(\d+)\b", text):
+        found.add(int(match.group(1)))
     return found
 
 
@@ -69,6 +83,23 @@ def scan(assembly: str) -> list[str]:
                     break
                 elapsed += _wait_states(earlier)
                 if elapsed >= WAIT_STATES:
+                    break
+        alu = _VECTOR_ALU.match(line)
+        if alu and not text.startswith("v_mfma"):
+            written = _vector_registers(alu.group(1).split(",")[0])
+            elapsed = 0
+            for earlier_number, earlier in reversed(window):
+                store = _WIDE_STORE.match(earlier)
+                if store:
+                    fields = [field.strip() for field in store.group(2).split(",")]
+                    # global_store: vaddr, vdata, saddr; buffer_store: vdata first
+                    data = fields[0] if store.group(1) == "buffer" else (fields[1] if len(fields) > 1 else "")
+                    if _vector_registers(data) & written:
+                        problems.append(f"{kernel}: line {number} '{text}' writes store data of line "
+                                        f"{earlier_number} '{earlier.strip()}' after {elapsed} wait states")
+                        break
+                elapsed += _wait_states(earlier)
+                if elapsed >= STORE_DATA_WAIT_STATES:
                     break
         window.append((number, line))
         if len(window) > 16:

@@ -38,6 +38,16 @@ kernel_c:
 """
     assert len(isa_hazards.scan(two_short)) == 1
     assert isa_hazards.scan("kernel_d:\n\tv_readfirstlane_b32 s16, v4\n\tglobal_load_dword v1, v[2:3], off\n") == []
+    # a 16-byte store reads its data late: no vector write of the data registers for 2 wait states
+    wide = """
+kernel_e:
+	global_store_dwordx4 v252, v[2:5], s[0:1] offset:0
+	v_accvgpr_read_b32 v3, a17
+"""
+    assert len(isa_hazards.scan(wide)) == 1
+    assert isa_hazards.scan(wide.replace("\tv_accvgpr", "\ts_nop 1\n\tv_accvgpr")) == []
+    assert isa_hazards.scan(wide.replace("v3, a17", "v9, a17")) == []
+    assert isa_hazards.scan(wide.replace("dwordx4 v252, v[2:5]", "dwordx2 v252, v[2:3]")) == []
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
