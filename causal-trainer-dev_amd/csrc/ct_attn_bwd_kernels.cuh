@@ -28,6 +28,15 @@ template <int D>
 using LeanTrFrags = std::conditional_t<(D / 8 >= 16), TrFragCompact<D / 8, KSlots::kAccum>,
                                        TrFragOffsets<D / 8, KSlots::kAccum>>;
 
+// P = exp2(S log2e - lse2), dS = P (dP - delta) for one 32-key block, in place in s.
+CT_DEVICE void dq_arith(f32x16& s, const f32x16& dp, float lse2, float delta_q) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float prob = exp2_fast(fmaf(s[r], kLog2e, -lse2));
+    s[r] = prob * (dp[r] - delta_q);
+  }
+}
+
 // One query tile (4 / HS row blocks x HS heads of one KV head), start to finish.
 template <int D, int HS>
 CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int qt, const lds_addr lds_base) {
@@ -100,34 +109,48 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
       nb = key_tile_bounds(ctx.meta_b, t + 1);
     }
     if (ctx.wave_visits(kb, t)) {
-      f32x16 s[2], dp[2];
-      scores_t<D>(CUR * kStage + KvStage<D>::kK, ro, qf, s);
-      scores_t<D>(CUR * kStage + KvStage<D>::kV, ro, dof, dp);
-      {
-        // Same specialisation as the forward: masked scores become -inf, so their
-        // probability exp2(-inf) is exactly 0 and so is dS.
-        const int k_uniform = uniform(kb.uniform);
-        const bool need_seg = ctx.mine.uniform == 0 || ctx.mine.uniform != k_uniform;
-        const bool need_causal = t * kKeyTile + kKeyTile - 1 > ctx.mine.end_min;
-        if (need_seg || need_causal) {
-          const int seg_cmp = ctx.row_valid ? ctx.seg_q : -1;
-          int last_rel = ctx.end_q - t * kKeyTile - 4 * half;
-          if (k_uniform == 0) {
-            mask_scores_t<true, true>(stage + KvStage<D>::kSeg, seg_cmp, last_rel, s);
-          } else {
-            if (seg_cmp != k_uniform) last_rel = -1;
-            mask_scores_t<false, true>(stage, seg_cmp, last_rel, s);
+      // Same specialisation as the forward: masked scores become -inf, so their
+      // probability exp2(-inf) is exactly 0 and so is dS.
+      const int k_uniform = uniform(kb.uniform);
+      const bool need_seg = ctx.mine.uniform == 0 || ctx.mine.uniform != k_uniform;
+      const bool need_causal = t * kKeyTile + kKeyTile - 1 > ctx.mine.end_min;
+      const int seg_cmp = ctx.row_valid ? ctx.seg_q : -1;
+      int last_rel = ctx.end_q - t * kKeyTile - 4 * half;
+      if (k_uniform != 0 && seg_cmp != k_uniform) last_rel = -1;
+      constexpr int kOff = CUR * kStage + KvStage<D>::kK, vOff = CUR * kStage + KvStage<D>::kV;
+      if constexpr (D == 128) {
+        // The tile is worked in its two 32-key halves, each start to finish (S and dP, the
+        // arithmetic, the half's share of dQ): 32 score registers are live at a time instead of
+        // 64, which is what leaves room for the fragment ring of the hand-scheduled sequences
+        // without spilling registers inside this loop.
+        const RowFragOffsets<16> rp = RowFragOffsets<16>::expand(ro);
+        const TrFragOffsets<16, KSlots::kAccum> tp =
+            TrFragOffsets<16, KSlots::kAccum>::expand(TrFragCompact<16, KSlots::kAccum>(lds_base, lane_id_here()));
+        auto half_tile = [&](auto kb_tag) {
+          constexpr int KB = decltype(kb_tag)::value;
+          f32x16 s, dp;
+          dq_sdp_half_128<kOff + KB * 8192, vOff + KB * 8192>(rp, qf, dof, s, dp);
+          if (need_seg || need_causal) {
+            if (k_uniform == 0) mask_block_t<true, true>(stage + KvStage<D>::kSeg, seg_cmp, last_rel, KB, s);
+            else mask_block_t<false, true>(stage, seg_cmp, last_rel, KB, s);
           }
+          dq_arith(s, dp, lse2, delta_q);
+          dq_acc_half_128<kOff + KB * 8192>(tp, pack_acc8(s, 0), pack_acc8(s, 1), dqacc);
+        };
+        half_tile(std::integral_constant<int, 0>{});
+        half_tile(std::integral_constant<int, 1>{});
+      } else {
+        f32x16 s[2], dp[2];
+        scores_t<D>(kOff, ro, qf, s);
+        scores_t<D>(vOff, ro, dof, dp);
+        if (need_seg || need_causal) {
+          if (k_uniform == 0) mask_scores_t<true, true>(stage + KvStage<D>::kSeg, seg_cmp, last_rel, s);
+          else mask_scores_t<false, true>(stage, seg_cmp, last_rel, s);
         }
+        dq_arith(s[0], dp[0], lse2, delta_q);
+        dq_arith(s[1], dp[1], lse2, delta_q);
+        accumulate_t<D>(kOff, LeanTrFrags<D>::fresh(lds_base), s, dqacc);
       }
-#pragma unroll
-      for (int kbk = 0; kbk < 2; ++kbk)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float prob = exp2_fast(fmaf(s[kbk][r], kLog2e, -lse2));
-          s[kbk][r] = prob * (dp[kbk][r] - delta_q);
-        }
-      accumulate_t<D>(CUR * kStage + KvStage<D>::kK, LeanTrFrags<D>::fresh(lds_base), s, dqacc);
     }
     dma_wait_all();
     __syncthreads();

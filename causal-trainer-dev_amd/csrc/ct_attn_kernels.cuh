@@ -171,26 +171,29 @@ CT_DEVICE void tile_mask(lds_addr segk, int tile, int seg_q, int end_q, bool row
 // key offset of accumulator register r of block kb the lane-independent constant
 // 32 kb + 8 (r / 4) + r % 4.
 template <bool SEG, bool CAUSAL>
-CT_DEVICE void mask_scores_t(lds_addr segk, int seg_q_or_never, int last_rel, f32x16* s) {
+CT_DEVICE void mask_block_t(lds_addr segk, int seg_q_or_never, int last_rel, int kb, f32x16& s) {
   // (opaque, so that the lane's share of the addresses below is recomputed here rather than
   // kept in a register across the caller's loop, where it ends up spilled)
   int lane = lane_id();
   asm volatile("" : "+v"(lane));
   const int half = lane >> 5;
 #pragma unroll
-  for (int kb = 0; kb < 2; ++kb)
+  for (int qd = 0; qd < 4; ++qd) {
+    i32x4 sk = {0, 0, 0, 0};
+    if constexpr (SEG) sk = lds_load<i32x4>(segk + (kb * 32 + 8 * qd + 4 * half) * 4);
 #pragma unroll
-    for (int qd = 0; qd < 4; ++qd) {
-      i32x4 sk = {0, 0, 0, 0};
-      if constexpr (SEG) sk = lds_load<i32x4>(segk + (kb * 32 + 8 * qd + 4 * half) * 4);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        bool ok = true;
-        if constexpr (SEG) ok = sk[e] == seg_q_or_never;
-        if constexpr (CAUSAL) ok = ok && (kb * 32 + 8 * qd + e <= last_rel);
-        s[kb][4 * qd + e] = ok ? s[kb][4 * qd + e] : kNegInf;
-      }
+    for (int e = 0; e < 4; ++e) {
+      bool ok = true;
+      if constexpr (SEG) ok = sk[e] == seg_q_or_never;
+      if constexpr (CAUSAL) ok = ok && (kb * 32 + 8 * qd + e <= last_rel);
+      s[4 * qd + e] = ok ? s[4 * qd + e] : kNegInf;
     }
+  }
+}
+template <bool SEG, bool CAUSAL>
+CT_DEVICE void mask_scores_t(lds_addr segk, int seg_q_or_never, int last_rel, f32x16* s) {
+  mask_block_t<SEG, CAUSAL>(segk, seg_q_or_never, last_rel, 0, s[0]);
+  mask_block_t<SEG, CAUSAL>(segk, seg_q_or_never, last_rel, 1, s[1]);
 }
 
 // acc (D x 32 queries, transposed) += X^T W^T where X is a 64-row LDS tile read
@@ -316,6 +319,30 @@ CT_DEVICE void qk_sequence_128(const RowFragOffsets<16>& ro, const bf16x8* qf, f
                : "v"(ro.ptr[0]), "v"(ro.ptr[1]), "v"(ro.ptr[2]), "v"(ro.ptr[3]), "v"(ro.ptr[4]),
                  "v"(ro.ptr[5]), "v"(ro.ptr[6]), "v"(ro.ptr[7]), "v"(qf[0]), "v"(qf[1]), "v"(qf[2]),
                  "v"(qf[3]), "v"(qf[4]), "v"(qf[5]), "v"(qf[6]), "v"(qf[7]), "i"(TILE_OFF)
+               : "memory", CT_ATTN_ASM_SCRATCH);
+}
+
+// dQ kernel, one 32-key half of a key tile (see gen_attn_asm.py): S^T and dP^T of the half, and
+// the half's contribution to dQ^T. K_OFF / V_OFF are the byte offsets of the half's K and V rows.
+template <int K_OFF, int V_OFF>
+CT_DEVICE void dq_sdp_half_128(const RowFragOffsets<16>& ro, const bf16x8* qf, const bf16x8* dof, f32x16& s,
+                               f32x16& dp) {
+  asm volatile(CT_DQ_SDP_HALF_SEQUENCE
+               : "=&v"(s), "=&v"(dp)
+               : "v"(ro.ptr[0]), "v"(ro.ptr[1]), "v"(ro.ptr[2]), "v"(ro.ptr[3]), "v"(ro.ptr[4]),
+                 "v"(ro.ptr[5]), "v"(ro.ptr[6]), "v"(ro.ptr[7]), "v"(qf[0]), "v"(qf[1]), "v"(qf[2]),
+                 "v"(qf[3]), "v"(qf[4]), "v"(qf[5]), "v"(qf[6]), "v"(qf[7]), "v"(dof[0]), "v"(dof[1]),
+                 "v"(dof[2]), "v"(dof[3]), "v"(dof[4]), "v"(dof[5]), "v"(dof[6]), "v"(dof[7]), "i"(K_OFF),
+                 "i"(V_OFF)
+               : "memory", CT_ATTN_ASM_SCRATCH);
+}
+template <int K_OFF>
+CT_DEVICE void dq_acc_half_128(const TrFragOffsets<16, KSlots::kAccum>& to, bf16x8 p0, bf16x8 p1, f32x16* acc) {
+  asm volatile(CT_DQ_ACC_HALF_SEQUENCE
+               : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])
+               : "v"(to.ptr[0][0]), "v"(to.ptr[0][1]), "v"(to.ptr[0][2]), "v"(to.ptr[0][3]),
+                 "v"(to.ptr[1][0]), "v"(to.ptr[1][1]), "v"(to.ptr[1][2]), "v"(to.ptr[1][3]), "v"(p0), "v"(p1),
+                 "i"(K_OFF)
                : "memory", CT_ATTN_ASM_SCRATCH);
 }
 

@@ -179,6 +179,70 @@ def dkv_acc_sequence(ahead=DKV_SLOTS, slots=DKV_SLOTS):
     return lines + DKV_TAIL
 
 
+# (Dropping the issue priority for these sequences, as the dK/dV ones do, measured neutral here.)
+DQ_HEAD = ["s_waitcnt lgkmcnt(0)"]
+DQ_TAIL = TAIL
+
+
+def dq_sdp_half_sequence(ahead=4, slots=4):
+    """dQ kernel, one 32-key half of a key tile: S^T = K_half Q^T and dP^T = V_half dO^T, the two
+    chains alternating (16 MFMAs, one ds_read_b128 fragment each, read `ahead` fragments in front).
+
+    operands: %0 S^T, %1 dP^T (written), %2-%9 row-fragment pointers (k-step), %10-%17 Q fragments,
+    %18-%25 dO fragments, %26 byte offset of the half's K rows, %27 that of its V rows.
+    """
+    n = 16
+    lines = list(DQ_HEAD)
+
+    def load(i):
+        ks, which = divmod(i, 2)
+        lo, hi = slot_regs(i % slots)
+        return ["ds_read_b128 v[%d:%d], %%%d offset:%%%d" % (lo, hi, 2 + ks, 26 + which)]
+
+    for i in range(min(ahead, n)):
+        lines += load(i)
+    for i in range(n):
+        later = min(ahead - 1, n - 1 - i)
+        lines.append("s_waitcnt lgkmcnt(%d)" % later)
+        ks, which = divmod(i, 2)
+        lo, hi = slot_regs(i % slots)
+        src_c = "0" if ks == 0 else "%%%d" % which
+        lines.append("v_mfma_f32_32x32x16_bf16 %%%d, v[%d:%d], %%%d, %s" % (which, lo, hi, (18 if which else 10) + ks, src_c))
+        if i + ahead < n:
+            lines += load(i + ahead)
+    return lines + DQ_TAIL
+
+
+def dq_acc_half_sequence(ahead=4, slots=4):
+    """dQ kernel, one 32-key half: dQ^T[db] += K_half^T frag(step, db) * dS^T[step], 8 MFMAs, each
+    fragment = 2 ds_read_b64_tr_b16.
+
+    operands: %0-%3 accumulators, %4-%7 lo pointers (column block db), %8-%11 hi pointers,
+    %12-%13 dS fragments (k-step), %14 byte offset of the half's K rows.
+    """
+    n = 8
+    lines = list(DQ_HEAD)
+
+    def load(i):
+        step, db = divmod(i, 4)
+        lo, _ = slot_regs(i % slots)
+        off = "%%14+%d" % (step * 4096)
+        return ["ds_read_b64_tr_b16 v[%d:%d], %%%d offset:%s" % (lo, lo + 1, 4 + db, off),
+                "ds_read_b64_tr_b16 v[%d:%d], %%%d offset:%s" % (lo + 2, lo + 3, 8 + db, off)]
+
+    for i in range(min(ahead, n)):
+        lines += load(i)
+    for i in range(n):
+        later = min(ahead - 1, n - 1 - i)
+        lines.append("s_waitcnt lgkmcnt(%d)" % (2 * later))
+        step, db = divmod(i, 4)
+        lo, hi = slot_regs(i % slots)
+        lines.append("v_mfma_f32_32x32x16_bf16 %%%d, v[%d:%d], %%%d, %%%d" % (db, lo, hi, 12 + step, db))
+        if i + ahead < n:
+            lines += load(i + ahead)
+    return lines + DQ_TAIL
+
+
 def clobbers():
     regs = ", ".join('"v%d"' % r for r in range(SCRATCH0, SCRATCH0 + 16))
     dkv = ", ".join('"v%d"' % r for r in range(DKV_SCRATCH0, 256))
@@ -189,6 +253,8 @@ if __name__ == "__main__":
     print("// Generated by gen_attn_asm.py -- do not edit by hand.")
     print(emit(pv_sequence(4, 4), "CT_ATTN_PV_SEQUENCE"))
     print(emit(qk_sequence(4, 4), "CT_ATTN_QK_SEQUENCE"))
+    print(emit(dq_sdp_half_sequence(), "CT_DQ_SDP_HALF_SEQUENCE"))
+    print(emit(dq_acc_half_sequence(), "CT_DQ_ACC_HALF_SEQUENCE"))
     print(emit(dkv_sdp_sequence(), "CT_DKV_SDP_SEQUENCE"))
     print(emit(dkv_acc_sequence(), "CT_DKV_ACC_SEQUENCE"))
     print(clobbers())
