@@ -194,6 +194,25 @@ def bench_attention(ct, torch, steps, warmup, preamble_steps):
     }
 
 
+def bench_dkv_wide(ct, torch, config, attention, steps, warmup):
+    """The same step with the other dK/dV kernel (one wavefront of 64 keys per SIMD), for the
+    record: the headline above uses the default kernel."""
+
+    ct.set_dkv_variant(1)
+    try:
+        step, _, _ = attention_step_for(ct, config, attention["inputs"])
+        elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
+    finally:
+        ct.set_dkv_variant(0)
+    ms_per_step = elapsed / steps * 1e3
+    return {
+        "note": "ct_attn_set_dkv_variant(1); not the headline",
+        "ms_per_step": ms_per_step,
+        "tflops": attention["flops"]["total"] / (ms_per_step * 1e-3) / 1e12,
+        "attn_dkv_kernel_ms": mean(kernels.get("attn_dkv_kernel", [0.0])),
+    }
+
+
 SHAPE_LABELS = {
     "packed_small": "C1 packed causal B=2 S=1024 Hq=Hkv=8 D=64, documents U[32,512]",
     "maskgit": "C4 MaskGIT hybrid mask B=2 S=8192 Hq=Hkv=16 D=128, 1-3 bidirectional 32x33 image blocks per segment",
@@ -493,6 +512,7 @@ def main():
         },
         "kernels": attention["kernels"],
     }
+    result["dkv_wide_variant"] = bench_dkv_wide(ct, torch, config, attention, min(args.steps, 50), min(args.warmup, 10))
     result["delta_pass"] = bench_delta_pass(ct, torch, config, attention["inputs"]["q"])
     if args.calibration_copy_bytes:
         calibration_copy(ct, torch, args.calibration_copy_bytes)

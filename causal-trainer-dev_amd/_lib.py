@@ -134,6 +134,7 @@ SYMBOLS = {
     "ct_attn_fwd": (c_int32, [c_void_p, POINTER(AttnFwdArgs)]),
     "ct_attn_bwd": (c_int32, [c_void_p, POINTER(AttnBwdArgs)]),
     "ct_attn_delta": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32]),
+    "ct_attn_set_dkv_variant": (c_int32, [c_int32]),
     "ct_cutce_fwd_workspace_bytes": (c_size_t, [POINTER(CutceShape)]),
     "ct_cutce_bwd_workspace_min_bytes": (c_size_t, [POINTER(CutceShape)]),
     "ct_cutce_bwd_workspace_bytes": (c_size_t, [POINTER(CutceShape)]),

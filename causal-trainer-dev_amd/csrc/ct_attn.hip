@@ -1,5 +1,8 @@
 // C ABI of the attention hot path: argument validation and launches.
+#include <atomic>
+
 #include "ct_attn_bwd_kernels.cuh"
+#include "ct_attn_dkv_wide.cuh"
 #include "ct_attn_kernels.cuh"
 #include "ct_error.h"
 
@@ -343,6 +346,10 @@ static int launch_dq(hipStream_t stream, const AttnParams& p) {
   return scope2.done();
 }
 
+// Which dK/dV kernel runs for head dimension 128: 0 the two-wavefronts-per-SIMD one, 1 the wide
+// one (ct_attn_dkv_wide.cuh). Process-wide, set by ct_attn_set_dkv_variant.
+static std::atomic<int> g_dkv_variant{0};
+
 template <int D>
 static int launch_dkv(hipStream_t stream, const AttnParams& p) {
   const size_t smem = QdoStage<D>::kTotalBytes;
@@ -353,9 +360,24 @@ static int launch_dkv(hipStream_t stream, const AttnParams& p) {
   }
   int rc = 0;
   const int grid = p.dkv_max_entries * p.Hkv;  // entries beyond the list's length exit at once
-  LaunchScope scope3("attn_dkv_kernel", stream);
-  hipLaunchKernelGGL((attn_dkv_kernel<D>), dim3(grid), dim3(256), smem, stream, p);
-  rc = scope3.done();
+  bool wide = false;
+  if constexpr (D == 128) wide = g_dkv_variant.load(std::memory_order_relaxed) == 1;
+  if (wide) {
+    static std::atomic<bool> wide_ready{false};
+    if (!wide_ready.load()) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dkv_wide_kernel),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)DkvWideLds::kTotalBytes);
+      if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
+      wide_ready.store(true);
+    }
+    LaunchScope scope3("attn_dkv_kernel", stream);
+    hipLaunchKernelGGL(attn_dkv_wide_kernel, dim3(grid), dim3(128), DkvWideLds::kTotalBytes, stream, p);
+    rc = scope3.done();
+  } else {
+    LaunchScope scope3("attn_dkv_kernel", stream);
+    hipLaunchKernelGGL((attn_dkv_kernel<D>), dim3(grid), dim3(256), smem, stream, p);
+    rc = scope3.done();
+  }
   if (rc) return rc;
   LaunchScope scope9("attn_dkv_reduce_kernel", stream);
   hipLaunchKernelGGL((attn_dkv_reduce_kernel<D>), dim3(grid), dim3(256), 4 * 32 * D * 2, stream, p);
@@ -395,6 +417,12 @@ static int dispatch_bwd(hipStream_t stream, const AttnParams& p) {
 }  // namespace ct
 
 using namespace ct;
+
+extern "C" int32_t ct_attn_set_dkv_variant(int32_t variant) {
+  if (variant != 0 && variant != 1) return fail(CT_INVALID_ARGUMENT, "ct_attn_set_dkv_variant: variant must be 0 or 1");
+  g_dkv_variant.store(variant, std::memory_order_relaxed);
+  return CT_OK;
+}
 
 extern "C" size_t ct_attn_meta_bytes(int32_t batch, int32_t seq) {
   if (batch <= 0 || seq <= 0) return 0;

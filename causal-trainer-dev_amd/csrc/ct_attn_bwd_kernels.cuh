@@ -95,8 +95,10 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
   }
   const float delta_q = pair_sum(delta_part);
   if (ctx.active && half == 0) {
-    p.delta[stat_t] = delta_q;
-    p.lse2[stat_t] = lse2;
+    // for the dK/dV kernel: the values it adds to its S and dP blocks, P = exp2((S - lse / scale) *
+    // scale * log2(e)) and dS = P (dP - delta)
+    p.delta[stat_t] = -delta_q;
+    p.lse2[stat_t] = -p.lse[ctx.stat_off] / p.scale;
   }
 
   auto step = [&](auto stage_tag) {
@@ -700,9 +702,9 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = 4 * qd + e;
-          const float pr = exp2_fast(fmaf(s[r], scale_log2e, -lse4[e]));
+          const float pr = exp2_fast((s[r] + lse4[e]) * scale_log2e);  // lse4 = -lse / scale
           prob[r] = pr;
-          dp[r] = pr * (dp[r] - del4[e]);
+          dp[r] = pr * (dp[r] + del4[e]);                              // del4 = -delta
         }
       }
       if constexpr (D == 128) {

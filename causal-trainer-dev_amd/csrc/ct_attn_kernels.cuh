@@ -45,7 +45,7 @@ struct AttnParams {
   float* lse;
   const bf16* dout;
   float* delta;     // backward: rowsum(out * dout), head-major [B, Hq, S] (written by dQ, read by dK/dV)
-  float* lse2;      // backward: lse * log2(e), head-major [B, Hq, S] (written by dQ, read by dK/dV)
+  float* lse2;      // backward: -lse / scale, head-major [B, Hq, S] (written by dQ, read by dK/dV)
   bf16* dq;
   bf16* dk;
   bf16* dv;

@@ -10,6 +10,8 @@ starts with lgkmcnt(0)).
 Run ``python gen_attn_asm.py > ct_attn_asm.inc`` after editing; the output is committed.
 """
 
+import os
+
 SCRATCH0 = 240
 # The compiler cannot see the MFMAs inside an asm statement, so it will not insert the wait
 # states that a vector ALU read of a fresh MFMA result needs; the sequences end with them.
@@ -243,10 +245,211 @@ def dq_acc_half_sequence(ahead=4, slots=4):
     return lines + DQ_TAIL
 
 
+# ---------------------------------------------------------------------------
+# dK/dV, wide form: one wavefront per SIMD owns 64 keys (two 32-key blocks) and runs a whole
+# (head, query block) step as one instruction stream. With nothing else resident on the SIMD the
+# wavefront's exponent / dS arithmetic has to sit between its own MFMAs: the arithmetic of key
+# block 0 is placed under the S / dP MFMAs of key block 1, that of key block 1 under the dV / dK
+# MFMAs of key block 0.
+#
+# Fixed registers (declared as clobbers): a ring of 5 fragment slots, the score / dP blocks of
+# both key blocks (their first 8 registers later hold the bf16 P and dS fragments) and the 16
+# lse2 / delta values of this lane's query rows.
+# ---------------------------------------------------------------------------
+W_RING0, W_SLOTS = 236, 5
+W_S = (172, 204)      # S^T accumulators of key block 0 / 1 (16 registers each)
+W_DP = (188, 220)     # dP accumulators
+W_ADDR = 171          # address of a V fragment
+W_FIRST = 171
+
+
+class Stream:
+    """Instruction list with in-order tracking of the LDS reads in flight (lgkmcnt)."""
+
+    def __init__(self):
+        self.lines = ["s_waitcnt lgkmcnt(0)"]
+        self.pending = []
+
+    def lds(self, text, tag):
+        self.lines.append(text)
+        self.pending.append(tag)
+        assert len(self.pending) <= 15, "lgkmcnt holds at most 15"
+
+    def wait(self, tag):
+        if tag not in self.pending:
+            return
+        i = len(self.pending) - 1 - self.pending[::-1].index(tag)
+        self.lines.append("s_waitcnt lgkmcnt(%d)" % (len(self.pending) - 1 - i))
+        self.pending = self.pending[i + 1:]
+
+    def emit(self, text):
+        self.lines.append(text)
+
+
+def w_acc(i):
+    """Accumulator i of the wide kernel: 0-3 dV of key block 0 (column block db), 4-7 dV of key
+    block 1, 8-11 dK of key block 0, 12-15 dK of key block 1. They live in fixed accumulation
+    registers for the whole kernel and are never handed to the compiler."""
+    return "a[%d:%d]" % (16 * i, 16 * i + 15)
+
+
+def dkvw_fast_sequence(masked=False):
+    """One (head, query block) step for both key blocks.
+
+    operands: %0-%7 K fragments of key block 0 (k-step), %8-%15 of key block 1; %16-%23
+    row-fragment pointers (k-step); %24-%27 lo and %28-%31 hi pointers of the transposed
+    fragments (column block); %32 pointer of this lane's statistics (LDS base + 16 * (lane /
+    32)); %33 scale * log2(e) (scalar); %34 byte offset of this wavefront's V rows (scalar; key
+    block 1: 8192 later); %35 byte offset of the stage (Q tile, dO tile 8192 later, -lse / scale
+    at 16384, -delta at 16512).
+
+    The copies of the next item (its Q and dO rows and statistics, into the other stage) are
+    issued from inside the stream, one behind each of the first ten MFMAs: %36-%39 this thread's
+    four source offsets of a 32 x 128 tile; %40, %41 the Q and dO rows (scalar pairs); %42, %43 the
+    two statistics arrays this wavefront fetches; %44 LDS address of this wavefront's first slot of
+    the other stage's Q tile; %45 LDS address of its first statistics array there; %46 16 * lane.
+
+    The S blocks start from -lse / scale of their query rows (read from the stage) and the dP
+    blocks from -delta. With `masked`, the starting values of the two S blocks come in registers
+    instead (%47, %48): the caller has put -inf where a pair is not allowed, and the sum, the
+    probability and dS of such a pair are then -inf, 0 and 0 without any instruction here knowing
+    about masks.
+    """
+    st = Stream()
+
+    def stats(kb):
+        # The S and dP blocks start from the per-row terms instead of 0: -lse / scale and -delta of
+        # the block's 16 query rows (4 consecutive rows per read, the accumulator's own order).
+        for qd in range(0 if masked else 4):
+            st.lds("ds_read_b128 v[%d:%d], %%32 offset:%%35+%d" % (W_S[kb] + 4 * qd, W_S[kb] + 4 * qd + 3, 16384 + 32 * qd),
+                   "stat%d" % kb)
+        for qd in range(4):
+            st.lds("ds_read_b128 v[%d:%d], %%32 offset:%%35+%d" % (W_DP[kb] + 4 * qd, W_DP[kb] + 4 * qd + 3, 16512 + 32 * qd),
+                   "stat%d" % kb)
+
+    stats(0)
+
+    def acc16(base):
+        return "v[%d:%d]" % (base, base + 15)
+
+    def slot(r):
+        lo = W_RING0 + 4 * (r % W_SLOTS)
+        return lo, "v[%d:%d]" % (lo, lo + 3)
+
+    # ---- the reads (in issue order) and the MFMAs (in issue order, each naming the reads it needs)
+    reads, mfmas = [], []
+    for kb in range(2):
+        for ks in range(8):
+            base = len(reads)
+            reads.append(["ds_read_b128 {v4}, %%%d offset:%%35" % (16 + ks)])                      # Q
+            reads.append(["ds_read_b128 {v4}, %%%d offset:%%35+8192" % (16 + ks)])                 # dO
+            reads.append(["v_add_u32_e32 v%d, %%34, %%%d" % (W_ADDR, 16 + ks),                       # V
+                          "ds_read_b128 {v4}, v%d offset:%d" % (W_ADDR, 8192 * kb)])
+            c_s = "%%%d" % (47 + kb) if (masked and ks == 0) else acc16(W_S[kb])
+            mfmas.append(("v_mfma_f32_32x32x16_bf16 %s, {r0}, %%%d, %s" % (acc16(W_S[kb]), 8 * kb + ks, c_s), [base]))
+            mfmas.append(("v_mfma_f32_32x32x16_bf16 %s, {r0}, {r1}, %s" % (acc16(W_DP[kb]), acc16(W_DP[kb])), [base + 1, base + 2]))
+    for kb in range(2):
+        for step in range(2):
+            for db in range(4):
+                for which in range(2):  # 0: dV (P^T, dO), 1: dK (dS^T, Q)
+                    off = "%%35+%d" % (step * 4096 + (8192 if which == 0 else 0))
+                    reads.append(["ds_read_b64_tr_b16 {v2lo}, %%%d offset:%s" % (24 + db, off),
+                                  "ds_read_b64_tr_b16 {v2hi}, %%%d offset:%s" % (28 + db, off)])
+                    acc = w_acc((0 if which == 0 else 8) + 4 * kb + db)
+                    src = (W_S if which == 0 else W_DP)[kb] + 4 * step
+                    mfmas.append(("v_mfma_f32_32x32x16_bf16 %s, v[%d:%d], {r0}, %s" % (acc, src, src + 3, acc),
+                                  [len(reads) - 1]))
+    assert len(mfmas) == 64
+
+    # ---- the arithmetic, attached to MFMA slots. Element e of key block kb starts under MFMA
+    # 16 + 16 kb + 11 e / 8: elements 0-7 are packed before the block's first dV / dK MFMA (32 + 16
+    # kb) needs them, elements 8-15 before its ninth does, and no MFMA has much more than one
+    # element behind it.
+    fill = [[] for _ in range(len(mfmas) + 1)]
+    for kb in range(2):
+        S, DP = W_S[kb], W_DP[kb]
+        done = {}
+        for e in range(16):
+            t = 16 + 16 * kb + (11 * e) // 8
+            fill[t] += ["v_mul_f32_e32 v%d, %%33, v%d" % (S + e, S + e),
+                        "v_exp_f32_e32 v%d, v%d" % (S + e, S + e)]
+            # the dP block is first read two MFMAs later: its last MFMA has long retired by then
+            fill[t + 2] += ["v_mul_f32_e32 v%d, v%d, v%d" % (DP + e, S + e, DP + e)]
+            done[e] = t + 2
+            if e % 2 == 1:
+                k = e // 2
+                fill[t + 2] += ["v_cvt_pk_bf16_f32 v%d, v%d, v%d" % (S + k, S + 2 * k, S + 2 * k + 1),
+                                "v_cvt_pk_bf16_f32 v%d, v%d, v%d" % (DP + k, DP + 2 * k, DP + 2 * k + 1)]
+        assert done[7] < 32 + 16 * kb and done[15] < 40 + 16 * kb
+
+    # ---- emission: reads run ahead of their MFMAs as far as the ring allows
+    state = {"issued": 0}
+    consumed = [False] * len(reads)
+
+    def issue_reads():
+        while state["issued"] < len(reads):
+            r = state["issued"]
+            if r >= W_SLOTS and not consumed[r - W_SLOTS]:
+                break
+            lo, v4 = slot(r)
+            for text in reads[r]:
+                text = text.format(v4=v4, v2lo="v[%d:%d]" % (lo, lo + 1), v2hi="v[%d:%d]" % (lo + 2, lo + 3))
+                if text.startswith("ds_"):
+                    st.lds(text, r)
+                else:
+                    st.emit(text)
+            state["issued"] += 1
+
+    # the copies: (instructions in front of the MFMA, instructions behind it)
+    copies = []
+    for which in range(2):
+        for n in range(4):
+            copies.append((["s_add_u32 m0, %%44, %d" % (8192 * which + 2048 * n)],
+                           ["global_load_lds_dwordx4 %%%d, %%%d" % (36 + n, 40 + which)]))
+    copies.append((["s_mov_b32 m0, %45"],
+                   ["s_mov_b64 exec, 0xff", "global_load_lds_dwordx4 %46, %42", "s_mov_b64 exec, -1"]))
+    copies.append((["s_add_u32 m0, %45, 128"],
+                   ["s_mov_b64 exec, 0xff", "global_load_lds_dwordx4 %46, %43", "s_mov_b64 exec, -1"]))
+
+    issue_reads()
+    for i, (text, needs) in enumerate(mfmas):
+        st.wait(needs[-1])
+        if i < len(copies):
+            for line in copies[i][0]:
+                st.emit(line)
+        names = {"r%d" % n: slot(r)[1] for n, r in enumerate(needs)}
+        st.emit(text.format(**names))
+        if i < len(copies):
+            for line in copies[i][1]:
+                st.emit(line)
+        for r in needs:
+            consumed[r] = True
+        if i == 3:
+            stats(1)   # (the registers are free: their last readers were the previous step's MFMAs)
+        issue_reads()
+        for line in fill[i]:
+            if not os.environ.get("KO_FILL"):
+                st.emit(line)
+    assert not fill[64] and state["issued"] == len(reads)
+    return st.lines + TAIL
+
+
+def dkvw_zero():
+    return ["v_accvgpr_write_b32 a%d, 0" % r for r in range(256)]
+
+
+def dkvw_read():
+    """operands: %0-%15 the 16 values of one accumulator, %16 its first register number."""
+    return ["v_accvgpr_read_b32 %%%d, a[%%16+%d]" % (e, e) for e in range(16)]
+
+
 def clobbers():
     regs = ", ".join('"v%d"' % r for r in range(SCRATCH0, SCRATCH0 + 16))
     dkv = ", ".join('"v%d"' % r for r in range(DKV_SCRATCH0, 256))
-    return "#define CT_ATTN_ASM_SCRATCH %s\n\n#define CT_DKV_ASM_SCRATCH %s\n" % (regs, dkv)
+    wide = ", ".join('"v%d"' % r for r in range(W_FIRST, 256))
+    accs = ", ".join('"a%d"' % r for r in range(256))
+    return ("#define CT_ATTN_ASM_SCRATCH %s\n\n#define CT_DKV_ASM_SCRATCH %s\n\n#define CT_DKVW_ASM_SCRATCH %s\n\n"
+            "#define CT_DKVW_ACCUMULATORS %s\n" % (regs, dkv, wide, accs))
 
 
 if __name__ == "__main__":
@@ -257,4 +460,8 @@ if __name__ == "__main__":
     print(emit(dq_acc_half_sequence(), "CT_DQ_ACC_HALF_SEQUENCE"))
     print(emit(dkv_sdp_sequence(), "CT_DKV_SDP_SEQUENCE"))
     print(emit(dkv_acc_sequence(), "CT_DKV_ACC_SEQUENCE"))
+    print(emit(dkvw_fast_sequence(), "CT_DKVW_FAST_SEQUENCE"))
+    print(emit(dkvw_fast_sequence(masked=True), "CT_DKVW_MASKED_SEQUENCE"))
+    print(emit(dkvw_zero(), "CT_DKVW_ZERO"))
+    print(emit(dkvw_read(), "CT_DKVW_READ"))
     print(clobbers())

@@ -280,6 +280,13 @@ def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=Non
     return _attn_backward(query, key, value, metadata, out, lse, dout.contiguous(), resolved, with_delta)
 
 
+def set_dkv_variant(variant: int) -> None:
+    """Choose the dK/dV kernel of the backward for head dimension 128, process-wide: 0 the default
+    (two wavefronts per SIMD), 1 the wide one (one wavefront per SIMD, 64 keys)."""
+
+    _lib.check(_lib.load().ct_attn_set_dkv_variant(int(variant)))
+
+
 __all__ = [
     "AttentionKernelProfile",
     "AttentionMetadata",
@@ -289,6 +296,7 @@ __all__ = [
     "efficient_attention",
     "prepare_attention_metadata",
     "resolve_attention_profile",
+    "set_dkv_variant",
     "tile_bounds_table",
     "validate_attention_profile",
 ]

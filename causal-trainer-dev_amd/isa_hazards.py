@@ -107,6 +107,44 @@ def scan(assembly: str) -> list[str]:
     return problems
 
 
+def private_accumulators(assembly: str, kernel: str) -> list[str]:
+    """Checks a kernel that keeps values in accumulation registers across inline-assembly
+    statements without telling the compiler (attn_dkv_wide_kernel): outside those statements the
+    compiler must not touch an accumulation register (it would, to park a spilled vector register
+    there), and no spilled register may be reloaded between the kernel's first and last workgroup
+    barrier, i.e. inside its item loop, where the wait for the reload also waits for every
+    asynchronous copy in flight."""
+
+    problems, inside, in_asm, found = [], False, False, False
+    reloads, barriers = [], []
+    for number, line in enumerate(assembly.splitlines(), 1):
+        text = line.strip()
+        label = re.match(r"([A-Za-z_][\w$]*):", text)
+        if label:
+            inside = kernel in label.group(1)
+            found = found or inside
+            continue
+        if not inside:
+            continue
+        if "#ASMSTART" in text:
+            in_asm = True
+        elif "#ASMEND" in text:
+            in_asm = False
+        elif not in_asm and not text.startswith((";", ".")):
+            if re.search(r"\ba\[?\d", text) or "accvgpr" in text:
+                problems.append(f"{kernel}: line {number} '{text}' uses an accumulation register outside the assembly statements")
+            if text.startswith("scratch_load"):
+                reloads.append((number, text))
+            if text.startswith("s_barrier"):
+                barriers.append(number)
+    for number, text in reloads:
+        if barriers and barriers[0] < number < barriers[-1]:
+            problems.append(f"{kernel}: line {number} '{text}' reloads a spilled register inside the item loop")
+    if not found:
+        problems.append(f"{kernel}: not found in the assembly")
+    return problems
+
+
 def device_assembly(source: Path, flags) -> str:
     from . import build as recipe
 
@@ -128,7 +166,11 @@ def scan_library() -> dict[str, list[str]]:
     sources = [recipe.CSRC / name for name in recipe.SOURCES]
     with ThreadPoolExecutor(max_workers=4) as pool:
         texts = list(pool.map(lambda path: device_assembly(path, recipe.HIP_FLAGS), sources))
-    return {path.name: scan(text) for path, text in zip(sources, texts)}
+    findings = {path.name: scan(text) for path, text in zip(sources, texts)}
+    for path, text in zip(sources, texts):
+        if path.name == "ct_attn.hip":
+            findings[path.name] += private_accumulators(text, "attn_dkv_wide_kernel")
+    return findings
 
 
 if __name__ == "__main__":

@@ -95,9 +95,19 @@ CASES = [
 ]
 
 
+@pytest.fixture(params=[0, 1], ids=["dkv32", "dkv64"])
+def dkv_variant(request, ct):
+    """Both dK/dV kernels of the backward: two wavefronts of 32 keys per SIMD (the default) and
+    one wavefront of 64 keys (head dimension 128 only; other dimensions run the default)."""
+
+    ct.set_dkv_variant(request.param)
+    yield request.param
+    ct.set_dkv_variant(0)
+
+
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_S%d_Hq%d_Hkv%d_D%d_%s%s" % (
     c[0], c[1], c[2], c[3], c[4], "holes" if c[5] else "packed", "_ends" if c[6] else ""))
-def test_forward_backward_match_oracle(ct, gpu, case):
+def test_forward_backward_match_oracle(ct, gpu, case, dkv_variant):
     batch, seq, q_heads, kv_heads, dim, holes, with_ends = case
     rng = np.random.default_rng(hash(case) % (2 ** 31))
     ids = _layout(rng, batch, seq, holes=holes)
@@ -112,7 +122,7 @@ def test_forward_backward_match_oracle(ct, gpu, case):
     _check_against_oracle(results, q, k, v, dout, ids, ends, scale)
 
 
-def test_edge_layouts(ct, gpu):
+def test_edge_layouts(ct, gpu, dkv_variant):
     rng = np.random.default_rng(11)
     batch, seq, q_heads, kv_heads, dim = 4, 256, 4, 2, 128
     ids = np.zeros((batch, seq), np.int32)
@@ -149,7 +159,7 @@ def test_reference_seeded_fixture(ct, gpu):
         assert (grad[:, ids[0] != 2] == 0).all()
 
 
-def test_neighbour_perturbation_leaves_other_segment_bitwise_unchanged(ct, gpu):
+def test_neighbour_perturbation_leaves_other_segment_bitwise_unchanged(ct, gpu, dkv_variant):
     # reference: tests/kernels/test_efficient_attention_tpu.py:395-424
     rng = np.random.default_rng(21)
     batch, seq, q_heads, kv_heads, dim = 1, 512, 4, 2, 128
@@ -170,7 +180,7 @@ def test_neighbour_perturbation_leaves_other_segment_bitwise_unchanged(ct, gpu):
         assert torch.equal(a, b)        # fixed summation order: bitwise reproducible
 
 
-def test_zero_cross_segment_mass(ct, gpu):
+def test_zero_cross_segment_mass(ct, gpu, dkv_variant):
     # V carries a one-hot of the key's segment id: any attention mass that leaks to another
     # segment shows up as a nonzero in a column that must be exactly 0.
     rng = np.random.default_rng(31)
@@ -296,8 +306,9 @@ def test_delta_pass_matches_torch(ct, gpu):
 
 
 def test_backward_leaves_delta_and_matches_the_pass_on_its_own(ct, gpu):
-    """The backward forms delta = rowsum(out * dout) inside its dQ kernel (head-major scratch);
-    it has to agree with the closed form on every row, padding rows and hybrid ends included."""
+    """The backward forms delta = rowsum(out * dout) inside its dQ kernel and leaves -delta in its
+    head-major scratch (the dK/dV kernel adds it to its dP blocks); it has to agree with the closed
+    form on every row, padding rows and hybrid ends included."""
 
     rng = np.random.default_rng(67)
     for (batch, seq, hq, hkv, dim, hybrid) in ((2, 256, 4, 1, 128, False), (1, 384, 8, 2, 64, True),
@@ -316,10 +327,10 @@ def test_backward_leaves_delta_and_matches_the_pass_on_its_own(ct, gpu):
         out, lse = ct.attention_forward_with_lse(qd, kd, vd, metadata, scale=dim ** -0.5)
         *_, delta = ct.attention_backward(qd, kd, vd, metadata, out, lse, dod, scale=dim ** -0.5, with_delta=True)
         expected = (out.float() * dod.float()).sum(-1).permute(0, 2, 1)  # [B, Hq, S]
-        torch.testing.assert_close(delta, expected, atol=1e-4, rtol=1e-5)
+        torch.testing.assert_close(-delta, expected, atol=1e-4, rtol=1e-5)
 
 
-def test_split_key_tiles_match_oracle(ct, gpu):
+def test_split_key_tiles_match_oracle(ct, gpu, dkv_variant):
     """One 2048-position segment, one KV head, a small batch: the dK/dV work list is far below
     one compute slot's share, so the chunk target sits at its minimum and the key tiles with the
     longest query lists are split into several chunks whose f32 partial sums the reduce kernel
@@ -491,7 +502,7 @@ def _self_contained_window(ids_row, limit):
 
 
 @pytest.mark.parametrize("name", ["packed_small", "llama3_8b", "maskgit", "long_70b"])
-def test_benchmark_shapes(ct, gpu, name):
+def test_benchmark_shapes(ct, gpu, name, dkv_variant):
     """Full benchmark shapes: size-independent properties everywhere, and the oracle on a
     self-contained window (whole segments) of one KV head with its query group."""
 

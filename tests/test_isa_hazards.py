@@ -50,6 +50,29 @@ kernel_e:
     assert isa_hazards.scan(wide.replace("dwordx4 v252, v[2:5]", "dwordx2 v252, v[2:3]")) == []
 
 
+def test_private_accumulator_check(ct):
+    from causal_trainer_dev_amd import isa_hazards
+
+    clean = """
+_ZN2ct20attn_dkv_wide_kernelENS_10AttnParamsE:
+	v_add_u32_e32 v1, v2, v3
+	;;#ASMSTART
+	v_mfma_f32_32x32x16_bf16 a[0:15], v[4:7], v[8:11], a[0:15]
+	;;#ASMEND
+	s_endpgm
+other_kernel:
+	v_accvgpr_write_b32 a0, v1
+"""
+    assert isa_hazards.private_accumulators(clean, "attn_dkv_wide_kernel") == []
+    parked = clean.replace("\tv_add_u32_e32 v1, v2, v3", "\tv_accvgpr_write_b32 a3, v1")
+    assert len(isa_hazards.private_accumulators(parked, "attn_dkv_wide_kernel")) == 1
+    spilled = clean.replace("\tv_add_u32_e32 v1, v2, v3", "\ts_barrier\n\tscratch_load_dword v1, off, off\n\ts_barrier")
+    assert len(isa_hazards.private_accumulators(spilled, "attn_dkv_wide_kernel")) == 1
+    outside = clean.replace("\tv_add_u32_e32 v1, v2, v3", "\ts_barrier\n\ts_barrier\n\tscratch_load_dword v1, off, off")
+    assert isa_hazards.private_accumulators(outside, "attn_dkv_wide_kernel") == []
+    assert len(isa_hazards.private_accumulators(clean, "missing_kernel")) == 1
+
+
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
 def test_library_sources_have_no_scalar_base_hazard(ct):
     from causal_trainer_dev_amd import isa_hazards
