@@ -83,55 +83,69 @@ CT_DEVICE f32x16 dkvw_read_accumulator() {
   return out;
 }
 
-// What the stream needs to issue the copies of the next item (all scalar except the lane offsets).
+// What a stream needs to issue the copies of the next item, besides this thread's source offsets:
+// all wave-uniform.
 struct DkvWideCopies {
   const char* q;       // Q rows of the next item
   const char* dout;    // dO rows
   const char* stat0;   // the two statistics arrays this wavefront fetches
   const char* stat1;
-  unsigned tile_dst;   // LDS address of this wavefront's first slot of the other stage's Q tile
-  unsigned stat_dst;   // LDS address of its first statistics array in the other stage
 };
 
-#define CT_DKVW_COPY_OPERANDS                                                                          \
-  "v"(dma.lane_off[0]), "v"(dma.lane_off[1]), "v"(dma.lane_off[2]), "v"(dma.lane_off[3]), "s"(cp.q),    \
-      "s"(cp.dout), "s"(cp.stat0), "s"(cp.stat1), "s"(cp.tile_dst), "s"(cp.stat_dst), "v"(lane16)
+// Everything that stays the same from step to step.
+struct DkvWideFrame {
+  bf16x8 kf[2][8];                          // K fragments of the two key blocks
+  RowFragOffsets<16> rp;                    // row-fragment pointers
+  TrFragOffsets<16, KSlots::kAccum> tp;     // transposed-fragment pointers
+  lds_addr stat_ptr;                        // LDS base + 16 * (lane / 32)
+  float scale_log2e;
+  unsigned v_off;                           // byte offset of this wavefront's V rows
+  unsigned tile_base, stat_base;            // LDS addresses of this wavefront's copy slots at stage offset 0
+};
 
-template <int STAGE_OFF>
-CT_DEVICE void dkvw_fast_step(const bf16x8 (*kf)[8], const RowFragOffsets<16>& rp,
-                              const TrFragOffsets<16, KSlots::kAccum>& tp, lds_addr stat_ptr, float scale_log2e,
-                              unsigned v_off, const TileDma128& dma, const DkvWideCopies& cp, unsigned lane16) {
+#define CT_DKVW_FRAME_OPERANDS                                                                                   \
+  "v"(f.kf[0][0]), "v"(f.kf[0][1]), "v"(f.kf[0][2]), "v"(f.kf[0][3]), "v"(f.kf[0][4]), "v"(f.kf[0][5]),           \
+      "v"(f.kf[0][6]), "v"(f.kf[0][7]), "v"(f.kf[1][0]), "v"(f.kf[1][1]), "v"(f.kf[1][2]), "v"(f.kf[1][3]),       \
+      "v"(f.kf[1][4]), "v"(f.kf[1][5]), "v"(f.kf[1][6]), "v"(f.kf[1][7]), "v"(f.rp.ptr[0]), "v"(f.rp.ptr[1]),     \
+      "v"(f.rp.ptr[2]), "v"(f.rp.ptr[3]), "v"(f.rp.ptr[4]), "v"(f.rp.ptr[5]), "v"(f.rp.ptr[6]), "v"(f.rp.ptr[7]), \
+      "v"(f.tp.ptr[0][0]), "v"(f.tp.ptr[0][1]), "v"(f.tp.ptr[0][2]), "v"(f.tp.ptr[0][3]), "v"(f.tp.ptr[1][0]),    \
+      "v"(f.tp.ptr[1][1]), "v"(f.tp.ptr[1][2]), "v"(f.tp.ptr[1][3]), "v"(f.stat_ptr), "s"(f.scale_log2e),         \
+      "s"(f.v_off), "s"(cp.q), "s"(cp.dout), "s"(cp.stat0), "s"(cp.stat1), "s"(f.tile_base), "s"(f.stat_base)
+
+// One step whose pairs are all allowed. STAGE: byte offset of the stage that is read; the next item
+// is copied into the other one.
+template <int STAGE, int OTHER>
+CT_DEVICE void dkvw_fast_step(const DkvWideFrame& f, const DkvWideCopies& cp, const TileDma128& dma, unsigned lane16) {
   asm volatile(CT_DKVW_FAST_SEQUENCE
                :
-               : "v"(kf[0][0]), "v"(kf[0][1]), "v"(kf[0][2]), "v"(kf[0][3]), "v"(kf[0][4]), "v"(kf[0][5]),
-                 "v"(kf[0][6]), "v"(kf[0][7]), "v"(kf[1][0]), "v"(kf[1][1]), "v"(kf[1][2]), "v"(kf[1][3]),
-                 "v"(kf[1][4]), "v"(kf[1][5]), "v"(kf[1][6]), "v"(kf[1][7]),
-                 "v"(rp.ptr[0]), "v"(rp.ptr[1]), "v"(rp.ptr[2]), "v"(rp.ptr[3]), "v"(rp.ptr[4]), "v"(rp.ptr[5]),
-                 "v"(rp.ptr[6]), "v"(rp.ptr[7]),
-                 "v"(tp.ptr[0][0]), "v"(tp.ptr[0][1]), "v"(tp.ptr[0][2]), "v"(tp.ptr[0][3]),
-                 "v"(tp.ptr[1][0]), "v"(tp.ptr[1][1]), "v"(tp.ptr[1][2]), "v"(tp.ptr[1][3]),
-                 "v"(stat_ptr), "s"(scale_log2e), "s"(v_off), "i"(STAGE_OFF), CT_DKVW_COPY_OPERANDS
+               : CT_DKVW_FRAME_OPERANDS, "i"(STAGE), "i"(OTHER), "v"(dma.lane_off[0]), "v"(dma.lane_off[1]),
+                 "v"(dma.lane_off[2]), "v"(dma.lane_off[3]), "v"(lane16)
                : "memory", "m0", "scc", CT_DKVW_ASM_SCRATCH, CT_DKVW_ACCUMULATORS);
 }
 
 // The same step with the starting values of the two S blocks handed over in registers (-lse /
 // scale of the row where the pair is allowed, -inf where it is not).
-template <int STAGE_OFF>
-CT_DEVICE void dkvw_masked_step(const bf16x8 (*kf)[8], const RowFragOffsets<16>& rp,
-                                const TrFragOffsets<16, KSlots::kAccum>& tp, lds_addr stat_ptr, float scale_log2e,
-                                unsigned v_off, const TileDma128& dma, const DkvWideCopies& cp, unsigned lane16,
+template <int STAGE, int OTHER>
+CT_DEVICE void dkvw_masked_step(const DkvWideFrame& f, const DkvWideCopies& cp, const TileDma128& dma, unsigned lane16,
                                 const f32x16& s_init0, const f32x16& s_init1) {
   asm volatile(CT_DKVW_MASKED_SEQUENCE
                :
-               : "v"(kf[0][0]), "v"(kf[0][1]), "v"(kf[0][2]), "v"(kf[0][3]), "v"(kf[0][4]), "v"(kf[0][5]),
-                 "v"(kf[0][6]), "v"(kf[0][7]), "v"(kf[1][0]), "v"(kf[1][1]), "v"(kf[1][2]), "v"(kf[1][3]),
-                 "v"(kf[1][4]), "v"(kf[1][5]), "v"(kf[1][6]), "v"(kf[1][7]),
-                 "v"(rp.ptr[0]), "v"(rp.ptr[1]), "v"(rp.ptr[2]), "v"(rp.ptr[3]), "v"(rp.ptr[4]), "v"(rp.ptr[5]),
-                 "v"(rp.ptr[6]), "v"(rp.ptr[7]),
-                 "v"(tp.ptr[0][0]), "v"(tp.ptr[0][1]), "v"(tp.ptr[0][2]), "v"(tp.ptr[0][3]),
-                 "v"(tp.ptr[1][0]), "v"(tp.ptr[1][1]), "v"(tp.ptr[1][2]), "v"(tp.ptr[1][3]),
-                 "v"(stat_ptr), "s"(scale_log2e), "s"(v_off), "i"(STAGE_OFF), CT_DKVW_COPY_OPERANDS, "v"(s_init0),
-                 "v"(s_init1)
+               : CT_DKVW_FRAME_OPERANDS, "v"(s_init0), "v"(s_init1), "i"(STAGE), "i"(OTHER), "v"(dma.lane_off[0]),
+                 "v"(dma.lane_off[1]), "v"(dma.lane_off[2]), "v"(dma.lane_off[3]), "v"(lane16)
+               : "memory", "m0", "scc", CT_DKVW_ASM_SCRATCH, CT_DKVW_ACCUMULATORS);
+}
+
+// `steps` all-allowed steps over consecutive query blocks of one head, starting on STAGE, with the
+// copy waits and workgroup barriers between them inside the statement. `cp` names the rows of the
+// item after the first; every step moves one query block (`q_stride` bytes of Q / dO rows, 128
+// bytes of statistics) further.
+template <int STAGE, int OTHER>
+CT_DEVICE void dkvw_run(const DkvWideFrame& f, const DkvWideCopies& cp, const TileDma128& dma, unsigned lane16,
+                        unsigned steps, unsigned q_stride) {
+  unsigned o0 = dma.lane_off[0], o1 = dma.lane_off[1], o2 = dma.lane_off[2], o3 = dma.lane_off[3], l16 = lane16;
+  asm volatile(CT_DKVW_RUN_SEQUENCE
+               : "+s"(steps), "+v"(o0), "+v"(o1), "+v"(o2), "+v"(o3), "+v"(l16)
+               : CT_DKVW_FRAME_OPERANDS, "s"(q_stride), "i"(STAGE), "i"(OTHER)
                : "memory", "m0", "scc", CT_DKVW_ASM_SCRATCH, CT_DKVW_ACCUMULATORS);
 }
 
@@ -172,30 +186,29 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const bool has_end = p.end != nullptr;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
 
-  // pointers of the row fragments and transposed fragments (held for the whole kernel: a lone
-  // wavefront has the registers)
-  const RowFragOffsets<16> rp(lds0);
-  const TrFragOffsets<16, KSlots::kAccum> tp(lds0);
-  const unsigned v_off = DkvWideLds::kVResident + w * (64 * 256);  // this wavefront's V rows
-  const lds_addr stat_ptr = lds0 + 16 * half;
-
-  bf16x8 kf[2][8];
+  // Fragment pointers and K fragments are held for the whole kernel: a lone wavefront has the registers.
+  DkvWideFrame f;
+  f.rp = RowFragOffsets<16>(lds0);
+  f.tp = TrFragOffsets<16, KSlots::kAccum>(lds0);
+  f.v_off = DkvWideLds::kVResident + w * (64 * 256);  // this wavefront's V rows
+  f.stat_ptr = lds0 + 16 * half;
+  f.scale_log2e = p.scale * kLog2e;
+  f.tile_base = uniform((unsigned)(uintptr_t)lds0 + w * 1024);
+  f.stat_base = uniform((unsigned)(uintptr_t)lds0 + QdoStage<D>::kLse + w * 256);
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb) {
     const size_t kv_off = (((size_t)b * p.S + (rb0 + kb) * 32 + j) * p.Hkv + kvh) * D;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      kf[kb][ks] = as_bf16x8(load_global16(p.k + kv_off + 16 * ks + 8 * half));
-      lds_store<u32x4>(rp.ptr[ks] + v_off + kb * 8192, load_global16(p.v + kv_off + 16 * ks + 8 * half));
+      f.kf[kb][ks] = as_bf16x8(load_global16(p.k + kv_off + 16 * ks + 8 * half));
+      lds_store<u32x4>(f.rp.ptr[ks] + f.v_off + kb * 8192, load_global16(p.v + kv_off + 16 * ks + 8 * half));
     }
   }
   dkvw_zero_accumulators();
 #pragma unroll
   for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(kf[kb][ks]));
-
-  const float scale_log2e = p.scale * kLog2e;
+    for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+v"(f.kf[kb][ks]));
 
   const int nq = (q_lo <= q_hi) ? (q_hi - q_lo + 1) : 0;
   const int per_chunk = (nq * g + nsplit - 1) / nsplit;
@@ -207,16 +220,80 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     qb += it % nq;
   }
   const TileDma128 dma((size_t)p.Hq * D * 2);
+  const unsigned q_stride = (unsigned)(kQueryTile * p.Hq * D * 2);  // bytes between the rows of consecutive query blocks
   if (it < items) {
     qdo_fetch_wide(dma, p, b, head, qb, lds0);
     dma_wait_all();
   }
   __syncthreads();
 
+  // Rows an item's copies read: Q / dO rows and the two statistics arrays of this wavefront.
+  auto rows_of = [&](int h, int q_block) {
+    DkvWideCopies cp;
+    const size_t origin = (((size_t)b * p.S + q_block * kQueryTile) * p.Hq + h) * D;
+    const size_t head_major = ((size_t)b * p.Hq + h) * p.S + q_block * kQueryTile;
+    const size_t row_major = (size_t)b * p.S + q_block * kQueryTile;
+    cp.q = reinterpret_cast<const char*>(p.q + origin);
+    cp.dout = reinterpret_cast<const char*>(p.dout + origin);
+    cp.stat0 = w == 0 ? reinterpret_cast<const char*>(p.lse2 + head_major) : reinterpret_cast<const char*>(p.seg + row_major);
+    cp.stat1 = w == 0 ? reinterpret_cast<const char*>(p.delta + head_major)
+                      : reinterpret_cast<const char*>(has_end ? p.end + row_major : p.seg + row_major);
+    return cp;
+  };
+  auto all_allowed = [&](const QueryBlockBounds& q) {
+    bool yes = true;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+      yes = yes && blocks_interact(q.min_nz, q.max_id, q.end_max, my_min[kb], my_max[kb], (rb0 + kb) * 32) &&
+            tile_is_interior(q.uniform, q.end_min, my_uni[kb], (rb0 + kb) * 32 + 31);
+    return yes;
+  };
+  // Number of consecutive query blocks from `first` on (at most 64, not beyond q_hi) whose steps
+  // are all-allowed for this wavefront: lane i looks at block first + i. The answer depends on the
+  // keys and the query block only, so it is remembered for the other heads of the group.
+  int run_first = -1, run_length = 0;
+  auto allowed_run = [&](int first) {
+    if (first == run_first) return run_length;
+    const int mine = first + lane_id_here();
+    bool yes = false;
+    if (mine <= q_hi) {
+      const int* m = meta_b + (size_t)mine * kMetaW;
+      QueryBlockBounds q;
+      q.min_nz = m[kMinNz];
+      q.max_id = m[kMaxId];
+      q.uniform = m[kUniform];
+      q.end_min = m[kEndMin];
+      q.end_max = m[kEndMax];
+      yes = all_allowed(q);
+    }
+    const unsigned long long stops = ~__ballot(yes);
+    run_first = first;
+    run_length = stops == 0 ? 64 : uniform(__builtin_ctzll(stops));
+    return run_length;
+  };
+
   QueryBlockBounds qb_bounds = query_block_bounds(meta_b, min(qb, nrb - 1));
   auto step = [&](auto stage_tag) {
     constexpr int CUR = decltype(stage_tag)::value;
-    const lds_addr stage = lds0 + CUR * kStage;
+    constexpr int kThis = CUR * kStage, kOther = (CUR ^ 1) * kStage;
+    const lds_addr stage = lds0 + kThis;
+    const unsigned lane16 = (unsigned)lane_id_here() * 16;
+
+    // A run of all-allowed steps within this head and chunk goes through one statement that loops
+    // by itself; an even number of steps, so that the stages are back where this step expects
+    // them, and the run's last block is left to the single step below (it copies whatever item
+    // comes next, which need not be the next query block).
+    if (all_allowed(qb_bounds)) {
+      const int within = min(min(allowed_run(qb), q_hi - qb + 1), items - it);
+      const int steps = (within - 1) & ~1;
+      if (steps >= 2) {
+        dkvw_run<kThis, kOther>(f, rows_of(head, qb + 1), dma, lane16, (unsigned)steps, q_stride);
+        it += steps;
+        qb += steps;
+        qb_bounds = query_block_bounds(meta_b, qb);
+      }
+    }
+
     const bool more = it + 1 < items;
     int qb_next = qb + 1, head_next = head;
     if (qb_next > q_hi) {
@@ -226,33 +303,17 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // The streams below issue the copies of the next item themselves (behind their first MFMAs); a
     // step that has nothing to compute issues them here. Past the last item the current one is
     // fetched again, into the stage nobody reads any more.
-    const int h_cp = more ? head_next : head, qb_cp = more ? qb_next : qb;
-    DkvWideCopies cp;
-    {
-      const size_t origin = (((size_t)b * p.S + qb_cp * kQueryTile) * p.Hq + h_cp) * D;
-      const size_t head_major = ((size_t)b * p.Hq + h_cp) * p.S + qb_cp * kQueryTile;
-      const size_t row_major = (size_t)b * p.S + qb_cp * kQueryTile;
-      cp.q = reinterpret_cast<const char*>(p.q + origin);
-      cp.dout = reinterpret_cast<const char*>(p.dout + origin);
-      cp.stat0 = w == 0 ? reinterpret_cast<const char*>(p.lse2 + head_major) : reinterpret_cast<const char*>(p.seg + row_major);
-      cp.stat1 = w == 0 ? reinterpret_cast<const char*>(p.delta + head_major)
-                        : reinterpret_cast<const char*>(has_end ? p.end + row_major : p.seg + row_major);
-      const unsigned other = (unsigned)(uintptr_t)(lds0 + (CUR ^ 1) * kStage);
-      cp.tile_dst = uniform(other + w * 1024);
-      cp.stat_dst = uniform(other + QdoStage<D>::kLse + w * 256);
-    }
-    const unsigned lane16 = (unsigned)lane_id_here() * 16;
-    const int q_min = qb_bounds.min_nz, q_max = qb_bounds.max_id, q_end_max = qb_bounds.end_max,
-              q_end_min = qb_bounds.end_min, q_uni = qb_bounds.uniform;
+    const DkvWideCopies cp = rows_of(more ? head_next : head, more ? qb_next : qb);
+    const QueryBlockBounds q = qb_bounds;
     if (more) qb_bounds = query_block_bounds(meta_b, qb_next);
     bool visit[2], interior[2];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
-      visit[kb] = blocks_interact(q_min, q_max, q_end_max, my_min[kb], my_max[kb], (rb0 + kb) * 32);
-      interior[kb] = tile_is_interior(q_uni, q_end_min, my_uni[kb], (rb0 + kb) * 32 + 31);
+      visit[kb] = blocks_interact(q.min_nz, q.max_id, q.end_max, my_min[kb], my_max[kb], (rb0 + kb) * 32);
+      interior[kb] = tile_is_interior(q.uniform, q.end_min, my_uni[kb], (rb0 + kb) * 32 + 31);
     }
     if (visit[0] && visit[1] && interior[0] && interior[1]) {
-      dkvw_fast_step<CUR * kStage>(kf, rp, tp, stat_ptr, scale_log2e, v_off, dma, cp, lane16);
+      dkvw_fast_step<kThis, kOther>(f, cp, dma, lane16);
     } else if (visit[0] || visit[1]) {
       // Some pair of the step is not allowed (or one block has nothing to do with this query
       // block): the S blocks start from -inf there.
@@ -280,9 +341,9 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           }
         }
       }
-      dkvw_masked_step<CUR * kStage>(kf, rp, tp, stat_ptr, scale_log2e, v_off, dma, cp, lane16, s_init[0], s_init[1]);
+      dkvw_masked_step<kThis, kOther>(f, cp, dma, lane16, s_init[0], s_init[1]);
     } else if (more) {
-      qdo_fetch_wide(dma, p, b, head_next, qb_next, lds0 + (CUR ^ 1) * kStage);
+      qdo_fetch_wide(dma, p, b, head_next, qb_next, lds0 + kOther);
     }
     dma_wait_all();
     __syncthreads();
@@ -297,7 +358,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   }
 
   // Accumulators out of their registers, one 32-key block at a time.
-  const lds_addr patch = lds0 + v_off;  // V rows are no longer needed
+  const lds_addr patch = lds0 + f.v_off;  // V rows are no longer needed
   auto finish = [&](auto kb_tag) {
     constexpr int kb = decltype(kb_tag)::value;
     f32x16 dvacc[4] = {dkvw_read_accumulator<4 * kb + 0>(), dkvw_read_accumulator<4 * kb + 1>(),

@@ -10,8 +10,6 @@ starts with lgkmcnt(0)).
 Run ``python gen_attn_asm.py > ct_attn_asm.inc`` after editing; the output is committed.
 """
 
-import os
-
 SCRATCH0 = 240
 # The compiler cannot see the MFMAs inside an asm statement, so it will not insert the wait
 # states that a vector ALU read of a fresh MFMA result needs; the sequences end with them.
@@ -293,25 +291,41 @@ def w_acc(i):
     return "a[%d:%d]" % (16 * i, 16 * i + 15)
 
 
-def dkvw_fast_sequence(masked=False):
-    """One (head, query block) step for both key blocks.
+class WideOperands:
+    """Names of the asm operands of one stream (strings such as "%12")."""
 
-    operands: %0-%7 K fragments of key block 0 (k-step), %8-%15 of key block 1; %16-%23
-    row-fragment pointers (k-step); %24-%27 lo and %28-%31 hi pointers of the transposed
-    fragments (column block); %32 pointer of this lane's statistics (LDS base + 16 * (lane /
-    32)); %33 scale * log2(e) (scalar); %34 byte offset of this wavefront's V rows (scalar; key
-    block 1: 8192 later); %35 byte offset of the stage (Q tile, dO tile 8192 later, -lse / scale
-    at 16384, -delta at 16512).
+    def __init__(self, first_input, masked):
+        n = first_input
+        self.k = [["%%%d" % (n + 8 * kb + ks) for ks in range(8)] for kb in range(2)]   # K fragments [kb][ks]
+        self.rp = ["%%%d" % (n + 16 + ks) for ks in range(8)]                          # row-fragment pointers
+        self.tlo = ["%%%d" % (n + 24 + db) for db in range(4)]                         # transposed fragments, lo
+        self.thi = ["%%%d" % (n + 28 + db) for db in range(4)]                         # ... hi
+        self.stat = "%%%d" % (n + 32)      # pointer of this lane's statistics (LDS base + 16 * (lane / 32))
+        self.scale = "%%%d" % (n + 33)     # scale * log2(e), scalar
+        self.voff = "%%%d" % (n + 34)      # byte offset of this wavefront's V rows, scalar
+        self.src = ["%%%d" % (n + 35 + i) for i in range(4)]   # Q rows, dO rows, two statistics arrays (scalar pairs)
+        self.tile_base = "%%%d" % (n + 39)  # LDS address of this wavefront's first slot of a Q tile at stage offset 0
+        self.stat_base = "%%%d" % (n + 40)  # LDS address of its first statistics array at stage offset 0
+        self.count = n + 41
+        if masked:
+            self.sinit = ["%%%d" % (n + 41), "%%%d" % (n + 42)]
+            self.count = n + 43
 
-    The copies of the next item (its Q and dO rows and statistics, into the other stage) are
-    issued from inside the stream, one behind each of the first ten MFMAs: %36-%39 this thread's
-    four source offsets of a 32 x 128 tile; %40, %41 the Q and dO rows (scalar pairs); %42, %43 the
-    two statistics arrays this wavefront fetches; %44 LDS address of this wavefront's first slot of
-    the other stage's Q tile; %45 LDS address of its first statistics array there; %46 16 * lane.
+
+def dkvw_stream(o, stage, other, loff, lane16, masked=False):
+    """One (head, query block) step of the wide dK/dV kernel for both key blocks.
+
+    `stage` / `other`: byte offsets (operand names or numbers) of the stage that is read (Q tile, dO
+    tile 8192 later, -lse / scale at 16384, -delta at 16512) and of the stage the next item is
+    copied into; `loff` the four registers with this thread's source offsets of a 32 x 128 tile,
+    `lane16` the register with 16 * lane.
+
+    The copies of the next item (its Q and dO rows and statistics) are issued from inside the
+    stream, one behind each of the first ten MFMAs.
 
     The S blocks start from -lse / scale of their query rows (read from the stage) and the dP
     blocks from -delta. With `masked`, the starting values of the two S blocks come in registers
-    instead (%47, %48): the caller has put -inf where a pair is not allowed, and the sum, the
+    instead (o.sinit): the caller has put -inf where a pair is not allowed, and the sum, the
     probability and dS of such a pair are then -inf, 0 and 0 without any instruction here knowing
     about masks.
     """
@@ -321,11 +335,11 @@ def dkvw_fast_sequence(masked=False):
         # The S and dP blocks start from the per-row terms instead of 0: -lse / scale and -delta of
         # the block's 16 query rows (4 consecutive rows per read, the accumulator's own order).
         for qd in range(0 if masked else 4):
-            st.lds("ds_read_b128 v[%d:%d], %%32 offset:%%35+%d" % (W_S[kb] + 4 * qd, W_S[kb] + 4 * qd + 3, 16384 + 32 * qd),
-                   "stat%d" % kb)
+            st.lds("ds_read_b128 v[%d:%d], %s offset:%s+%d" % (W_S[kb] + 4 * qd, W_S[kb] + 4 * qd + 3, o.stat, stage,
+                                                                16384 + 32 * qd), "stat%d" % kb)
         for qd in range(4):
-            st.lds("ds_read_b128 v[%d:%d], %%32 offset:%%35+%d" % (W_DP[kb] + 4 * qd, W_DP[kb] + 4 * qd + 3, 16512 + 32 * qd),
-                   "stat%d" % kb)
+            st.lds("ds_read_b128 v[%d:%d], %s offset:%s+%d" % (W_DP[kb] + 4 * qd, W_DP[kb] + 4 * qd + 3, o.stat, stage,
+                                                                16512 + 32 * qd), "stat%d" % kb)
 
     stats(0)
 
@@ -341,20 +355,20 @@ def dkvw_fast_sequence(masked=False):
     for kb in range(2):
         for ks in range(8):
             base = len(reads)
-            reads.append(["ds_read_b128 {v4}, %%%d offset:%%35" % (16 + ks)])                      # Q
-            reads.append(["ds_read_b128 {v4}, %%%d offset:%%35+8192" % (16 + ks)])                 # dO
-            reads.append(["v_add_u32_e32 v%d, %%34, %%%d" % (W_ADDR, 16 + ks),                       # V
+            reads.append(["ds_read_b128 {v4}, %s offset:%s" % (o.rp[ks], stage)])                   # Q
+            reads.append(["ds_read_b128 {v4}, %s offset:%s+8192" % (o.rp[ks], stage)])              # dO
+            reads.append(["v_add_u32_e32 v%d, %s, %s" % (W_ADDR, o.voff, o.rp[ks]),                  # V
                           "ds_read_b128 {v4}, v%d offset:%d" % (W_ADDR, 8192 * kb)])
-            c_s = "%%%d" % (47 + kb) if (masked and ks == 0) else acc16(W_S[kb])
-            mfmas.append(("v_mfma_f32_32x32x16_bf16 %s, {r0}, %%%d, %s" % (acc16(W_S[kb]), 8 * kb + ks, c_s), [base]))
+            c_s = o.sinit[kb] if (masked and ks == 0) else acc16(W_S[kb])
+            mfmas.append(("v_mfma_f32_32x32x16_bf16 %s, {r0}, %s, %s" % (acc16(W_S[kb]), o.k[kb][ks], c_s), [base]))
             mfmas.append(("v_mfma_f32_32x32x16_bf16 %s, {r0}, {r1}, %s" % (acc16(W_DP[kb]), acc16(W_DP[kb])), [base + 1, base + 2]))
     for kb in range(2):
         for step in range(2):
             for db in range(4):
                 for which in range(2):  # 0: dV (P^T, dO), 1: dK (dS^T, Q)
-                    off = "%%35+%d" % (step * 4096 + (8192 if which == 0 else 0))
-                    reads.append(["ds_read_b64_tr_b16 {v2lo}, %%%d offset:%s" % (24 + db, off),
-                                  "ds_read_b64_tr_b16 {v2hi}, %%%d offset:%s" % (28 + db, off)])
+                    off = "%s+%d" % (stage, step * 4096 + (8192 if which == 0 else 0))
+                    reads.append(["ds_read_b64_tr_b16 {v2lo}, %s offset:%s" % (o.tlo[db], off),
+                                  "ds_read_b64_tr_b16 {v2hi}, %s offset:%s" % (o.thi[db], off)])
                     acc = w_acc((0 if which == 0 else 8) + 4 * kb + db)
                     src = (W_S if which == 0 else W_DP)[kb] + 4 * step
                     mfmas.append(("v_mfma_f32_32x32x16_bf16 %s, v[%d:%d], {r0}, %s" % (acc, src, src + 3, acc),
@@ -371,7 +385,7 @@ def dkvw_fast_sequence(masked=False):
         done = {}
         for e in range(16):
             t = 16 + 16 * kb + (11 * e) // 8
-            fill[t] += ["v_mul_f32_e32 v%d, %%33, v%d" % (S + e, S + e),
+            fill[t] += ["v_mul_f32_e32 v%d, %s, v%d" % (S + e, o.scale, S + e),
                         "v_exp_f32_e32 v%d, v%d" % (S + e, S + e)]
             # the dP block is first read two MFMAs later: its last MFMA has long retired by then
             fill[t + 2] += ["v_mul_f32_e32 v%d, v%d, v%d" % (DP + e, S + e, DP + e)]
@@ -404,12 +418,12 @@ def dkvw_fast_sequence(masked=False):
     copies = []
     for which in range(2):
         for n in range(4):
-            copies.append((["s_add_u32 m0, %%44, %d" % (8192 * which + 2048 * n)],
-                           ["global_load_lds_dwordx4 %%%d, %%%d" % (36 + n, 40 + which)]))
-    copies.append((["s_mov_b32 m0, %45"],
-                   ["s_mov_b64 exec, 0xff", "global_load_lds_dwordx4 %46, %42", "s_mov_b64 exec, -1"]))
-    copies.append((["s_add_u32 m0, %45, 128"],
-                   ["s_mov_b64 exec, 0xff", "global_load_lds_dwordx4 %46, %43", "s_mov_b64 exec, -1"]))
+            copies.append((["s_add_u32 m0, %s, %s+%d" % (o.tile_base, other, 8192 * which + 2048 * n)],
+                           ["global_load_lds_dwordx4 %s, %s" % (loff[n], o.src[which])]))
+    for which in range(2):
+        copies.append((["s_add_u32 m0, %s, %s+%d" % (o.stat_base, other, 128 * which)],
+                       ["s_mov_b64 exec, 0xff", "global_load_lds_dwordx4 %s, %s" % (lane16, o.src[2 + which]),
+                        "s_mov_b64 exec, -1"]))
 
     issue_reads()
     for i, (text, needs) in enumerate(mfmas):
@@ -428,10 +442,43 @@ def dkvw_fast_sequence(masked=False):
             stats(1)   # (the registers are free: their last readers were the previous step's MFMAs)
         issue_reads()
         for line in fill[i]:
-            if not os.environ.get("KO_FILL"):
-                st.emit(line)
+            st.emit(line)
     assert not fill[64] and state["issued"] == len(reads)
-    return st.lines + TAIL
+    return st.lines
+
+
+def dkvw_step_sequence(masked=False):
+    """A single step. operands: %0-%40 as WideOperands(0) lays them out, %41 / %42 the S starting
+    values (masked form only), then the stage offset, the other stage's offset (immediates), the four
+    source offsets of this thread and 16 * lane."""
+    o = WideOperands(0, masked)
+    n = o.count
+    stage, other = "%%%d" % n, "%%%d" % (n + 1)
+    loff = ["%%%d" % (n + 2 + i) for i in range(4)]
+    return dkvw_stream(o, stage, other, loff, "%%%d" % (n + 6), masked) + TAIL
+
+
+def dkvw_run_sequence():
+    """A run of all-allowed steps over consecutive query blocks of one head: the stream of the
+    stage the run starts on, then the stream of the other stage, and so on, each followed by the
+    wait for the copies it issued and the workgroup barrier; the source offsets advance by one
+    query block per step.
+
+    operands: %0 steps left (scalar, counted down to 0); %1-%4 this thread's source offsets and %5
+    16 * lane (advanced); %6-%46 as WideOperands(6) lays them out; %47 bytes between the Q rows of
+    consecutive query blocks (scalar); %48 / %49 byte offsets of the stage the run starts on and of
+    the other one.
+    """
+    o = WideOperands(6, False)
+    assert o.count == 47
+    loff, lane16 = ["%1", "%2", "%3", "%4"], "%5"
+    close = ["s_waitcnt vmcnt(0)", "s_barrier"] + ["v_add_u32_e32 %s, %%47, %s" % (r, r) for r in loff] + [
+        "v_add_u32_e32 %s, 0x80, %s" % (lane16, lane16), "s_sub_u32 %0, %0, 1", "s_cmp_eq_u32 %0, 0"]
+    lines = ["dkvw_run_%=:"]
+    lines += dkvw_stream(o, "%48", "%49", loff, lane16) + close + ["s_cbranch_scc1 dkvw_run_end_%="]
+    lines += dkvw_stream(o, "%49", "%48", loff, lane16) + close + ["s_cbranch_scc0 dkvw_run_%="]
+    lines += ["dkvw_run_end_%=:"]
+    return lines + TAIL
 
 
 def dkvw_zero():
@@ -460,8 +507,9 @@ if __name__ == "__main__":
     print(emit(dq_acc_half_sequence(), "CT_DQ_ACC_HALF_SEQUENCE"))
     print(emit(dkv_sdp_sequence(), "CT_DKV_SDP_SEQUENCE"))
     print(emit(dkv_acc_sequence(), "CT_DKV_ACC_SEQUENCE"))
-    print(emit(dkvw_fast_sequence(), "CT_DKVW_FAST_SEQUENCE"))
-    print(emit(dkvw_fast_sequence(masked=True), "CT_DKVW_MASKED_SEQUENCE"))
+    print(emit(dkvw_step_sequence(), "CT_DKVW_FAST_SEQUENCE"))
+    print(emit(dkvw_step_sequence(masked=True), "CT_DKVW_MASKED_SEQUENCE"))
+    print(emit(dkvw_run_sequence(), "CT_DKVW_RUN_SEQUENCE"))
     print(emit(dkvw_zero(), "CT_DKVW_ZERO"))
     print(emit(dkvw_read(), "CT_DKVW_READ"))
     print(clobbers())
