@@ -178,6 +178,45 @@ __device__ __forceinline__ void apply_rotary_chunk(const ct_rotary_args& a, long
   }
 }
 
+// Any head_dim and any even rotary dimension, one thread per (token, head) row and one channel
+// pair at a time: the shapes the 16-byte kernel above does not take (e.g. 4 rotated channels of 8).
+// Same arithmetic, element for element.
+template <bool ADJACENT>
+__global__ __launch_bounds__(256) void apply_rotary_rows_kernel(ct_rotary_args a) {
+  const int heads = a.q_heads + a.kv_heads;
+  const long gid = (long)blockIdx.x * 256 + threadIdx.x;
+  if (gid >= (long)a.tokens * heads) return;
+  const long t = gid / heads;
+  const int h = (int)(gid % heads);
+  const bool is_q = h < a.q_heads;
+  const bf16* in = reinterpret_cast<const bf16*>(is_q ? a.q_in : a.k_in);
+  bf16* out = reinterpret_cast<bf16*>(is_q ? a.q_out : a.k_out);
+  const size_t base = (is_q ? ((size_t)t * a.q_heads + h) : ((size_t)t * a.kv_heads + (h - a.q_heads))) * a.head_dim;
+  const bool scale_on = is_q && a.q_scale != 1.0f;
+  const float s = (float)(bf16)a.q_scale;
+  const float sign = a.inverse ? -1.f : 1.f;
+  const bf16* cs = reinterpret_cast<const bf16*>(a.cosine) + (size_t)t * a.rotary_pairs;
+  const bf16* sn = reinterpret_cast<const bf16*>(a.sine) + (size_t)t * a.rotary_pairs;
+  for (int i = 0; i < a.rotary_pairs; ++i) {
+    const int c1 = ADJACENT ? 2 * i : i, c2 = ADJACENT ? 2 * i + 1 : i + a.rotary_pairs;
+    bf16 x1 = in[base + c1], x2 = in[base + c2];
+    if (a.inverse) {
+      x1 = scaled(x1, s, scale_on);
+      x2 = scaled(x2, s, scale_on);
+    }
+    const float co = (float)cs[i], si = sign * (float)sn[i];
+    bf16 r1 = (bf16)((float)x1 * co - (float)x2 * si);
+    bf16 r2 = (bf16)((float)x2 * co + (float)x1 * si);
+    if (!a.inverse) {
+      r1 = scaled(r1, s, scale_on);
+      r2 = scaled(r2, s, scale_on);
+    }
+    out[base + c1] = r1;
+    out[base + c2] = r2;
+  }
+  for (int c = 2 * a.rotary_pairs; c < a.head_dim; ++c) out[base + c] = scaled(in[base + c], s, scale_on);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -314,6 +353,55 @@ __global__ __launch_bounds__(256) void rms_norm_bwd_kernel(const uint16_t* x, co
 // dscale[col] = sum of the wavefronts' partial rows in a fixed order: thread (c, g) adds the rows
 // of sixteenth g for column 64 blockIdx.x + c (four independent chains, joined in order), then the
 // sixteen group sums are added in order.
+// Any hidden size that is a multiple of 8: the row is walked three times (sum of squares, the
+// dot product, dx; the repeats are served from cache) and the wavefront's dscale sums live in its
+// row of `partial` instead of registers (a lane only ever touches its own columns of it).
+__global__ __launch_bounds__(256) void rms_norm_bwd_any_kernel(const uint16_t* x, const uint16_t* scale,
+                                                               const uint16_t* dy, float eps, long rows, int d,
+                                                               uint16_t* dx, float* partial) {
+  const int lane = threadIdx.x & 63, chunks = d / 8;
+  const long wv = (long)blockIdx.x * 4 + (threadIdx.x >> 6), waves = (long)gridDim.x * 4;
+  float* prow = partial + (size_t)wv * d;
+  for (int c = lane; c < chunks; c += 64)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) prow[c * 8 + e] = 0.f;
+  for (long row = wv; row < rows; row += waves) {
+    const uint16_t* xr = x + (size_t)row * d;
+    const uint16_t* gr = dy + (size_t)row * d;
+    float ss = 0.f;
+    for (int c = lane; c < chunks; c += 64) {
+      const bf16x8 xv = as_bf16x8(*reinterpret_cast<const u32x4*>(xr + c * 8));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ss += (float)xv[e] * (float)xv[e];
+    }
+    ss = wave_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)d + eps);
+    float dot = 0.f;
+    for (int c = lane; c < chunks; c += 64) {
+      const bf16x8 xv = as_bf16x8(*reinterpret_cast<const u32x4*>(xr + c * 8));
+      const bf16x8 gv = as_bf16x8(*reinterpret_cast<const u32x4*>(gr + c * 8));
+      const bf16x8 wv8 = as_bf16x8(*reinterpret_cast<const u32x4*>(scale + c * 8));
+#pragma unroll
+      for (int e = 0; e < 8; ++e) dot += (float)gv[e] * (float)wv8[e] * ((float)xv[e] * r);
+    }
+    dot = wave_sum(dot) / (float)d;
+    uint16_t* dr = dx + (size_t)row * d;
+    for (int c = lane; c < chunks; c += 64) {
+      const bf16x8 xv = as_bf16x8(*reinterpret_cast<const u32x4*>(xr + c * 8));
+      const bf16x8 gv = as_bf16x8(*reinterpret_cast<const u32x4*>(gr + c * 8));
+      const bf16x8 wv8 = as_bf16x8(*reinterpret_cast<const u32x4*>(scale + c * 8));
+      bf16x8 o;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float xhat = (float)xv[e] * r;
+        o[e] = (bf16)(r * ((float)gv[e] * (float)wv8[e] - xhat * dot));
+        prow[c * 8 + e] += (float)gv[e] * (float)(bf16)xhat;
+      }
+      *reinterpret_cast<u32x4*>(dr + c * 8) = as_u32x4(o);
+    }
+  }
+}
+
 __global__ __launch_bounds__(1024) void rms_norm_dscale_kernel(const float* partial, int waves, int d,
                                                                float* dscale) {
   __shared__ float group[16][64];
@@ -386,16 +474,24 @@ extern "C" int32_t ct_apply_rotary(void* stream, const ct_rotary_args* a) {
   const int rotary_dim = 2 * a->rotary_pairs;
   CT_REQUIRE(a->rotary_pairs > 0 && rotary_dim <= a->head_dim,
              "ct_apply_rotary: invalid rotary dimension %d for head_dim=%d", rotary_dim, a->head_dim);
-  CT_REQUIRE(a->head_dim % 8 == 0 && rotary_dim % 16 == 0,
-             "ct_apply_rotary: head_dim %d must be a multiple of 8 and the rotary dimension %d of 16",
-             a->head_dim, rotary_dim);
+  const bool vector_path = a->head_dim % 8 == 0 && rotary_dim % 16 == 0;
   CT_REQUIRE(a->q_scale == a->q_scale && a->q_scale - a->q_scale == 0.f,
              "ct_apply_rotary: q_scale must be finite");
-  CT_REQUIRE(aligned16(a->q_in) && aligned16(a->k_in) && aligned16(a->q_out) && aligned16(a->k_out) &&
-                 aligned16(a->cosine) && aligned16(a->sine),
+  CT_REQUIRE(!vector_path || (aligned16(a->q_in) && aligned16(a->k_in) && aligned16(a->q_out) && aligned16(a->k_out) &&
+                              aligned16(a->cosine) && aligned16(a->sine)),
              "ct_apply_rotary: pointers must be 16-byte aligned");
   CT_REQUIRE(a->tokens <= 0x7fffffffll, "ct_apply_rotary: at most 2^31 - 1 tokens per call");
   LaunchScope scope("apply_rotary_kernel", (hipStream_t)stream);
+  if (!vector_path) {
+    // head_dim not a multiple of 8 or fewer than 16 rotated channels at a time: element-wise kernel
+    const long rows = (long)a->tokens * (a->q_heads + a->kv_heads);
+    const dim3 grid((unsigned)((rows + 255) / 256));
+    if (a->rope_style == CT_ROPE_GPT_J)
+      hipLaunchKernelGGL((apply_rotary_rows_kernel<true>), grid, dim3(256), 0, (hipStream_t)stream, *a);
+    else
+      hipLaunchKernelGGL((apply_rotary_rows_kernel<false>), grid, dim3(256), 0, (hipStream_t)stream, *a);
+    return scope.done();
+  }
   if (a->rope_style == CT_ROPE_GPT_J)
     hipLaunchKernelGGL((apply_rotary_kernel<true>), dim3((unsigned)a->tokens), dim3(256), 0,
                        (hipStream_t)stream, *a);
@@ -438,8 +534,7 @@ extern "C" int32_t ct_rms_norm_bwd(void* stream_, const uint16_t* x, const uint1
                                    size_t workspace_bytes) {
   CT_REQUIRE(x && scale && dy && dx && dscale && workspace, "ct_rms_norm_bwd: null pointer");
   CT_REQUIRE(rows > 0, "ct_rms_norm_bwd: rows must be positive");
-  CT_REQUIRE(hidden == 512 || hidden == 1024 || hidden == 2048 || hidden == 4096 || hidden == 8192,
-             "ct_rms_norm_bwd: hidden size must be 512, 1024, 2048, 4096 or 8192, got %d", hidden);
+  CT_REQUIRE(hidden > 0 && hidden % 8 == 0, "ct_rms_norm_bwd: hidden size must be a multiple of 8, got %d", hidden);
   CT_REQUIRE(aligned16(x) && aligned16(scale) && aligned16(dy) && aligned16(dx) && aligned16(workspace),
              "ct_rms_norm_bwd: pointers must be 16-byte aligned");
   if (workspace_bytes < ct_rms_norm_bwd_workspace_bytes(hidden))
@@ -449,7 +544,10 @@ extern "C" int32_t ct_rms_norm_bwd(void* stream_, const uint16_t* x, const uint1
   float* partial = static_cast<float*>(workspace);
   LaunchScope scope("rms_norm_bwd_kernel", stream);
   const dim3 grid(kNormBwdBlocks), block(256);
-  switch (hidden / 512) {
+  // rows held in registers for 512 * {1, 2, 4, 8, 16}; any other multiple of 8 walks the row
+  const bool in_registers = hidden == 512 || hidden == 1024 || hidden == 2048 || hidden == 4096 || hidden == 8192;
+  switch (in_registers ? hidden / 512 : 0) {
+    case 0: hipLaunchKernelGGL(rms_norm_bwd_any_kernel, grid, block, 0, stream, x, scale, dy, eps, (long)rows, hidden, dx, partial); break;
     case 1: hipLaunchKernelGGL((rms_norm_bwd_kernel<1>), grid, block, 0, stream, x, scale, dy, eps, (long)rows, dx, partial); break;
     case 2: hipLaunchKernelGGL((rms_norm_bwd_kernel<2>), grid, block, 0, stream, x, scale, dy, eps, (long)rows, dx, partial); break;
     case 4: hipLaunchKernelGGL((rms_norm_bwd_kernel<4>), grid, block, 0, stream, x, scale, dy, eps, (long)rows, dx, partial); break;

@@ -266,7 +266,9 @@ typedef struct ct_rotary_args {
 /*
  * Partial rotary embedding of Q and K from precomputed tables. The rotation is
  * evaluated in f32 from the bf16 operands and rounded once to bf16.
- * Supported: head_dim % 8 == 0, rotary_dim % 16 == 0, rotary_dim <= head_dim.
+ * Supported: any head_dim and any even rotary_dim <= head_dim (head_dim % 8 == 0 with
+ * rotary_dim % 16 == 0 takes the 16-byte kernel and needs 16-byte aligned pointers, other
+ * shapes an element-wise one).
  * Replaces: apply_rotary_cos_sin (src/modeling/rotary.py:160-204) and its
  * transpose under autodiff.
  */
@@ -285,7 +287,8 @@ size_t ct_rms_norm_bwd_workspace_bytes(int32_t hidden);
 
 /*
  * Gradients of ct_rms_norm_fwd: dx bf16 [rows, hidden], dscale f32 [hidden]
- * (summed over rows in a fixed order). hidden in {512, 1024, 2048, 4096, 8192}.
+ * (summed over rows in a fixed order). hidden % 8 == 0 (512 * {1, 2, 4, 8, 16}
+ * keeps the row in registers; other sizes walk it three times).
  * Replaces: the autodiff transpose of rms_norm (src/modeling/architecture.py:155-162).
  */
 int32_t ct_rms_norm_bwd(void* stream, const uint16_t* x, const uint16_t* scale, const uint16_t* dy,

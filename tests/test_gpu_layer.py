@@ -78,7 +78,9 @@ def _pair_bound(x, rotary_dim, style):
 
 @pytest.mark.parametrize("style", ["gpt-j", "gpt-neox"])
 @pytest.mark.parametrize("shape", [(1, 5, 2, 1, 16, 16), (2, 130, 8, 2, 64, 32), (2, 512, 32, 8, 128, 64),
-                                   (1, 64, 4, 4, 128, 128)])
+                                   (1, 64, 4, 4, 128, 128),
+                                   # outside the 16-byte kernel's granularity: the element-wise kernel
+                                   (1, 4, 2, 2, 8, 4), (2, 37, 3, 1, 12, 6), (1, 9, 2, 1, 64, 24), (1, 3, 1, 1, 10, 10)])
 def test_rotary_matches_oracle(ct, gpu, style, shape):
     batch, seq, q_heads, kv_heads, head_dim, rotary_dim = shape
     rng = np.random.default_rng(sum(shape))
@@ -103,20 +105,21 @@ def test_rotary_matches_oracle(ct, gpu, style, shape):
                      <= 2.0 ** -8 * 1.4143 * _pair_bound(x, rotary_dim, style).double() + 1e-30).all())
 
 
-def test_rotary_reference_example_with_tail_channels(ct, gpu):
-    # reference tests/modeling/test_rotary.py:92-98: rotary_dim 4 of 8 is below this library's
-    # granularity (16 rotated channels), so the same construction is run at 16 of 32 channels.
+@pytest.mark.parametrize("head_dim,rotary_dim", [(8, 4), (32, 16)])
+def test_rotary_reference_example_with_tail_channels(ct, gpu, head_dim, rotary_dim):
+    # reference tests/modeling/test_rotary.py:92-98 (rotary_dim 4 of 8: the element-wise kernel) and the
+    # same construction at 16 of 32 channels (the 16-byte kernel)
     positions = np.array([[0, 1, 0, 2_000_000]], dtype=np.int32)
-    inv_freq = layer_ref.inverse_frequencies(16, 1e4)
-    query = torch.arange(1 * 4 * 2 * 32, dtype=torch.float32).reshape(1, 4, 2, 32).to(torch.bfloat16)
+    inv_freq = layer_ref.inverse_frequencies(rotary_dim, 1e4)
+    query = torch.arange(1 * 4 * 2 * head_dim, dtype=torch.float32).reshape(1, 4, 2, head_dim).to(torch.bfloat16)
     key = (query + torch.tensor(0.5, dtype=torch.bfloat16)).to(torch.bfloat16)
     cosine, sine = ct.rotary_cos_sin(torch.from_numpy(positions).to(gpu), torch.from_numpy(inv_freq).to(gpu))
     pre_q, pre_k = ct.apply_rotary_cos_sin(query.to(gpu), key.to(gpu), cosine, sine)
     direct_q, direct_k = ct.apply_rotary_embedding(query.to(gpu), key.to(gpu), torch.from_numpy(positions).to(gpu),
                                                    torch.from_numpy(inv_freq).to(gpu))
     assert torch.equal(pre_q, direct_q) and torch.equal(pre_k, direct_k)
-    assert torch.equal(pre_q[..., 16:].cpu(), query[..., 16:])
-    assert torch.equal(pre_k[..., 16:].cpu(), key[..., 16:])
+    assert torch.equal(pre_q[..., rotary_dim:].cpu(), query[..., rotary_dim:])
+    assert torch.equal(pre_k[..., rotary_dim:].cpu(), key[..., rotary_dim:])
     # position 0 rotates by nothing
     assert torch.equal(pre_q[:, 0].cpu(), query[:, 0]) and torch.equal(pre_q[:, 2].cpu(), query[:, 2])
 
@@ -197,7 +200,9 @@ def test_rms_norm_special_rows(ct, gpu):
     assert ct.rms_norm(x[:0], scale, 1e-6).shape == (0, 512)
 
 
-@pytest.mark.parametrize("rows,hidden", [(3, 512), (257, 1024), (4100, 4096), (33, 8192)])
+@pytest.mark.parametrize("rows,hidden", [(3, 512), (257, 1024), (4100, 4096), (33, 8192),
+                                         # sizes outside 512 * 2^k: the kernel that walks the row
+                                         (2, 8), (700, 136), (1030, 768), (65, 5120), (5, 16384)])
 def test_rms_norm_gradients_match_oracle(ct, gpu, rows, hidden):
     rng = np.random.default_rng(rows * 3 + hidden)
     x = _bf16(rng.standard_normal((rows, hidden)) * rng.uniform(0.1, 4.0, size=(rows, 1)))
@@ -211,6 +216,6 @@ def test_rms_norm_gradients_match_oracle(ct, gpu, rows, hidden):
     assert attention_ref.relative_l2(xg.grad.cpu(), dx64) <= 1e-2
     assert attention_ref.relative_l2(sg.grad.cpu(), want_dscale) <= 2e-2
     assert attention_ref.relative_l2(sg.grad.cpu(), dscale64) <= 1e-2
-    with pytest.raises(RuntimeError, match="hidden size must be"):
-        bad = torch.ones((2, 136), dtype=torch.bfloat16, device=gpu, requires_grad=True)
-        ct.rms_norm(bad, torch.ones(136, dtype=torch.bfloat16, device=gpu), 1e-6).sum().backward()
+    with pytest.raises((RuntimeError, ValueError), match="multiple of 8"):
+        bad = torch.ones((2, 132), dtype=torch.bfloat16, device=gpu, requires_grad=True)
+        ct.rms_norm(bad, torch.ones(132, dtype=torch.bfloat16, device=gpu), 1e-6).sum().backward()
