@@ -100,6 +100,32 @@ def mean(values):
     return sum(values) / len(values)
 
 
+def graph_replay_ms(torch, step, steps):
+    """ms per step when the step's launches are replayed from one captured HIP graph (the entry
+    points only enqueue kernels, so they capture as they are): what a caller that submits the step
+    as a graph sees. None if capture is refused."""
+
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - start) / steps * 1e3
+    except RuntimeError:
+        return None
+
+
 def attention_step_for(ct, config, inputs):
     W = ct.workloads
     pairs = W.count_allowed_pairs(inputs["segment_ids"], inputs["attention_end"])
@@ -189,6 +215,7 @@ def bench_attention(ct, torch, steps, warmup, preamble_steps):
     ms_per_step = elapsed / steps * 1e3
     return {
         "config": config, "pairs": pairs, "flops": flops, "ms_per_step": ms_per_step,
+        "graph_replay_ms_per_step": graph_replay_ms(torch, step, steps),
         "tflops": flops["total"] / (ms_per_step * 1e-3) / 1e12, "kernels": kernel_table(config, pairs, kernels),
         "inputs": inputs,
     }
@@ -235,6 +262,7 @@ def bench_attention_shapes(ct, torch, steps, warmup):
         tflops = flops["total"] / (ms * 1e-3) / 1e12
         entries.append({"shape": name, "workload": label, "allowed_pairs": pairs, "flops_per_step": flops["total"],
                         "steps": steps, "ms_per_step": ms, "mask_aware_tflops": tflops,
+                        "graph_replay_ms_per_step": graph_replay_ms(torch, step, steps),
                         "pct_bf16_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
                         "kernels": [{k: v for k, v in e.items() if k != "launches"}
                                     for e in kernel_table(config, pairs, kernels)]})
@@ -511,6 +539,8 @@ def main():
             "traffic": measured_traffic(dominant["kernel"]),
         },
         "kernels": attention["kernels"],
+        # the same step replayed from a captured HIP graph (not the headline: `value` is the eager step)
+        "graph_replay_ms_per_step": attention["graph_replay_ms_per_step"],
     }
     result["dkv_wide_variant"] = bench_dkv_wide(ct, torch, config, attention, min(args.steps, 50), min(args.warmup, 10))
     result["delta_pass"] = bench_delta_pass(ct, torch, config, attention["inputs"]["q"])
