@@ -28,6 +28,14 @@ template <int D>
 using LeanTrFrags = std::conditional_t<(D / 8 >= 16), TrFragCompact<D / 8, KSlots::kAccum>,
                                        TrFragOffsets<D / 8, KSlots::kAccum>>;
 
+// The dK/dV kernels work on unscaled Q K^T and put the softmax scale into the exponent. Any finite
+// scale is legal (the operator only asks for a finite one): a scale of exactly 0 is replaced there
+// by a positive number so small that scale * S vanishes against lse in f32 all the same (dK is
+// still multiplied by the true scale, 0), and a masked pair is marked by the infinity that the
+// scale's sign turns into -inf in the exponent.
+CT_DEVICE float exponent_scale(float scale) { return scale == 0.f ? 1e-30f : scale; }
+CT_DEVICE float masked_score(float scale) { return scale < 0.f ? -kNegInf : kNegInf; }
+
 // P = exp2(S log2e - lse2), dS = P (dP - delta) for one 32-key block, in place in s.
 CT_DEVICE void dq_arith(f32x16& s, const f32x16& dp, float lse2, float delta_q) {
 #pragma unroll
@@ -98,7 +106,7 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
     // for the dK/dV kernel: the values it adds to its S and dP blocks, P = exp2((S - lse / scale) *
     // scale * log2(e)) and dS = P (dP - delta)
     p.delta[stat_t] = -delta_q;
-    p.lse2[stat_t] = -p.lse[ctx.stat_off] / p.scale;
+    p.lse2[stat_t] = -p.lse[ctx.stat_off] / exponent_scale(p.scale);
   }
 
   auto step = [&](auto stage_tag) {
@@ -616,7 +624,8 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   // The Q tiles stay unscaled in LDS: the softmax scale enters the exponent in f32
   // (S = scale * (Q K^T); the forward rounded scale * Q to bf16 first, a difference of one
   // bf16 rounding per element of Q) and dK = scale * (dS^T Q) is scaled once at the end.
-  const float scale_log2e = p.scale * kLog2e;
+  const float scale_log2e = exponent_scale(p.scale) * kLog2e;
+  const float masked = masked_score(p.scale);
 
   // Work items: (head of the group, query block) pairs, flattened; query block fastest.
   const int nq = (q_lo <= q_hi) ? (q_hi - q_lo + 1) : 0;
@@ -690,7 +699,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const bool ok = (seg4[e] == seg_k_or_never) & (key <= end4[e]);
-            s[4 * qd + e] = ok ? s[4 * qd + e] : kNegInf;
+            s[4 * qd + e] = ok ? s[4 * qd + e] : masked;
           }
         }
       }

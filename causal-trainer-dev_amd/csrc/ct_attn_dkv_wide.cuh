@@ -192,7 +192,8 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   f.tp = TrFragOffsets<16, KSlots::kAccum>(lds0);
   f.v_off = DkvWideLds::kVResident + w * (64 * 256);  // this wavefront's V rows
   f.stat_ptr = lds0 + 16 * half;
-  f.scale_log2e = p.scale * kLog2e;
+  f.scale_log2e = exponent_scale(p.scale) * kLog2e;
+  const float masked = masked_score(p.scale);
   f.tile_base = uniform((unsigned)(uintptr_t)lds0 + w * 1024);
   f.stat_base = uniform((unsigned)(uintptr_t)lds0 + QdoStage<D>::kLse + w * 256);
 #pragma unroll
@@ -316,7 +317,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       dkvw_fast_step<kThis, kOther>(f, cp, dma, lane16);
     } else if (visit[0] || visit[1]) {
       // Some pair of the step is not allowed (or one block has nothing to do with this query
-      // block): the S blocks start from -inf there.
+      // block): the S blocks start from the infinity that the exponent turns into -inf there.
       f32x16 s_init[2];
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
@@ -337,7 +338,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const bool ok = visit[kb] & (interior[kb] | ((seg4[e] == seg_k_or_never) & (key <= end4[e])));
-            s_init[kb][4 * qd + e] = ok ? lse4[e] : kNegInf;
+            s_init[kb][4 * qd + e] = ok ? lse4[e] : masked;
           }
         }
       }

@@ -122,6 +122,36 @@ def test_forward_backward_match_oracle(ct, gpu, case, dkv_variant):
     _check_against_oracle(results, q, k, v, dout, ids, ends, scale)
 
 
+@pytest.mark.parametrize("scale", [0.0, -0.09, 1.0])
+@pytest.mark.parametrize("dim", [64, 128])
+def test_any_finite_scale(ct, gpu, dkv_variant, scale, dim):
+    """The operator accepts any finite scale (src/kernels/efficient_attention.py:1947-1957): 0 gives
+    uniform attention over the allowed keys (dQ and dK exactly 0), a negative one turns the order of
+    the scores around; the dK/dV kernels, which carry the scale in the exponent, must follow."""
+
+    rng = np.random.default_rng(int(abs(scale) * 100) + dim)
+    batch, seq, q_heads, kv_heads = 2, 256, 4, 2
+    ids = _layout(rng, batch, seq, holes=True)
+    ends = _random_ends(rng, ids)
+    # scale 1 needs small scores to stay inside the stated tolerances of bf16 probabilities
+    spread = 0.25 if scale == 1.0 else 1.0
+    q = _bf16(rng.standard_normal((batch, seq, q_heads, dim)) * spread)
+    k = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)) * spread)
+    v = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
+    dout = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
+    results = _run_gpu(ct, gpu, q, k, v, dout, ids, ends, scale)
+    if scale == 0.0:
+        assert not results[2].any() and not results[3].any()
+        out, lse, _, _, dv = results
+        allowed = ref.allowed_from_canonical(ids, ends)
+        out_ref, _, _, dv_ref = ref.vanilla_attention_vjp(q, k, v, allowed, dout, scale=scale)
+        assert float((out.float() - out_ref.float()).abs().max()) <= O_ATOL
+        assert float((lse - ref.efficient_lse(q, k, allowed, scale=scale)).abs().max()) <= LSE_ATOL
+        assert ref.relative_l2(dv, dv_ref) <= GRAD_RTOL
+    else:
+        _check_against_oracle(results, q, k, v, dout, ids, ends, scale)
+
+
 def test_edge_layouts(ct, gpu, dkv_variant):
     rng = np.random.default_rng(11)
     batch, seq, q_heads, kv_heads, dim = 4, 256, 4, 2, 128
