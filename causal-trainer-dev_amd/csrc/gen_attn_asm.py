@@ -254,11 +254,12 @@ def dq_acc_half_sequence(ahead=4, slots=4):
 # both key blocks (their first 8 registers later hold the bf16 P and dS fragments) and the 16
 # lse2 / delta values of this lane's query rows.
 # ---------------------------------------------------------------------------
-W_RING0, W_SLOTS = 236, 5
-W_S = (172, 204)      # S^T accumulators of key block 0 / 1 (16 registers each)
-W_DP = (188, 220)     # dP accumulators
-W_ADDR = 171          # address of a V fragment
-W_FIRST = 171
+W_SLOTS = 5
+W_RING0 = 256 - 4 * W_SLOTS
+W_S = (W_RING0 - 64, W_RING0 - 32)      # S^T accumulators of key block 0 / 1 (16 registers each)
+W_DP = (W_RING0 - 48, W_RING0 - 16)     # dP accumulators
+W_ADDR = W_RING0 - 65                   # address of a V fragment
+W_FIRST = W_ADDR
 
 
 class Stream:

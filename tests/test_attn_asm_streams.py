@@ -129,8 +129,10 @@ def test_model_catches_the_mistakes_it_is_meant_for(gen):
     assert any("no MFMA has read" in p for p in Model().run(lost).problems)
     # arithmetic directly behind the MFMA that produces its input
     wide = gen.dkvw_step_sequence()
-    last_s0 = max(i for i, line in enumerate(wide) if line.startswith("v_mfma") and line.split()[1].startswith("v[172:187]"))
-    early = wide[:last_s0 + 1] + ["v_mul_f32_e32 v172, %33, v172"] + wide[last_s0 + 1:]
+    s0 = gen.W_S[0]
+    block = "v[%d:%d]" % (s0, s0 + 15)
+    last_s0 = max(i for i, line in enumerate(wide) if line.startswith("v_mfma") and line.split()[1].startswith(block))
+    early = wide[:last_s0 + 1] + ["v_mul_f32_e32 v%d, %%33, v%d" % (s0, s0)] + wide[last_s0 + 1:]
     assert any("after the MFMA that wrote it" in p for p in Model().run(early).problems)
 
 
