@@ -223,14 +223,14 @@ def bench_attention(ct, torch, steps, warmup, preamble_steps):
 
 def bench_dkv_wide(ct, torch, config, attention, steps, warmup):
     """The same step with the other dK/dV kernel (one wavefront of 64 keys per SIMD), for the
-    record: the headline above uses the default kernel."""
+    record: at this sequence length the default is the kernel with two wavefronts per SIMD."""
 
     ct.set_dkv_variant(1)
     try:
         step, _, _ = attention_step_for(ct, config, attention["inputs"])
         elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
     finally:
-        ct.set_dkv_variant(0)
+        ct.set_dkv_variant(-1)
     ms_per_step = elapsed / steps * 1e3
     return {
         "note": "ct_attn_set_dkv_variant(1); not the headline",

@@ -281,8 +281,8 @@ def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=Non
 
 
 def set_dkv_variant(variant: int) -> None:
-    """Choose the dK/dV kernel of the backward for head dimension 128, process-wide: 0 the default
-    (two wavefronts per SIMD), 1 the wide one (one wavefront per SIMD, 64 keys)."""
+    """Choose the dK/dV kernel of the backward for head dimension 128, process-wide: 0 two wavefronts
+    per SIMD, 1 the wide one (one wavefront per SIMD, 64 keys), -1 (the default) by sequence length."""
 
     _lib.check(_lib.load().ct_attn_set_dkv_variant(int(variant)))
 

@@ -173,11 +173,12 @@ int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16_t* dout,
                       float* delta, int64_t rows, int32_t head_dim);
 
 /* Chooses the dK/dV kernel ct_attn_bwd runs for head dimension 128 (process-wide; no counterpart
- * in the reference, which has one backward). 0 (the default): two wavefronts per SIMD, 32 keys
- * each. 1: one wavefront per SIMD with 64 keys, the (dK, dV) sums in the accumulation registers
- * and each step as one generated instruction stream with the exponent / dS arithmetic and the
- * next item's copies between its own MFMAs. Both give the same results within the operator's
- * tolerances (not bitwise: f32 summation order differs). */
+ * in the reference, which has one backward). 0: two wavefronts per SIMD, 32 keys each. 1: one
+ * wavefront per SIMD with 64 keys, the (dK, dV) sums in the accumulation registers and each step
+ * as one generated instruction stream with the exponent / dS arithmetic and the next item's copies
+ * between its own MFMAs. -1 (the default): by sequence length, kernel 1 from 16384 positions on
+ * (its looping streams need long segments to pay off), kernel 0 below. Both give the same results
+ * within the operator's tolerances (not bitwise: f32 summation order differs). */
 int32_t ct_attn_set_dkv_variant(int32_t variant);
 
 /* ------------------------------------------------------------------------

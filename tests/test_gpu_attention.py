@@ -97,12 +97,13 @@ CASES = [
 
 @pytest.fixture(params=[0, 1], ids=["dkv32", "dkv64"])
 def dkv_variant(request, ct):
-    """Both dK/dV kernels of the backward: two wavefronts of 32 keys per SIMD (the default) and
-    one wavefront of 64 keys (head dimension 128 only; other dimensions run the default)."""
+    """Both dK/dV kernels of the backward: two wavefronts of 32 keys per SIMD and one wavefront of
+    64 keys (head dimension 128 only; other dimensions run the first). Tests without this fixture
+    run the default, which chooses by sequence length."""
 
     ct.set_dkv_variant(request.param)
     yield request.param
-    ct.set_dkv_variant(0)
+    ct.set_dkv_variant(-1)
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_S%d_Hq%d_Hkv%d_D%d_%s%s" % (
@@ -120,6 +121,30 @@ def test_forward_backward_match_oracle(ct, gpu, case, dkv_variant):
     print("case", case, flush=True)
     results = _run_gpu(ct, gpu, q, k, v, dout, ids, ends, scale)
     _check_against_oracle(results, q, k, v, dout, ids, ends, scale)
+
+
+@pytest.mark.parametrize("seq,expected", [(8192, 0), (16384, 1)])
+def test_default_dkv_kernel_goes_by_sequence_length(ct, gpu, seq, expected):
+    """Left to itself the backward runs the wide dK/dV kernel from 16384 positions on and the other
+    one below; each kernel is deterministic, so the default's dK and dV are bitwise those of the
+    kernel it should have chosen (and, the summation order being different, not the other's)."""
+
+    rng = np.random.default_rng(seq)
+    ids = _layout(rng, 1, seq, max_len=3000)
+    q, dout = (_bf16(rng.standard_normal((1, seq, 2, 128))) for _ in range(2))
+    k, v = (_bf16(rng.standard_normal((1, seq, 1, 128))) for _ in range(2))
+    results = {}
+    try:
+        for variant in (-1, 0, 1):
+            ct.set_dkv_variant(variant)
+            print("seq", seq, "variant", variant, flush=True)
+            results[variant] = _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5)
+    finally:
+        ct.set_dkv_variant(-1)
+    for index in (3, 4):
+        assert torch.equal(results[-1][index], results[expected][index])
+        assert not torch.equal(results[-1][index], results[1 - expected][index])
+        assert ref.relative_l2(results[0][index], results[1][index]) <= 1e-2
 
 
 @pytest.mark.parametrize("scale", [0.0, -0.09, 1.0])
