@@ -25,6 +25,7 @@ Exactly one JSON line is printed on stdout.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -86,13 +87,20 @@ def timed_region(torch, step, steps, warmup, timer_factory):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    with timer_factory() as timer:
-        torch.cuda.synchronize()
-        start = time.perf_counter()
-        for _ in range(steps):
-            step()
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - start
+    # No cyclic garbage collection inside the timed region: a collection that happens to free an
+    # earlier phase's few hundred timing events costs tens of milliseconds of host time.
+    gc.collect()
+    gc.disable()
+    try:
+        with timer_factory() as timer:
+            torch.cuda.synchronize()
+            start = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            elapsed = time.perf_counter() - start
+    finally:
+        gc.enable()
     return elapsed, timer.durations_ms()
 
 

@@ -48,4 +48,7 @@ class KernelTimer:
         result = collections.defaultdict(list)
         for name, begin, end in self._pending:
             result[name].append(begin.elapsed_time(end))
+        # the events are released here, in the caller's time, not whenever a later garbage
+        # collection finds this object (it holds a callback that refers back to it)
+        self._pending = []
         return dict(result)
