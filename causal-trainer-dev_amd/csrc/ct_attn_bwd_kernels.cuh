@@ -124,7 +124,7 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
       const int k_uniform = uniform(kb.uniform);
       const bool need_seg = ctx.mine.uniform == 0 || ctx.mine.uniform != k_uniform;
       const bool need_causal = t * kKeyTile + kKeyTile - 1 > ctx.mine.end_min;
-      const int seg_cmp = ctx.row_valid ? ctx.seg_q : -1;
+      const int seg_cmp = ctx.row_valid() ? ctx.seg_q : -1;
       int last_rel = ctx.end_q - t * kKeyTile - 4 * half;
       if (k_uniform != 0 && seg_cmp != k_uniform) last_rel = -1;
       constexpr int kOff = CUR * kStage + KvStage<D>::kK, vOff = CUR * kStage + KvStage<D>::kV;

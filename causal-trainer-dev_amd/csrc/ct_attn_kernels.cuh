@@ -121,7 +121,9 @@ struct QueryWork {
   // explicit coordinates: batch row, KV head, head slice of the group, query tile
   CT_DEVICE QueryWork(const AttnParams& p, int b_, int kvh_, int slice, int qt_)
       : b(b_), kvh(kvh_), qt(qt_) {
-    const int w = threadIdx.x >> 6;
+    // (wave-uniform, and said so: head and row block are then scalars that cost nothing to keep
+    // or to form again, instead of per-lane values hoisted out of the caller's loop)
+    const int w = uniform(threadIdx.x >> 6);
     h = kvh * (p.Hq / p.Hkv) + slice * HS + (w % HS);
     rb = qt * PB + (w / HS);
   }
@@ -252,7 +254,6 @@ struct QueryTileContext {
   QueryBlockBounds mine;
   int first, last;
   int pos, seg_q, end_q;
-  bool row_valid;
   bool active;  // false for the row blocks past the end of a partial last tile
   size_t q_off, stat_off;
   const bf16* kbase;
@@ -265,9 +266,7 @@ struct QueryTileContext {
   }
   CT_DEVICE void init(const AttnParams& p) {
     const int nrb = p.S / 32;
-    meta_b = p.meta + (size_t)work.b * nrb * kMetaW;
-    active = work.rb < nrb;
-    if (!active) work.rb = nrb - 1;  // keeps every address below in range
+    derive(p);
     mine = query_block_bounds(meta_b, work.rb);
     if (!active) mine.min_nz = 0;    // interacts with nothing
     first = INT_MAX;
@@ -279,16 +278,62 @@ struct QueryTileContext {
       first = min(first, uniform(m[kKvFirst]));
       last = max(last, uniform(m[kKvLast]));
     }
-    pos = work.rb * 32 + (lane_id() & 31);
     seg_q = p.seg[(size_t)work.b * p.S + pos];
     end_q = p.end ? p.end[(size_t)work.b * p.S + pos] : pos;
-    row_valid = seg_q != 0;
+  }
+  // everything that follows from the coordinates by arithmetic
+  CT_DEVICE void derive(const AttnParams& p) {
+    const int nrb = p.S / 32;
+    meta_b = p.meta + (size_t)work.b * nrb * kMetaW;
+    active = work.rb < nrb;
+    if (!active) work.rb = nrb - 1;  // keeps every address below in range
+    pos = work.rb * 32 + (lane_id_here() & 31);
     q_off = (((size_t)work.b * p.S + pos) * p.Hq + work.h) * D;
     stat_off = ((size_t)work.b * p.S + pos) * p.Hq + work.h;
     kbase = p.k + ((size_t)work.b * p.S * p.Hkv + work.kvh) * D;
     vbase = p.v + ((size_t)work.b * p.S * p.Hkv + work.kvh) * D;
     segb = p.seg + (size_t)work.b * p.S;
   }
+
+  // The same context from values read earlier: the bounds (scalar loads, so that waiting for
+  // them is no wait for vector memory) and the row's id and visible end.
+  struct TileBounds {
+    // as loaded: nothing is computed from them where they are requested, so nothing waits there
+    QueryBlockBounds mine;
+    int kv_first[PB], kv_last[PB];
+  };
+  CT_DEVICE static TileBounds tile_bounds(const AttnParams& p, const QueryWork<HS, NW>& work) {
+    const int nrb = p.S / 32;
+    const int* meta = p.meta + (size_t)work.b * nrb * kMetaW;
+    TileBounds t;
+    t.mine = query_block_bounds(meta, min(work.rb, nrb - 1));
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+      const MetaPtr m = meta_const(meta + min(work.qt * PB + i, nrb - 1) * kMetaW);
+      t.kv_first[i] = m[kKvFirst];
+      t.kv_last[i] = m[kKvLast];
+    }
+    return t;
+  }
+  CT_DEVICE QueryTileContext(const AttnParams& p, int b, int kvh, int slice, int qt, const TileBounds& t,
+                             int seg_q_, int end_q_)
+      : work(p, b, kvh, slice, qt) {
+    const int nrb = p.S / 32;
+    derive(p);
+    mine = t.mine;
+    if (!active) mine.min_nz = 0;
+    first = INT_MAX;
+    last = -1;
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+      if (work.qt * PB + i >= nrb) break;
+      first = min(first, uniform(t.kv_first[i]));
+      last = max(last, uniform(t.kv_last[i]));
+    }
+    seg_q = seg_q_;
+    end_q = p.end ? end_q_ : pos;
+  }
+  CT_DEVICE bool row_valid() const { return seg_q != 0; }
   // does this wavefront's row block have anything in key tile t (bounds kb)?
   CT_DEVICE bool wave_visits(const KeyTileBounds& kb, int t) const {
     return blocks_interact(mine.min_nz, mine.max_id, mine.end_max, uniform(kb.min_nz),
@@ -410,22 +455,57 @@ struct VkFetcher {
   }
 };
 
-// One query tile (kFwdWaves / HS row blocks x HS heads of one KV head), start to finish.
+// What a query tile reads from memory before its first key tile can be fetched, read ahead by the
+// tile before it (one workgroup owns the compute unit: nothing else would hide these round
+// trips). The bounds are requested at the start of the previous tile, as scalar loads that
+// complete with that tile's own; the rows (id, visible end, Q) behind its last key tile.
 template <int D, int HS>
-CT_DEVICE void attn_fwd_item(const AttnParams& p, int b, int kvh, int slice, int qt,
-                             const lds_addr lds0, const RowFragOffsets<D / 8>& ro,
+struct FwdAhead {
+  using Context = QueryTileContext<D, HS, kFwdWaves>;
+  int b, qt;
+  typename Context::TileBounds bounds;
+  int seg_q, end_q;
+  u32x4 q[D / 16];
+  CT_DEVICE void request_bounds(const AttnParams& p, int b_, int kvh, int slice, int qt_) {
+    b = b_;
+    qt = qt_;
+    bounds = Context::tile_bounds(p, QueryWork<HS, kFwdWaves>(p, b, kvh, slice, qt));
+  }
+  // rows of tile (b, qt), as set by request_bounds
+  CT_DEVICE void request_rows(const AttnParams& p, int kvh, int slice) {
+    const QueryWork<HS, kFwdWaves> work(p, b, kvh, slice, qt);
+    // (lane id made opaque: the lane's share of the addresses is rebuilt here instead of being
+    // kept in registers across the whole kernel)
+    const int l = lane_id_here();
+    const size_t position = (size_t)b * p.S + min(work.rb, p.S / 32 - 1) * 32 + (l & 31);
+    seg_q = p.seg[position];
+    // (always a load: a value formed here instead would first have to wait for the load before
+    // it, which may still own the register; the context ignores it without visible ends)
+    end_q = (p.end ? p.end : p.seg)[position];
+    const bf16* rows = p.q + (position * p.Hq + work.h) * D + 8 * (l >> 5);
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) q[ks] = load_global16(rows + 16 * ks);
+  }
+};
+
+// One query tile (kFwdWaves / HS row blocks x HS heads of one KV head), start to finish. `ahead`
+// holds what this tile read ahead on entry and what tile (batch row next_b, tile next_qt) did on
+// return. The request is unconditional (the last tile of a workgroup names itself again): a
+// conditional one would keep the old Q registers alive through the whole tile.
+template <int D, int HS>
+CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int next_b,
+                             int next_qt, int kvh, int slice, const lds_addr lds0,
+                             const RowFragOffsets<D / 8>& ro,
                              const TrFragOffsets<D / 8, KSlots::kAccum>& to) {
   constexpr int kStage = VkStage<D>::kBytes;
-  const QueryTileContext<D, HS, kFwdWaves> ctx(p, b, kvh, slice, qt);
+  const QueryTileContext<D, HS, kFwdWaves> ctx(p, ahead.b, kvh, slice, ahead.qt, ahead.bounds, ahead.seg_q,
+                                                ahead.end_q);
+
   const int l = lane_id(), half = l >> 5, w = threadIdx.x >> 6;
   const bool late = uniform(w) >= kFwdWaves / 2;
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
 
-  bf16x8 qf[D / 16];
-#pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks)
-    qf[ks] = scale_bf16x8(as_bf16x8(load_global16(p.q + ctx.q_off + 16 * ks + 8 * half)), p.scale);
 
   f32x16 oacc[D / 32];
 #pragma unroll
@@ -446,21 +526,19 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, int b, int kvh, int slice, int
     if (t + 1 <= last) nb = key_tile_bounds(ctx.meta_b, t + 1);
     visit = ctx.wave_visits(kb, t);
   }
+  // the next tile's bounds: scalar loads behind this tile's first copies; nothing here uses them
+  ahead.request_bounds(p, next_b, kvh, slice, next_qt);
+  // (the Q rows are touched only now: the first copies above needed nothing but the bounds)
+  bf16x8 qf[D / 16];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) qf[ks] = scale_bf16x8(as_bf16x8(ahead.q[ks]), p.scale);
   dma_wait_all();
   __syncthreads();
   if (visit) scores_t<D>(kStage + VkStage<D>::kK, ro, qf, s);
   if (late) __builtin_amdgcn_s_barrier();
 
-  // One step = VALU phase + MFMA phase of tile t; CUR is the buffer of stage t.
-  auto step = [&](auto stage_tag) {
-    constexpr int CUR = decltype(stage_tag)::value;
-    const lds_addr next_stage = lds0 + (CUR ^ 1) * kStage;
-    // ---- VALU phase ----
-    if (late) fetch.issue_stage(t + 1, last, next_stage, lds0);
-    // bounds of tile t + 2: requested now, first needed one step from now
-    KeyTileBounds nnb = nb;
-    if (t + 2 <= last) nnb = key_tile_bounds(ctx.meta_b, t + 2);
-    bf16x8 pf[4];
+  // The VALU phase of tile t: masks, running maximum and sum, probabilities as bf16 fragments.
+  auto softmax_phase = [&](bf16x8* pf) {
     if (visit) {
       float mx = kNegInf;
       {
@@ -472,7 +550,7 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, int b, int kvh, int slice, int
         const bool need_seg = ctx.mine.uniform == 0 || ctx.mine.uniform != k_uniform;
         const bool need_causal = t * kKeyTile + kKeyTile - 1 > ctx.mine.end_min;
         if (need_seg || need_causal) {
-          const int seg_cmp = ctx.row_valid ? ctx.seg_q : -1;
+          const int seg_cmp = ctx.row_valid() ? ctx.seg_q : -1;
           int last_rel = ctx.end_q - t * kKeyTile - 4 * half;
           if (mixed_keys) {
             mask_scores_t<true, true>(lds0 + VkStage<D>::seg_slot(t), seg_cmp, last_rel, s);
@@ -515,22 +593,41 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, int b, int kvh, int slice, int
 #pragma unroll
       for (int step4 = 0; step4 < 4; ++step4) pf[step4] = pack_acc8(s[step4 >> 1], step4 & 1);
     }
+  };
+  // O^T += V^T P^T for the tile in buffer CUR
+  auto pv_phase = [&](auto stage_tag, const bf16x8* pf) {
+    constexpr int CUR = decltype(stage_tag)::value;
+    if constexpr (D == 128) {
+      pv_sequence_128<CUR * kStage + VkStage<D>::kV>(to, pf, oacc);
+    } else {
+#pragma unroll
+      for (int step4 = 0; step4 < 4; ++step4)
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+          oacc[db] = mfma32(to.load(CUR * kStage + VkStage<D>::kV, step4, db), pf[step4], oacc[db]);
+    }
+  };
+
+  // One step = VALU phase + MFMA phase of tile t < last; CUR is the buffer of stage t.
+  auto step = [&](auto stage_tag) {
+    constexpr int CUR = decltype(stage_tag)::value;
+    const lds_addr next_stage = lds0 + (CUR ^ 1) * kStage;
+    // ---- VALU phase ----
+    if (late) fetch.issue_stage(t + 1, last, next_stage, lds0);
+    // bounds of tile t + 2: requested now, first needed one step from now
+    KeyTileBounds nnb = nb;
+    if (t + 2 <= last) nnb = key_tile_bounds(ctx.meta_b, t + 2);
+    bf16x8 pf[4];
+    softmax_phase(pf);
     if (!late) dma_wait_all();  // stage t, issued one step ago
     __builtin_amdgcn_s_barrier();
     // ---- MFMA phase ----
     if (!late) fetch.issue_stage(t + 1, last, next_stage, lds0);
-    const bool visit_next = (t + 1 <= last) && ctx.wave_visits(nb, t + 1);
+    const bool visit_next = ctx.wave_visits(nb, t + 1);
+    if (visit) pv_phase(stage_tag, pf);
     if constexpr (D == 128) {
-      if (visit) pv_sequence_128<CUR * kStage + VkStage<D>::kV>(to, pf, oacc);
       if (visit_next) qk_sequence_128<CUR * kStage + VkStage<D>::kK>(ro, qf, s);
     } else {
-      if (visit) {
-#pragma unroll
-        for (int step4 = 0; step4 < 4; ++step4)
-#pragma unroll
-          for (int db = 0; db < D / 32; ++db)
-            oacc[db] = mfma32(to.load(CUR * kStage + VkStage<D>::kV, step4, db), pf[step4], oacc[db]);
-      }
       if (visit_next) scores_t<D>(CUR * kStage + VkStage<D>::kK, ro, qf, s);
     }
     if (late) dma_wait_all();  // stage t + 1, issued at the start of this step
@@ -540,20 +637,47 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, int b, int kvh, int slice, int
     nb = nnb;
     ++t;
   };
-  while (t <= last) {
+  const bool any_tile = t <= last;
+  while (t < last) {
     step(std::integral_constant<int, 0>{});
-    if (t > last) break;
+    if (t >= last) break;
     step(std::integral_constant<int, 1>{});
   }
+  // The step of the last tile: nothing to fetch and no scores to form, so the Q registers are
+  // free, and no later wait of this tile is a wait for memory: the next tile's rows are requested
+  // behind the last such wait and land under the PV product, the stores of O and the next
+  // tile's first copies. (One call site for every path: several would meet in register copies
+  // that wait for the loads.)
+  bf16x8 pf[4];
+  if (any_tile) {
+    softmax_phase(pf);
+    if (!late) dma_wait_all();  // stage t, issued one step ago
+    __builtin_amdgcn_s_barrier();
+  }
+  ahead.request_rows(p, kvh, slice);
+  if (any_tile) {
+    if (visit) {
+      if (((last - ctx.first) & 1) == 0)
+        pv_phase(std::integral_constant<int, 0>{}, pf);
+      else
+        pv_phase(std::integral_constant<int, 1>{}, pf);
+    }
+    __builtin_amdgcn_s_barrier();
+  }
   if (!late) __builtin_amdgcn_s_barrier();
-  dma_wait_all();
-  __syncthreads();  // every wavefront is done with the stages before they become store patches
+  // Every copy of this tile has been waited for by the wavefronts that issued it, so only LDS
+  // traffic has to settle before the stages become store patches (a wait for memory here would
+  // wait for the next tile's loads).
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
 
   const float l_tot = pair_sum(l_run);
   const bool has = l_tot > 0.f;
   const float inv = has ? 1.f / l_tot : 0.f;
   if (ctx.active) {
-    if (half == 0) p.lse[ctx.stat_off] = has ? (__logf(l_tot) + m_run * kLn2) : 0.f;
+    const int le = lane_id_here();
+    const size_t stat = ((size_t)ctx.work.b * p.S + ctx.work.rb * 32 + (le & 31)) * p.Hq + ctx.work.h;
+    if (le < 32) p.lse[stat] = has ? (__logf(l_tot) + m_run * kLn2) : 0.f;
     const lds_addr patch = lds0 + w * 32 * D * 2;
     bf16* obase = p.out + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
     store_rows_t<D>(oacc, inv, patch, obase, q_row_stride);
@@ -584,9 +708,17 @@ attn_fwd_kernel(AttnParams p) {
   const MetaPtr region = meta_const(p.meta + bin_region_offset(p.B, nrb, PB));
   const int tpr = bin_tiles_per_row(nrb, PB);
   const int it_end = uniform(region[bin + 1]);
-  for (int it = uniform(region[bin]); it < it_end; ++it) {
+  int it = uniform(region[bin]);
+  if (it >= it_end) return;
+  FwdAhead<D, HS> ahead;
+  {
     const int item = uniform(region[kBins + 1 + it]);
-    attn_fwd_item<D, HS>(p, item / tpr, kvh, slice, item % tpr, lds0, ro, to);
+    ahead.request_bounds(p, item / tpr, kvh, slice, item % tpr);
+    ahead.request_rows(p, kvh, slice);
+  }
+  for (; it < it_end; ++it) {
+    const int next_item = uniform(region[kBins + 1 + min(it + 1, it_end - 1)]);
+    attn_fwd_item<D, HS>(p, ahead, next_item / tpr, next_item % tpr, kvh, slice, lds0, ro, to);
   }
 }
 
