@@ -13,7 +13,10 @@ HBM rate of the delta pass, and a CPU baseline: this repository's CPU restatemen
 reference's pure path, timed on the host cores on a bounded sample.
 
 Before the warm-up a fixed, disclosed clock-ramp preamble runs (``preamble_steps`` untimed
-attention steps) so that short runs (--steps 20 --warmup 5) see the same clocks as long ones.
+attention steps) so that short runs (--steps 20 --warmup 5) see the same clocks as long ones; it
+runs directly in front of the warm-up, with the per-launch timer already in place, because the
+clock falls back within milliseconds of the device going idle (measured: host work between the
+preamble and 5 + 20 steps made them 12 % slower than the same steps in a 50 + 200 run).
 The line also carries the other named attention shapes (``attention_shapes``: C1 packed small,
 C4 MaskGIT hybrid mask, C5 long context), cut-CE with the f32 logits cache (``cutce``) and
 without it (``cutce_recompute``, the reference's residual contract: nothing but lse is kept),
@@ -83,17 +86,24 @@ def calibration_copy(ct, torch, nbytes):
     torch.cuda.synchronize()
 
 
-def timed_region(torch, step, steps, warmup, timer_factory):
-    for _ in range(warmup):
-        step()
-    torch.cuda.synchronize()
-    # No cyclic garbage collection inside the timed region: a collection that happens to free an
+def timed_region(torch, step, steps, warmup, timer_factory, preamble=0):
+    """`preamble` + W untimed steps, then exactly K timed ones between two device synchronisations.
+    Nothing but the synchronisation sits between the untimed steps and the first timed one, and
+    nothing between the preamble and the warm-up: the shader clock drops within milliseconds of the
+    device going idle and takes tens of milliseconds of work to come back, so host work in such a
+    gap (a garbage collection, setting up the per-launch timer) made a 20-step region 12 % slower
+    than a 200-step one on the same device."""
+
+    # No cyclic garbage collection inside the region either: a collection that happens to free an
     # earlier phase's few hundred timing events costs tens of milliseconds of host time.
     gc.collect()
     gc.disable()
     try:
         with timer_factory() as timer:
+            for _ in range(preamble + warmup):
+                step()
             torch.cuda.synchronize()
+            timer.mark()  # launches recorded so far are warm-up
             start = time.perf_counter()
             for _ in range(steps):
                 step()
@@ -106,6 +116,19 @@ def timed_region(torch, step, steps, warmup, timer_factory):
 
 def mean(values):
     return sum(values) / len(values)
+
+
+def ramp_steps(torch, step, cap, seconds=0.3):
+    """How many untimed steps make up about `seconds` of work (at most `cap`): the clock-ramp
+    preamble of a shape whose step time is not known beforehand."""
+
+    step()
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    step()
+    torch.cuda.synchronize()
+    once = max(time.perf_counter() - start, 1e-6)
+    return max(0, min(cap, int(seconds / once)))
 
 
 def graph_replay_ms(torch, step, steps):
@@ -122,7 +145,7 @@ def graph_replay_ms(torch, step, steps):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             step()
-        for _ in range(3):
+        for _ in range(max(3, min(100, 2 * steps))):  # the capture idled the device: ramp the clock again
             graph.replay()
         torch.cuda.synchronize()
         start = time.perf_counter()
@@ -216,10 +239,9 @@ def bench_attention(ct, torch, steps, warmup, preamble_steps):
     inputs = W.make_attention_inputs(config, "cuda")
     step, _, pairs = attention_step_for(ct, config, inputs)
     flops = W.attention_flops(config, pairs)
-    for _ in range(preamble_steps):     # clock ramp, disclosed as preamble_steps
-        step()
-    torch.cuda.synchronize()
-    elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
+    # (the clock ramp, disclosed as preamble_steps, runs inside the helper so that nothing idles the
+    # device between it and the warm-up)
+    elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer, preamble=preamble_steps)
     ms_per_step = elapsed / steps * 1e3
     return {
         "config": config, "pairs": pairs, "flops": flops, "ms_per_step": ms_per_step,
@@ -229,14 +251,14 @@ def bench_attention(ct, torch, steps, warmup, preamble_steps):
     }
 
 
-def bench_dkv_wide(ct, torch, config, attention, steps, warmup):
+def bench_dkv_wide(ct, torch, config, attention, steps, warmup, preamble_steps):
     """The same step with the other dK/dV kernel (one wavefront of 64 keys per SIMD), for the
     record: at this sequence length the default is the kernel with two wavefronts per SIMD."""
 
     ct.set_dkv_variant(1)
     try:
         step, _, _ = attention_step_for(ct, config, attention["inputs"])
-        elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
+        elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer, preamble=preamble_steps)
     finally:
         ct.set_dkv_variant(-1)
     ms_per_step = elapsed / steps * 1e3
@@ -255,8 +277,10 @@ SHAPE_LABELS = {
 }
 
 
-def bench_attention_shapes(ct, torch, steps, warmup):
-    """Forward + backward at the other named attention shapes: ms, mask-aware TFLOP/s, pairs."""
+def bench_attention_shapes(ct, torch, steps, warmup, preamble_steps):
+    """Forward + backward at the other named attention shapes: ms, mask-aware TFLOP/s, pairs. Each
+    shape gets its own clock-ramp preamble of about 0.3 s of untimed steps (at most the headline's
+    preamble_steps; the count is in the entry)."""
 
     W = ct.workloads
     entries = []
@@ -265,11 +289,12 @@ def bench_attention_shapes(ct, torch, steps, warmup):
         inputs = W.make_attention_inputs(config, "cuda")
         step, _, pairs = attention_step_for(ct, config, inputs)
         flops = W.attention_flops(config, pairs)
-        elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer)
+        preamble = ramp_steps(torch, step, preamble_steps)
+        elapsed, kernels = timed_region(torch, step, steps, warmup, ct.profiling.KernelTimer, preamble=preamble)
         ms = elapsed / steps * 1e3
         tflops = flops["total"] / (ms * 1e-3) / 1e12
         entries.append({"shape": name, "workload": label, "allowed_pairs": pairs, "flops_per_step": flops["total"],
-                        "steps": steps, "ms_per_step": ms, "mask_aware_tflops": tflops,
+                        "steps": steps, "preamble_steps": preamble, "ms_per_step": ms, "mask_aware_tflops": tflops,
                         "graph_replay_ms_per_step": graph_replay_ms(torch, step, steps),
                         "pct_bf16_mfma_peak": 100.0 * tflops / PEAK_BF16_TFLOPS,
                         "kernels": [{k: v for k, v in e.items() if k != "launches"}
@@ -550,12 +575,14 @@ def main():
         # the same step replayed from a captured HIP graph (not the headline: `value` is the eager step)
         "graph_replay_ms_per_step": attention["graph_replay_ms_per_step"],
     }
-    result["dkv_wide_variant"] = bench_dkv_wide(ct, torch, config, attention, min(args.steps, 50), min(args.warmup, 10))
+    result["dkv_wide_variant"] = bench_dkv_wide(ct, torch, config, attention, min(args.steps, 50), min(args.warmup, 10),
+                                                    args.preamble_steps)
     result["delta_pass"] = bench_delta_pass(ct, torch, config, attention["inputs"]["q"])
     if args.calibration_copy_bytes:
         calibration_copy(ct, torch, args.calibration_copy_bytes)
     if not args.no_shapes:
-        result["attention_shapes"] = bench_attention_shapes(ct, torch, min(args.steps, 20), min(args.warmup, 5))
+        result["attention_shapes"] = bench_attention_shapes(ct, torch, min(args.steps, 20), min(args.warmup, 5),
+                                                             args.preamble_steps)
     cutce_for_cpu = None
     if not args.no_cutce:
         cut_steps = args.cutce_steps or min(args.steps, 10)

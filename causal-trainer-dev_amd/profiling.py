@@ -20,6 +20,7 @@ class KernelTimer:
     """Context manager: collects (kernel name -> list of durations in ms)."""
 
     def __init__(self):
+        self._first = 0
         self._pending = []
         self._open = {}
         self._callback = _lib.LAUNCH_HOOK(self._on_launch)
@@ -41,14 +42,21 @@ class KernelTimer:
         _lib.load().ct_set_launch_hook(ctypes.cast(None, _lib.LAUNCH_HOOK), None)
         return False
 
+    def mark(self) -> None:
+        """Launches recorded up to here are left out of durations_ms (warm-up). Costs nothing on
+        the device: their events are kept until the timer is read."""
+
+        self._first = len(self._pending)
+
     def durations_ms(self) -> dict[str, list[float]]:
-        """Synchronises and returns every recorded launch, grouped by kernel name."""
+        """Synchronises and returns every launch recorded since the last mark, grouped by kernel name."""
 
         torch.cuda.synchronize()
         result = collections.defaultdict(list)
-        for name, begin, end in self._pending:
+        for name, begin, end in self._pending[self._first:]:
             result[name].append(begin.elapsed_time(end))
         # the events are released here, in the caller's time, not whenever a later garbage
         # collection finds this object (it holds a callback that refers back to it)
         self._pending = []
+        self._first = 0
         return dict(result)
