@@ -19,7 +19,12 @@ from . import _lib
 class KernelTimer:
     """Context manager: collects (kernel name -> list of durations in ms)."""
 
-    def __init__(self):
+    def __init__(self, only=None):
+        """`only`: names of the kernels to time (default: every launch). Two events on the stream per
+        timed launch are not free on the device (2.5 % of a 1.1 ms step of five launches), so a
+        region whose total time matters times only the kernel it needs."""
+
+        self._only = None if only is None else frozenset(only)
         self._first = 0
         self._pending = []
         self._open = {}
@@ -27,6 +32,8 @@ class KernelTimer:
 
     def _on_launch(self, _user, kernel, phase, stream):
         name = kernel.decode()
+        if self._only is not None and name not in self._only:
+            return
         event = torch.cuda.Event(enable_timing=True)
         event.record(torch.cuda.ExternalStream(stream) if stream else torch.cuda.current_stream())
         if phase == 0:
