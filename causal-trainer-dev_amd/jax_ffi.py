@@ -21,7 +21,7 @@ GPU instead of a TPU.
 
 Every custom call goes through ``_call``, which checks operand, result and attribute counts
 against ``HANDLERS``, the table of the handlers that csrc/ct_ffi.cc defines
-(tests/test_host_and_abi.py keeps the two, and the list in INTEGRATION.md, in step).
+(tests/test_host_and_abi.py keeps the two, and the documented list of handlers, in step).
 
 jax is not installed in the build environment of this repository: this module has never been
 executed. Importing it does not import jax; the C ABI underneath it is exercised through ctypes.

@@ -165,7 +165,7 @@ def _ffi_handlers_in_source():
 
 def test_jax_binding_matches_the_ffi_handlers_and_the_documentation(ct):
     """The JAX side cannot run here (no jax): what can be held is static agreement between the
-    handlers csrc/ct_ffi.cc defines, the table and call sites of jax_ffi.py, and INTEGRATION.md."""
+    handlers csrc/ct_ffi.cc defines, the table and call sites of jax_ffi.py, and the integration document."""
 
     import ast
     import inspect
