@@ -181,7 +181,7 @@ def graph_replay_ms(torch, step, steps):
         return None
 
 
-def attention_step_for(ct, config, inputs):
+def attention_step_for(ct, config, inputs, **backward_pins):
     W = ct.workloads
     pairs = W.count_allowed_pairs(inputs["segment_ids"], inputs["attention_end"])
     profile = ct.resolve_attention_profile(inputs["q"].shape, inputs["k"].shape, None,
@@ -192,7 +192,7 @@ def attention_step_for(ct, config, inputs):
 
     def step():
         out, lse = ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
-        ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=config.scale)
+        ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=config.scale, **backward_pins)
 
     return step, metadata, pairs
 
@@ -203,18 +203,29 @@ ROOFLINE_CUTCE_KERNELS = ("cutce_stats_kernel", "cutce_dhidden_kernel", "cutce_d
 
 
 def kernel_table(config, pairs, kernels):
-    per_kernel_flops = {
-        "attn_fwd_kernel": 4 * config.head_dim * config.q_heads * pairs,
-        # backward = 5 GEMMs of algorithmic work, split by which kernel owns the result:
+    unit = config.head_dim * config.q_heads * pairs
+    if "attn_dq_blocks_kernel" in kernels:
+        # backward = 5 GEMMs, none evaluated twice: the dK/dV kernel owns S, dP, dV, dK (8 D per pair)
+        # and stores dS; dQ = dS K (2 D per pair) reads the blocks back and is bound by their bytes
+        per_kernel_flops = {"attn_fwd_kernel": 4 * unit, "attn_dkv_kernel": 8 * unit, "attn_dq_blocks_kernel": 2 * unit}
+    else:
+        # dQ recomputes S and dP: algorithmic work split by which kernel owns the result:
         # dQ kernel 4*D*Hq*pairs (dP, dQ), dK/dV kernel 6*D*Hq*pairs (S, dV, dK)
-        "attn_dq_kernel": 4 * config.head_dim * config.q_heads * pairs,
-        "attn_dkv_kernel": 6 * config.head_dim * config.q_heads * pairs,
+        per_kernel_flops = {"attn_fwd_kernel": 4 * unit, "attn_dq_kernel": 4 * unit, "attn_dkv_kernel": 6 * unit}
+    per_kernel_bytes = {
+        # O and dO read once, lse read, two statistics written
+        "attn_bwd_stats_kernel": config.batch * config.seq * config.q_heads * (4 * config.head_dim + 12),
+        # 2 bytes per allowed pair and head at least (blocks are stored whole: masked pairs of a visited
+        # 32 x 32 block are bytes too, so the executed figure is higher)
+        "attn_dq_blocks_kernel": 2 * config.q_heads * pairs,
     }
     table = []
     for name, durations in kernels.items():
         entry = {"kernel": name, "launches": len(durations), "avg_ms": mean(durations)}
         if name in per_kernel_flops:
             entry["algorithmic_tflops"] = per_kernel_flops[name] / (entry["avg_ms"] * 1e-3) / 1e12
+        if name in per_kernel_bytes:
+            entry["algorithmic_gbps"] = per_kernel_bytes[name] / (entry["avg_ms"] * 1e-3) / 1e9
         table.append(entry)
     return table
 
@@ -281,23 +292,22 @@ def bench_attention(ct, torch, steps, warmup, preamble_steps):
     }
 
 
-def bench_dkv_wide(ct, torch, config, attention, steps, warmup, preamble_steps):
-    """The same step with the other dK/dV kernel (one wavefront of 64 keys per SIMD), for the
-    record: at this sequence length the default is the kernel with two wavefronts per SIMD."""
+def bench_backward_forms(ct, torch, config, attention, steps, warmup, preamble_steps):
+    """The same step with the other forms of the backward pinned (ct_attn_bwd_args.variant), for the
+    record: dQ from dS blocks that the dK/dV kernel stores, and the wide dK/dV kernel."""
 
-    ct.set_dkv_variant(1)
-    try:
-        step, _, _ = attention_step_for(ct, config, attention["inputs"])
+    forms = {}
+    for name, pins in (("dq_from_ds", dict(dq_form="from_ds")),
+                       ("dq_recompute_dkv_wide", dict(dq_form="recompute", dkv_kernel="wide"))):
+        step, _, _ = attention_step_for(ct, config, attention["inputs"], **pins)
         elapsed, kernels, _ = timed_with_table(torch, ct, step, steps, warmup, preamble=preamble_steps)
-    finally:
-        ct.set_dkv_variant(-1)
-    ms_per_step = elapsed / steps * 1e3
-    return {
-        "note": "ct_attn_set_dkv_variant(1); not the headline",
-        "ms_per_step": ms_per_step,
-        "tflops": attention["flops"]["total"] / (ms_per_step * 1e-3) / 1e12,
-        "attn_dkv_kernel_ms": mean(kernels.get("attn_dkv_kernel", [0.0])),
-    }
+        ms_per_step = elapsed / steps * 1e3
+        forms[name] = {
+            "ms_per_step": ms_per_step,
+            "tflops": attention["flops"]["total"] / (ms_per_step * 1e-3) / 1e12,
+            "kernels_ms": {kernel: mean(times) for kernel, times in kernels.items()},
+        }
+    return forms
 
 
 SHAPE_LABELS = {
@@ -608,8 +618,8 @@ def main():
         # the same step replayed from a captured HIP graph (not the headline: `value` is the eager step)
         "graph_replay_ms_per_step": attention["graph_replay_ms_per_step"],
     }
-    result["dkv_wide_variant"] = bench_dkv_wide(ct, torch, config, attention, min(args.steps, 50), min(args.warmup, 10),
-                                                    args.preamble_steps)
+    result["backward_forms"] = bench_backward_forms(ct, torch, config, attention, min(args.steps, 50),
+                                                    min(args.warmup, 10), args.preamble_steps)
     result["delta_pass"] = bench_delta_pass(ct, torch, config, attention["inputs"]["q"])
     if args.calibration_copy_bytes:
         calibration_copy(ct, torch, args.calibration_copy_bytes)

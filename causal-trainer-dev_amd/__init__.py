@@ -14,7 +14,6 @@ from .efficient_attention import (  # noqa: F401
     efficient_attention,
     prepare_attention_metadata,
     resolve_attention_profile,
-    set_dkv_variant,
     tile_bounds_table,
     validate_attention_profile,
 )

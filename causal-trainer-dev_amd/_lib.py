@@ -20,7 +20,13 @@ CT_WORKSPACE_TOO_SMALL = -3
 CT_LAUNCH_FAILED = -4
 
 ATTN_META_WIDTH = 12
-ABI_VERSION = 2
+ABI_VERSION = 3
+
+# ct_attn_bwd_args.variant (0 = every choice left to the library)
+ATTN_BWD_DKV_NARROW = 1
+ATTN_BWD_DKV_WIDE = 2
+ATTN_BWD_DQ_RECOMPUTE = 0x10
+ATTN_BWD_DQ_FROM_DS = 0x20
 
 
 class CtError(RuntimeError):
@@ -50,7 +56,7 @@ class AttnBwdArgs(Structure):
         ("dq", c_void_p), ("dk", c_void_p), ("dv", c_void_p), ("delta", c_void_p),
         ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("batch", c_int32), ("seq", c_int32), ("q_heads", c_int32), ("kv_heads", c_int32),
-        ("head_dim", c_int32), ("scale", c_float),
+        ("head_dim", c_int32), ("scale", c_float), ("variant", c_int32),
     ]
 
 
@@ -128,13 +134,13 @@ SYMBOLS = {
     "ct_sparse_ce_bwd": (c_int32, [c_void_p, POINTER(SparseCeArgs), c_void_p, c_void_p, c_void_p]),
     "ct_attn_meta_bytes": (c_size_t, [c_int32, c_int32]),
     "ct_attn_bwd_workspace_bytes": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32]),
+    "ct_attn_bwd_workspace_bytes_from_ds": (c_size_t, [c_int32, c_int32, c_int32, c_int32, c_int32, c_int32]),
     "ct_attn_prepare": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_void_p]),
     "ct_attn_block_summary": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32,
                                         c_void_p]),
     "ct_attn_fwd": (c_int32, [c_void_p, POINTER(AttnFwdArgs)]),
     "ct_attn_bwd": (c_int32, [c_void_p, POINTER(AttnBwdArgs)]),
     "ct_attn_delta": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32]),
-    "ct_attn_set_dkv_variant": (c_int32, [c_int32]),
     "ct_cutce_fwd_workspace_bytes": (c_size_t, [POINTER(CutceShape)]),
     "ct_cutce_bwd_workspace_min_bytes": (c_size_t, [POINTER(CutceShape)]),
     "ct_cutce_bwd_workspace_bytes": (c_size_t, [POINTER(CutceShape)]),

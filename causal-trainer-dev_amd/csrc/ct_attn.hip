@@ -1,5 +1,6 @@
 // C ABI of the attention hot path: argument validation and launches.
 #include <atomic>
+#include <algorithm>
 
 #include "ct_attn_bwd_kernels.cuh"
 #include "ct_attn_dkv_wide.cuh"
@@ -99,6 +100,34 @@ __global__ __launch_bounds__(1024) void attn_prepare_kernel(const int* seg, cons
   }
   __threadfence();  // the table and (for long rows) the scratch arrays are re-read through global memory
   __syncthreads();
+
+  // Where the dS blocks of each key block start (kDsOff): exclusive prefix sum of the lengths of
+  // the query-block ranges. Every thread sums a contiguous run of row blocks, the runs are
+  // scanned across the workgroup, and each thread then walks its run again.
+  {
+    __shared__ long long scan_buf[1024];
+    const int per = (nrb + (int)blockDim.x - 1) / (int)blockDim.x;
+    const int lo = min(nrb, (int)threadIdx.x * per), hi = min(nrb, lo + per);
+    auto pairs_of = [&](int rb) {
+      const int* m = mb + rb * kMetaW;
+      return m[kQLast] >= m[kQFirst] ? (long long)(m[kQLast] - m[kQFirst] + 1) : 0ll;
+    };
+    long long local = 0;
+    for (int rb = lo; rb < hi; ++rb) local += pairs_of(rb);
+    scan_buf[threadIdx.x] = local;
+    __syncthreads();
+    for (int off = 1; off < (int)blockDim.x; off <<= 1) {
+      const long long below = (int)threadIdx.x >= off ? scan_buf[threadIdx.x - off] : 0ll;
+      __syncthreads();
+      scan_buf[threadIdx.x] += below;
+      __syncthreads();
+    }
+    long long run = scan_buf[threadIdx.x] - local;
+    for (int rb = lo; rb < hi; ++rb) {
+      mb[rb * kMetaW + kDsOff] = (int)min(run, (long long)INT_MAX);
+      run += pairs_of(rb);
+    }
+  }
 
   // Phase 3: amount of work per tile, for the four schedules, into LDS (the
   // summaries are no longer needed): [0, nrb) query tiles of 1 row block,
@@ -288,6 +317,10 @@ static int validate_shape(const char* fn, int B, int S, int Hq, int Hkv, int D) 
   // (block tables and work lists index 32-position blocks of the whole batch with 32-bit ints)
   if ((long long)B * S > (1ll << 26))
     return fail(CT_UNSUPPORTED, "%s: batch %d x sequence %d exceeds 2^26 positions", fn, B, S);
+  // (the tile ranking of ct_attn_prepare is quadratic in the row blocks of one batch row: rows up to
+  // 2^20 positions are what it is built and tested for)
+  if (S > (1 << 20))
+    return fail(CT_UNSUPPORTED, "%s: sequence %d exceeds 2^20 positions per batch row", fn, S);
   return CT_OK;
 }
 
@@ -304,16 +337,28 @@ static int heads_per_group(int Hq, int Hkv) {
   return g % 4 == 0 ? 4 : (g % 2 == 0 ? 2 : 1);
 }
 
+// Kernels that need more than the default 64 KB of dynamic LDS say so once per kernel and device
+// (the attribute belongs to the loaded code object of that device), not on every launch.
+static int ensure_lds(const char* fn, const void* kernel, size_t bytes, std::atomic<unsigned>& done) {
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 32) device = -1;
+  if (device >= 0 && (done.load(std::memory_order_acquire) >> device & 1u)) return CT_OK;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "%s: %s", fn, hipGetErrorString(e));
+  if (device >= 0) done.fetch_or(1u << device, std::memory_order_release);
+  return CT_OK;
+}
+#define CT_ENSURE_LDS(fn, kernel, bytes)                                                  \
+  do {                                                                                    \
+    static std::atomic<unsigned> done_{0};                                                \
+    int rc_ = ensure_lds(fn, reinterpret_cast<const void*>(kernel), (bytes), done_);      \
+    if (rc_) return rc_;                                                                  \
+  } while (0)
+
 template <int D, int HS>
 static int launch_fwd(hipStream_t stream, const AttnParams& p) {
-  constexpr int PB = kFwdWaves / HS;
   const size_t smem = VkStage<D>::kTotalBytes;
-  {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, HS>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_fwd: %s", hipGetErrorString(e));
-  }
-  (void)PB;
+  CT_ENSURE_LDS("ct_attn_fwd", (&attn_fwd_kernel<D, HS>), smem);
   const int grid = (p.Hq / HS) * kBins;  // (head slice, KV head) groups x work bins
   LaunchScope scope1("attn_fwd_kernel", stream);
   hipLaunchKernelGGL((attn_fwd_kernel<D, HS>), dim3(grid), dim3(kFwdWaves * 64), smem, stream, p);
@@ -329,63 +374,64 @@ static int dispatch_fwd(hipStream_t stream, const AttnParams& p) {
   }
 }
 
+// Workgroups of the persistent dQ kernels: 64 per (head slice, KV head) group, two per compute
+// unit when there are 8 groups; more per group when a pass has fewer groups than that.
+static int dq_grid(const AttnParams& p, int hs) {
+  const int groups = ((p.Hq / p.Hkv) / hs) * p.kvh_count;
+  const int members = groups >= 8 ? 2 * kBins : (2 * kBins * 8 + groups - 1) / groups;
+  return groups * members;
+}
+
 template <int D, int HS>
 static int launch_dq(hipStream_t stream, const AttnParams& p) {
-  constexpr int PB = 4 / HS;
   const size_t smem = 2 * KvStage<D>::kBytes;
-  {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dq_kernel<D, HS>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
-  }
-  (void)PB;
-  // (head slice, KV head) groups x 64 workgroups: two per compute unit when there are 8 groups
-  const int grid = (p.Hq / HS) * kBins * 2;
+  CT_ENSURE_LDS("ct_attn_bwd", (&attn_dq_kernel<D, HS>), smem);
   LaunchScope scope2("attn_dq_kernel", stream);
-  hipLaunchKernelGGL((attn_dq_kernel<D, HS>), dim3(grid), dim3(256), smem, stream, p);
+  hipLaunchKernelGGL((attn_dq_kernel<D, HS>), dim3(dq_grid(p, HS)), dim3(256), smem, stream, p);
   return scope2.done();
 }
 
-// Which dK/dV kernel runs for head dimension 128: 0 the two-wavefronts-per-SIMD one, 1 the wide
-// one (ct_attn_dkv_wide.cuh), -1 (the default) by sequence length: the wide kernel's streams pay
-// off where runs of all-allowed steps are long, which needs long segments; measured 8 % faster at
-// S = 32768 with segments up to the whole row and 3 % slower at S = 4096 with segments of 64 to
-// 4096 positions. Process-wide, set by ct_attn_set_dkv_variant.
-static std::atomic<int> g_dkv_variant{-1};
+template <int D, int HS>
+static int launch_dq_blocks(hipStream_t stream, const AttnParams& p) {
+  const size_t smem = DsStage<D>::kTotalBytes;
+  CT_ENSURE_LDS("ct_attn_bwd", (&attn_dq_blocks_kernel<D, HS>), smem);
+  LaunchScope scope("attn_dq_blocks_kernel", stream);
+  hipLaunchKernelGGL((attn_dq_blocks_kernel<D, HS>), dim3(dq_grid(p, HS)), dim3(kDqbWaves * 64), smem, stream, p);
+  return scope.done();
+}
+
+// Which dK/dV kernel runs for head dimension 128 when the caller leaves the choice open: the wide
+// kernel's streams pay off where runs of all-allowed steps are long, which needs long segments;
+// measured 8 % faster at S = 32768 with segments up to the whole row and 3 % slower at S = 4096
+// with segments of 64 to 4096 positions.
 constexpr int kWideDkvFromSeq = 16384;
 
+// One pass of the dK/dV kernel over the KV heads p.kvh_base ... (all of them unless dS is stored).
 template <int D>
-static int launch_dkv(hipStream_t stream, const AttnParams& p) {
+static int launch_dkv(hipStream_t stream, const AttnParams& p, bool wide) {
   const size_t smem = QdoStage<D>::kTotalBytes;
-  {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dkv_kernel<D>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
-  }
-  int rc = 0;
-  const int grid = p.dkv_max_entries * p.Hkv;  // entries beyond the list's length exit at once
-  bool wide = false;
+  const int grid = p.dkv_max_entries * p.kvh_count;  // entries beyond the list's length exit at once
+  LaunchScope scope3("attn_dkv_kernel", stream);
   if constexpr (D == 128) {
-    const int variant = g_dkv_variant.load(std::memory_order_relaxed);
-    wide = variant == 1 || (variant < 0 && p.S >= kWideDkvFromSeq);
-  }
-  if (wide) {
-    static std::atomic<bool> wide_ready{false};
-    if (!wide_ready.load()) {
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_dkv_wide_kernel),
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)DkvWideLds::kTotalBytes);
-      if (e != hipSuccess) return fail(CT_LAUNCH_FAILED, "ct_attn_bwd: %s", hipGetErrorString(e));
-      wide_ready.store(true);
+    if (wide) {
+      CT_ENSURE_LDS("ct_attn_bwd", &attn_dkv_wide_kernel, DkvWideLds::kTotalBytes);
+      hipLaunchKernelGGL(attn_dkv_wide_kernel, dim3(grid), dim3(128), DkvWideLds::kTotalBytes, stream, p);
+      return scope3.done();
     }
-    LaunchScope scope3("attn_dkv_kernel", stream);
-    hipLaunchKernelGGL(attn_dkv_wide_kernel, dim3(grid), dim3(128), DkvWideLds::kTotalBytes, stream, p);
-    rc = scope3.done();
-  } else {
-    LaunchScope scope3("attn_dkv_kernel", stream);
-    hipLaunchKernelGGL((attn_dkv_kernel<D>), dim3(grid), dim3(256), smem, stream, p);
-    rc = scope3.done();
   }
-  if (rc) return rc;
+  if (p.ds) {
+    CT_ENSURE_LDS("ct_attn_bwd", (&attn_dkv_kernel<D, true>), smem);
+    hipLaunchKernelGGL((attn_dkv_kernel<D, true>), dim3(grid), dim3(256), smem, stream, p);
+  } else {
+    CT_ENSURE_LDS("ct_attn_bwd", (&attn_dkv_kernel<D, false>), smem);
+    hipLaunchKernelGGL((attn_dkv_kernel<D, false>), dim3(grid), dim3(256), smem, stream, p);
+  }
+  return scope3.done();
+}
+
+template <int D>
+static int launch_dkv_reduce(hipStream_t stream, const AttnParams& p) {
+  const int grid = p.dkv_max_entries * p.Hkv;
   LaunchScope scope9("attn_dkv_reduce_kernel", stream);
   hipLaunchKernelGGL((attn_dkv_reduce_kernel<D>), dim3(grid), dim3(256), 4 * 32 * D * 2, stream, p);
   return scope9.done();
@@ -403,14 +449,19 @@ static int launch_delta(hipStream_t stream, const bf16* out, const bf16* dout, f
 }
 
 template <int D>
-static int dispatch_bwd(hipStream_t stream, const AttnParams& p) {
-  // The work list of dK/dV depends on the metadata only: built first, by the launch that also
-  // clears dQ's work counters. dQ computes delta and lse * log2(e) for its rows on the way.
+static int launch_schedule(hipStream_t stream, const AttnParams& p, int kvh_side_by_side) {
   LaunchScope scope7("attn_dkv_schedule_kernel", stream);
   hipLaunchKernelGGL(attn_dkv_schedule_kernel, dim3(1), dim3(1024), 0, stream, p.meta, p.B, p.S,
-                     p.Hkv, p.Hq / p.Hkv, p.dkv_max_entries, p.dkv_max_partials, p.dkv_header,
+                     kvh_side_by_side, p.Hq / p.Hkv, p.dkv_max_entries, p.dkv_max_partials, p.dkv_header,
                      p.dkv_entries, p.dq_counters, kDqCounters);
-  int rc = scope7.done();
+  return scope7.done();
+}
+
+// Recompute form: the work list; dQ per query tile (evaluates S and dP itself and computes delta
+// and -lse / scale for its rows on the way); dK/dV per key tile; the sum of split chunks.
+template <int D>
+static int dispatch_bwd_recompute(hipStream_t stream, const AttnParams& p, bool wide) {
+  int rc = launch_schedule<D>(stream, p, p.Hkv);
   if (rc) return rc;
   switch (heads_per_group(p.Hq, p.Hkv)) {
     case 4: rc = launch_dq<D, 4>(stream, p); break;
@@ -418,30 +469,66 @@ static int dispatch_bwd(hipStream_t stream, const AttnParams& p) {
     default: rc = launch_dq<D, 1>(stream, p); break;
   }
   if (rc) return rc;
-  return launch_dkv<D>(stream, p);
+  rc = launch_dkv<D>(stream, p, wide);
+  if (rc) return rc;
+  return launch_dkv_reduce<D>(stream, p);
+}
+
+// Stored-dS form: row statistics; the work list; then per pass of KV heads the dK/dV kernel, which
+// leaves its dS blocks in the region, and dQ as a product over those blocks; the sum of split chunks.
+template <int D>
+static int dispatch_bwd_blocks(hipStream_t stream, AttnParams p, int kvh_per_pass, bool wide) {
+  {
+    const long tiles = (long)p.B * p.Hq * (p.S / (D == 128 ? 64 : 128));
+    LaunchScope scope("attn_bwd_stats_kernel", stream);
+    hipLaunchKernelGGL((attn_bwd_stats_kernel<D>), dim3((unsigned)(tiles < 8192 ? tiles : 8192)), dim3(256), 0,
+                       stream, p.out, p.dout, p.lse, p.delta, p.lse2, p.B, p.S, p.Hq, exponent_scale(p.scale));
+    int rc = scope.done();
+    if (rc) return rc;
+  }
+  int rc = launch_schedule<D>(stream, p, kvh_per_pass);
+  if (rc) return rc;
+  for (int base = 0; base < p.Hkv; base += kvh_per_pass) {
+    p.kvh_base = base;
+    p.kvh_count = min(kvh_per_pass, p.Hkv - base);
+    rc = launch_dkv<D>(stream, p, wide);
+    if (rc) return rc;
+    switch (heads_per_group(p.Hq, p.Hkv)) {
+      case 4: rc = launch_dq_blocks<D, 4>(stream, p); break;
+      case 2: rc = launch_dq_blocks<D, 2>(stream, p); break;
+      default: rc = launch_dq_blocks<D, 1>(stream, p); break;
+    }
+    if (rc) return rc;
+  }
+  return launch_dkv_reduce<D>(stream, p);
 }
 
 }  // namespace ct
 
 using namespace ct;
 
-extern "C" int32_t ct_attn_set_dkv_variant(int32_t variant) {
-  if (variant < -1 || variant > 1) return fail(CT_INVALID_ARGUMENT, "ct_attn_set_dkv_variant: variant must be -1, 0 or 1");
-  g_dkv_variant.store(variant, std::memory_order_relaxed);
-  return CT_OK;
-}
-
 extern "C" size_t ct_attn_meta_bytes(int32_t batch, int32_t seq) {
   if (batch <= 0 || seq <= 0) return 0;
   return meta_total_ints(batch, seq / 32) * sizeof(int32_t);
 }
 
+static bool bwd_shape_ok(int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads, int32_t head_dim) {
+  return batch > 0 && seq > 0 && q_heads > 0 && kv_heads > 0 && head_dim > 0 && seq % kDkvKeys == 0 &&
+         q_heads % kv_heads == 0;
+}
+
 extern "C" size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t q_heads,
                                              int32_t kv_heads, int32_t head_dim) {
-  if (batch <= 0 || seq <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 ||
-      seq % kDkvKeys != 0)
-    return 0;
-  return dkv_layout(batch, seq, q_heads, kv_heads, head_dim).total;
+  if (!bwd_shape_ok(batch, seq, q_heads, kv_heads, head_dim)) return 0;
+  return bwd_plan(batch, seq, q_heads, kv_heads, head_dim, false, 0, false).total;
+}
+
+extern "C" size_t ct_attn_bwd_workspace_bytes_from_ds(int32_t batch, int32_t seq, int32_t q_heads,
+                                                     int32_t kv_heads, int32_t head_dim,
+                                                     int32_t has_attention_end) {
+  if (!bwd_shape_ok(batch, seq, q_heads, kv_heads, head_dim)) return 0;
+  const BwdPlan plan = bwd_plan(batch, seq, q_heads, kv_heads, head_dim, has_attention_end != 0, 0, true);
+  return plan.spill ? plan.total : 0;
 }
 
 extern "C" int32_t ct_attn_prepare(void* stream, const int32_t* segment_ids,
@@ -572,10 +659,27 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   p.Hq = a->q_heads;
   p.Hkv = a->kv_heads;
   p.scale = round_to_bf16(a->scale);
-  const DkvLayout L = dkv_layout(a->batch, a->seq, a->q_heads, a->kv_heads, a->head_dim);
-  if (a->workspace_bytes < L.total)
+  const int kernel_choice = a->variant & 0xf, path_choice = a->variant & 0xf0;
+  CT_REQUIRE((a->variant & ~0xff) == 0 && kernel_choice <= CT_ATTN_BWD_DKV_WIDE &&
+                 (path_choice == 0 || path_choice == CT_ATTN_BWD_DQ_RECOMPUTE || path_choice == CT_ATTN_BWD_DQ_FROM_DS),
+             "ct_attn_bwd: unknown variant 0x%x", a->variant);
+  // The wide dK/dV kernel does not store dS: asking for it settles the dQ form as well.
+  const bool wide_forced = kernel_choice == CT_ATTN_BWD_DKV_WIDE && a->head_dim == 128;
+  CT_REQUIRE(!(wide_forced && path_choice == CT_ATTN_BWD_DQ_FROM_DS),
+             "ct_attn_bwd: the wide dK/dV kernel has no stored-dS form");
+  const bool allow_blocks = path_choice == CT_ATTN_BWD_DQ_FROM_DS;
+  const BwdPlan plan = bwd_plan(a->batch, a->seq, a->q_heads, a->kv_heads, a->head_dim,
+                                a->attention_end != nullptr, a->workspace_bytes, allow_blocks);
+  if (a->workspace_bytes < plan.total)
     return fail(CT_WORKSPACE_TOO_SMALL, "ct_attn_bwd: workspace %zu < %zu bytes", a->workspace_bytes,
-                L.total);
+                plan.total);
+  if (path_choice == CT_ATTN_BWD_DQ_FROM_DS && !plan.spill)
+    return fail(CT_WORKSPACE_TOO_SMALL,
+                "ct_attn_bwd: the stored-dS form needs %zu bytes of workspace for one KV head, got %zu",
+                plan.L.total + ds_bytes_per_kv_head(a->batch, a->seq, a->q_heads, a->kv_heads,
+                                                    a->attention_end != nullptr),
+                a->workspace_bytes);
+  const DkvLayout& L = plan.L;
   char* ws = static_cast<char*>(a->workspace);
   p.dkv_header = reinterpret_cast<int*>(ws + L.header);
   p.dq_counters = p.dkv_header + 64;
@@ -584,6 +688,16 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   p.lse2 = reinterpret_cast<float*>(ws + L.lse2);
   p.dkv_max_entries = L.max_entries;
   p.dkv_max_partials = L.max_partials;
-  return a->head_dim == 128 ? dispatch_bwd<128>((hipStream_t)stream, p)
-                            : dispatch_bwd<64>((hipStream_t)stream, p);
+  p.kvh_base = 0;
+  p.kvh_count = a->kv_heads;
+  hipStream_t s = (hipStream_t)stream;
+  if (plan.spill) {
+    p.ds = ws + plan.ds;
+    p.ds_row_blocks = plan.row_blocks;
+    return a->head_dim == 128 ? dispatch_bwd_blocks<128>(s, p, plan.kvh_per_pass, false)
+                              : dispatch_bwd_blocks<64>(s, p, plan.kvh_per_pass, false);
+  }
+  const bool wide = a->head_dim == 128 &&
+                    (wide_forced || (kernel_choice == 0 && a->seq >= kWideDkvFromSeq));
+  return a->head_dim == 128 ? dispatch_bwd_recompute<128>(s, p, wide) : dispatch_bwd_recompute<64>(s, p, wide);
 }

@@ -29,12 +29,14 @@ using LeanTrFrags = std::conditional_t<(D / 8 >= 16), TrFragCompact<D / 8, KSlot
                                        TrFragOffsets<D / 8, KSlots::kAccum>>;
 
 // The dK/dV kernels work on unscaled Q K^T and put the softmax scale into the exponent. Any finite
-// scale is legal (the operator only asks for a finite one): a scale of exactly 0 is replaced there
-// by a positive number so small that scale * S vanishes against lse in f32 all the same (dK is
-// still multiplied by the true scale, 0), and a masked pair is marked by the infinity that the
-// scale's sign turns into -inf in the exponent.
-CT_DEVICE float exponent_scale(float scale) { return scale == 0.f ? 1e-30f : scale; }
-CT_DEVICE float masked_score(float scale) { return scale < 0.f ? -kNegInf : kNegInf; }
+// scale is legal (the operator only asks for a finite one): a scale too small for lse / scale to
+// stay finite (|scale| < 1e-30, zero included) is replaced there by 1e-30, for which scale * S
+// vanishes against lse in f32 all the same (dK is still multiplied by the true scale), and a
+// masked pair is marked by the infinity that the sign of the exponent's scale turns into -inf.
+__host__ __device__ inline float exponent_scale(float scale) {
+  return (scale < 1e-30f && scale > -1e-30f) ? 1e-30f : scale;
+}
+CT_DEVICE float masked_score(float scale) { return exponent_scale(scale) < 0.f ? -kNegInf : kNegInf; }
 
 // P = exp2(S log2e - lse2), dS = P (dP - delta) for one 32-key block, in place in s.
 CT_DEVICE void dq_arith(f32x16& s, const f32x16& dp, float lse2, float delta_q) {
@@ -199,16 +201,16 @@ __global__ __launch_bounds__(256, 2) void attn_dq_kernel(AttnParams p) {
   constexpr int PB = 4 / HS;
   const int nrb = p.S / 32;
   const int slices = (p.Hq / p.Hkv) / HS;
-  const int groups = slices * p.Hkv;
+  const int groups = slices * p.kvh_count;
   const int group = blockIdx.x % groups, member = blockIdx.x / groups, members = gridDim.x / groups;
-  const int kvh = group % p.Hkv, slice = group / p.Hkv;
+  const int kvh = p.kvh_base + group % p.kvh_count, slice = group / p.kvh_count;
   const int tpr = bin_tiles_per_row(nrb, PB);
   const int total = p.B * tpr;
   const MetaPtr sched = meta_const(p.sched + query_schedule_offset(nrb, PB));
-  const bool dynamic = groups <= kDqCounters;
+  const bool dynamic = slices * p.Hkv <= kDqCounters;
   for (int pull = member;; pull += members) {
     if (dynamic) {
-      if (threadIdx.x == 0) next_pull = atomicAdd(&p.dq_counters[group], 1);
+      if (threadIdx.x == 0) next_pull = atomicAdd(&p.dq_counters[slice * p.Hkv + kvh], 1);
       __syncthreads();
       pull = uniform(next_pull);
       __syncthreads();
@@ -560,7 +562,17 @@ __global__ __launch_bounds__(256) void attn_dkv_reduce_kernel(AttnParams p) {
   store_rows<D>(dvacc, patch, p.dv + out_off, kv_row_stride);
 }
 
-template <int D>
+// Byte address of the dS block (key block rb with table entries ds_off / q_first, query block qb)
+// of query head `head`, batch row b: wave-uniform.
+CT_DEVICE char* ds_block_address(const AttnParams& p, int head, int b, int ds_off, int q_first, int qb) {
+  const int first_head = p.kvh_base * (p.Hq / p.Hkv);
+  const size_t block = ((size_t)(head - first_head) * p.B + b) * p.ds_row_blocks + (size_t)(ds_off + qb - q_first);
+  return p.ds + block * kDsBlockBytes;
+}
+
+// SPILL: every (key block, query block) step also stores its bf16 dS block to the dS region, for
+// attn_dq_blocks_kernel.
+template <int D, bool SPILL>
 __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   extern __shared__ __align__(16) char smem_raw[];
   const lds_addr lds0 = lds_address_of(smem_raw);
@@ -568,7 +580,7 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
 
   const int l = lane_id(), j = l & 31, half = l >> 5, w = threadIdx.x >> 6;
   const int nrb = p.S / 32;
-  const int kvh = blockIdx.x % p.Hkv, entry = blockIdx.x / p.Hkv;
+  const int kvh = p.kvh_base + blockIdx.x % p.kvh_count, entry = blockIdx.x / p.kvh_count;
   if (entry >= uniform(p.dkv_header[0])) return;
   const int2 work_entry = p.dkv_entries[entry];
   const int tile = uniform(work_entry.x), packed = uniform(work_entry.y);
@@ -590,6 +602,8 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   const int my_min = uniform(meta_const(meta_b)[my_rb * kMetaW + kMinNz]);
   const int my_max = uniform(meta_const(meta_b)[my_rb * kMetaW + kMaxId]);
   const int my_uni = uniform(meta_const(meta_b)[my_rb * kMetaW + kUniform]);
+  const int my_q_first = uniform(meta_const(meta_b)[my_rb * kMetaW + kQFirst]);
+  const int my_ds_off = uniform(meta_const(meta_b)[my_rb * kMetaW + kDsOff]);
 
   const int key = my_rb * 32 + j;
   const int seg_k = p.seg[(size_t)b * p.S + key];
@@ -661,7 +675,8 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
     const int q_min = qb_bounds.min_nz, q_max = qb_bounds.max_id, q_end_max = qb_bounds.end_max,
               q_end_min = qb_bounds.end_min, q_uni = qb_bounds.uniform;
     if (more) qb_bounds = query_block_bounds(meta_b, qb_next);
-    if (blocks_interact(q_min, q_max, q_end_max, my_min, my_max, my_rb * 32)) {
+    const bool visit = blocks_interact(q_min, q_max, q_end_max, my_min, my_max, my_rb * 32);
+    if (visit) {
       f32x16 s, dp;
       if constexpr (D == 128) {
         // (fragment pointers built here from the lane id: held across the loop they would
@@ -716,6 +731,14 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
           dp[r] = pr * (dp[r] + del4[e]);                              // del4 = -delta
         }
       }
+      if constexpr (SPILL) {
+        // The block as the lanes hold it: the two operands of the dK product (8 query rows of one
+        // key each) as two runs of 64 x 16 bytes in lane order, so a store writes 1 KB end to end.
+        char* block = ds_block_address(p, head, b, my_ds_off, my_q_first, qb);
+        const unsigned lane_off = (unsigned)lane_id_here() * 16;
+        store_global16_s<0>(block, lane_off, __builtin_bit_cast(f32x4, pack_acc8(dp, 0)));
+        store_global16_s<1024>(block, lane_off, __builtin_bit_cast(f32x4, pack_acc8(dp, 1)));
+      }
       if constexpr (D == 128) {
         const TrFragOffsets<16, KSlots::kAccum> tp =
             TrFragOffsets<16, KSlots::kAccum>::expand(TrFragCompact<16, KSlots::kAccum>(lds0, lane_id_here()));
@@ -725,7 +748,11 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
         accumulate_keys<D>(CUR * kStage + QdoStage<D>::kQ, to, dp, dkacc);
       }
     }
-    dma_wait_all();
+    // Vector memory operations complete in the order they were issued: the two stores of this
+    // step are the youngest, so waiting for all but two has waited for every copy of the next
+    // stage without waiting for the stores (they are long done one step later).
+    if (SPILL && visit) __builtin_amdgcn_s_waitcnt(0x0F72);
+    else dma_wait_all();
     __syncthreads();
     ++it;
     qb = qb_next;
@@ -767,6 +794,269 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
   store_rows<D>(dkacc, patch, p.dk + out_off, kv_row_stride);
   __builtin_amdgcn_wave_barrier();
   store_rows<D>(dvacc, patch, p.dv + out_off, kv_row_stride);
+}
+
+// ---------------------------------------------------------------------------
+// dQ from stored dS blocks: dQ = scale * sum over visited key blocks of dS K
+// (src/kernels/efficient_attention.py:1046-1048 with the dS of :1040-1045 read back instead of
+// formed again). Same workgroup shape, work pulling and key-tile walk as attn_dq_kernel; a stage
+// holds the K rows of a 64-key tile (shared by the 4 wavefronts) and, per wavefront, the dS blocks
+// of its query block against the tile's two key blocks, copied straight from the dS region. A
+// block is read back as the B operand of dQ^T += K^T dS^T with transposing LDS reads, which is
+// the transposition between the key-stationary kernel that wrote it (lanes along keys) and this
+// query-stationary product (lanes along queries). Bound by the bytes of the blocks it reads.
+// ---------------------------------------------------------------------------
+// Eight wavefronts per workgroup (HS heads x 8 / HS query blocks). A stage: the K rows of one
+// 32-key block (shared by all wavefronts) and, per wavefront, the dS block of its query block
+// against that key block. A dS block sits in LDS as it sits in memory (two runs of 64 x 16 bytes,
+// lane (half, key) order), the second run 64 bytes further than its 1 KB so that the transposing
+// reads of one fragment spread over all banks. Three stages: two key blocks are in flight while
+// one is worked on (the kernel lives on bytes in flight; what bounds them is LDS, and with eight
+// wavefronts per K block four fifths of a stage are dS).
+constexpr int kDqbWaves = 8;
+template <int D>
+struct DsStage {
+  static constexpr int kK = 0;
+  static constexpr int kKBytes = 32 * D * 2;
+  static constexpr int kRun = 1024 + 64;
+  static constexpr int kPatch = 2 * kRun;
+  static constexpr int kDs = kKBytes;  // [wavefront][kPatch]
+  static constexpr int kBytes = kKBytes + kDqbWaves * kPatch;
+  static constexpr int kStages = 3;
+  static constexpr int kTotalBytes =
+      kStages * kBytes > kDqbWaves * 32 * D * 2 ? kStages * kBytes : kDqbWaves * 32 * D * 2;  // >= the store patches
+};
+
+// Transposed-fragment pointers into a dS block: the B operand of dQ^T += K^T dS^T wants, for
+// query slot n = lane % 32, the keys of a k-step in accumulator order (matching the K fragments).
+// The 8-byte piece (key, slots 4 m .. 4 m + 3) is the half (slots & 4) of lane (half = slot >> 4,
+// key)'s 16 bytes in run (slot >> 3) & 1.
+struct DsFragPtrs {
+  lds_addr ptr[2];
+  CT_DEVICE DsFragPtrs(lds_addr base, int l) {
+    const int pp = l & 15, q16 = (l >> 4) & 1, half = l >> 5;
+#pragma unroll
+    for (int second = 0; second < 2; ++second) {
+      const int key = 4 * half + 8 * second + (pp >> 2);
+      const int run = (pp & 3) >> 1, piece = pp & 1;
+      ptr[second] = base + (run * (1024 + 64) + q16 * 512 + key * 16 + piece * 8);
+    }
+  }
+  // keys 16 ks .. 16 ks + 15 of the block at byte offset `off`
+  CT_DEVICE bf16x8 load(int off, int ks) const {
+    const bf16x4_vs lo = lds_load_tr(ptr[0] + (off + ks * 256));
+    const bf16x4_vs hi = lds_load_tr(ptr[1] + (off + ks * 256));
+    bf16x8 out;
+    out[0] = lo[0]; out[1] = lo[1]; out[2] = lo[2]; out[3] = lo[3];
+    out[4] = hi[0]; out[5] = hi[1]; out[6] = hi[2]; out[7] = hi[3];
+    return out;
+  }
+};
+
+// What the walk needs to know about a 32-key block (scalar loads).
+struct DsKeyBlockInfo {
+  int k_min, k_max, q_first, ds_off;
+};
+CT_DEVICE DsKeyBlockInfo ds_key_block_info(const int* meta_b, int rbk) {
+  const MetaPtr m = meta_const(meta_b + rbk * kMetaW);
+  DsKeyBlockInfo info;
+  info.k_min = m[kMinNz];
+  info.k_max = m[kMaxId];
+  info.q_first = m[kQFirst];
+  info.ds_off = m[kDsOff];
+  return info;
+}
+
+// store_rows_t for an accumulator whose lane j holds the query row ds_slot_row(j) of the block.
+template <int D>
+CT_DEVICE void store_slot_rows_t(const f32x16* acc, float row_scale, lds_addr patch, bf16* gbase,
+                                 size_t row_stride) {
+  constexpr int CPR = D / 8;
+  int l = lane_id();
+  asm volatile("" : "+v"(l));
+  const int row_of_lane = ds_slot_row(l & 31), half = l >> 5;
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db) {
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      const int d0 = db * 32 + 8 * qd + 4 * half;
+      bf16x4 pk;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pk[e] = (bf16)(acc[db][4 * qd + e] * row_scale);
+      lds_store<bf16x4>(patch + tile_byte_offset<CPR>(row_of_lane, d0 >> 3) + (d0 & 4) * 2, pk);
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int n = 0; n < 32 * CPR / 64; ++n) {
+    const int e = l + 64 * n;
+    const int row = e / CPR, c = e % CPR;
+    const u32x4 val = lds_load<u32x4>(patch + tile_byte_offset<CPR>(row, c));
+    store_global16(gbase + (size_t)row * row_stride + c * 8, val);
+  }
+}
+
+// s_waitcnt vmcnt(n) for a wave-uniform n that is one of the few values the walk produces.
+CT_DEVICE void wait_all_copies_but(int n) {
+  if (n == 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+  else if (n == 1) __builtin_amdgcn_s_waitcnt(0x0F71);
+  else if (n == 2) __builtin_amdgcn_s_waitcnt(0x0F72);
+  else __builtin_amdgcn_s_waitcnt(0x0F73);
+}
+
+template <int D, int HS>
+CT_DEVICE void attn_dq_blocks_item(const AttnParams& p, int b, int kvh, int slice, int qt, const lds_addr lds0,
+                                   const TileDma<32, D / 8, (D == 128 ? 512 : 256)>& kdma,
+                                   const DsFragPtrs& frags, const TrFragOffsets<D / 8, KSlots::kAccum>& tp) {
+  constexpr int PB = kDqbWaves / HS;
+  constexpr int kStage = DsStage<D>::kBytes;
+  const int nrb = p.S / 32;
+  const int g = p.Hq / p.Hkv;
+  const int w = uniform(threadIdx.x >> 6);
+  const int h = kvh * g + slice * HS + (w % HS);
+  int rb = qt * PB + (w / HS);
+  const bool active = rb < nrb;
+  if (!active) rb = nrb - 1;
+  const int* meta_b = p.meta + (size_t)b * nrb * kMetaW;
+  QueryBlockBounds mine = query_block_bounds(meta_b, rb);
+  if (!active) mine.min_nz = 0;  // interacts with nothing
+  int first_tile = INT_MAX, last_tile = -1;  // 64-key tiles, as the table has them
+#pragma unroll
+  for (int i = 0; i < PB; ++i) {
+    if (qt * PB + i >= nrb) break;
+    const MetaPtr m = meta_const(meta_b + (qt * PB + i) * kMetaW);
+    first_tile = min(first_tile, uniform(m[kKvFirst]));
+    last_tile = max(last_tile, uniform(m[kKvLast]));
+  }
+  // the walk is in 32-key blocks (a tile without keys is the pair INT_MAX / -1: converted only
+  // when there is a range, and clamped to the row so that no table entry can lead outside it)
+  const bool any = first_tile <= last_tile && first_tile >= 0 && last_tile < nrb / 2;
+  const int first = any ? 2 * first_tile : 0;
+  const int last = any ? 2 * last_tile + 1 : -1;
+  const char* kbase = reinterpret_cast<const char*>(p.k + ((size_t)b * p.S * p.Hkv + kvh) * D);
+  const size_t kv_row_bytes = (size_t)p.Hkv * D * 2;
+  const unsigned ds_lane_off = (unsigned)lane_id_here() * 16;
+  const int my_ds = DsStage<D>::kDs + w * DsStage<D>::kPatch;  // this wavefront's block inside a stage
+  // copies of the K rows this wavefront issues per stage (head dimension 64: 256 threads cover the block)
+  const bool copies_k = D == 128 || w < 4;
+
+  f32x16 dqacc[D / 32];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db) dqacc[db] = zero16();
+
+  auto visits = [&](const DsKeyBlockInfo& info, int rbk) {
+    return blocks_interact(mine.min_nz, mine.max_id, mine.end_max, uniform(info.k_min), uniform(info.k_max),
+                           rbk * 32);
+  };
+  // K rows of key block rbk (all wavefronts) and this wavefront's dS block against it; returns the
+  // number of copy instructions this wavefront issued
+  auto issue = [&](int rbk, const DsKeyBlockInfo& info, lds_addr stage) {
+    int issued = 0;
+    if (copies_k) {
+      kdma.issue(kbase + (size_t)rbk * 32 * kv_row_bytes, stage + DsStage<D>::kK);
+      issued = 1;
+    }
+    if (visits(info, rbk)) {
+      const char* block = ds_block_address(p, h, b, uniform(info.ds_off), uniform(info.q_first), rb);
+      dma16_s(block, ds_lane_off, stage + my_ds);
+      dma16_s(block + 1024, ds_lane_off, stage + (my_ds + DsStage<D>::kRun));
+      issued += 2;
+    }
+    return issued;
+  };
+
+  // info[i]: key block t + i; stage of key block t + i is (stage of t + i) mod 3
+  int t = first;
+  DsKeyBlockInfo cur = {}, next = {}, after = {};
+  int pending = 0;  // copy instructions of the youngest key block in flight
+  if (t <= last) {
+    cur = ds_key_block_info(meta_b, t);
+    issue(t, cur, lds0);
+    if (t + 1 <= last) {
+      next = ds_key_block_info(meta_b, t + 1);
+      pending = issue(t + 1, next, lds0 + kStage);
+      if (t + 2 <= last) after = ds_key_block_info(meta_b, t + 2);
+    }
+  }
+  wait_all_copies_but(pending);
+  __syncthreads();
+
+  auto step = [&](auto stage_tag) {
+    constexpr int CUR = decltype(stage_tag)::value;
+    constexpr int kFill = (CUR + 2) % 3;  // last read one step ago: every wavefront is past that barrier
+    DsKeyBlockInfo later = after;
+    pending = 0;
+    if (t + 2 <= last) {
+      pending = issue(t + 2, after, lds0 + kFill * kStage);
+      if (t + 3 <= last) later = ds_key_block_info(meta_b, t + 3);
+    }
+    if (visits(cur, t)) {
+      constexpr int ds_off = CUR * kStage;  // + my_ds, inside the pointers
+      constexpr int k_off = CUR * kStage + DsStage<D>::kK;
+      const bf16x8 ds0 = frags.load(ds_off, 0), ds1 = frags.load(ds_off, 1);
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db) dqacc[db] = mfma32(tp.load(k_off, 0, db), ds0, dqacc[db]);
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db) dqacc[db] = mfma32(tp.load(k_off, 1, db), ds1, dqacc[db]);
+    }
+    // Copies complete in the order they were issued: all but the ones just issued means key
+    // block t + 1 has landed.
+    wait_all_copies_but(pending);
+    __syncthreads();
+    cur = next;
+    next = after;
+    after = later;
+    ++t;
+  };
+  while (t <= last) {
+    step(std::integral_constant<int, 0>{});
+    if (t > last) break;
+    step(std::integral_constant<int, 1>{});
+    if (t > last) break;
+    step(std::integral_constant<int, 2>{});
+  }
+
+  if (active) {
+    const lds_addr patch = lds0 + w * 32 * D * 2;
+    bf16* gbase = p.dq + (((size_t)b * p.S + rb * 32) * p.Hq + h) * D;
+    store_slot_rows_t<D>(dqacc, p.scale, patch, gbase, (size_t)p.Hq * D);
+  }
+  // the store patches overlap the stages of the next item
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __syncthreads();
+}
+
+template <int D, int HS>
+__global__ __launch_bounds__(kDqbWaves * 64, 2) void attn_dq_blocks_kernel(AttnParams p) {
+  extern __shared__ __align__(16) char smem_raw[];
+  const lds_addr lds0 = lds_address_of(smem_raw);
+  __shared__ int next_pull;
+  constexpr int PB = kDqbWaves / HS;
+  const int nrb = p.S / 32;
+  const int slices = (p.Hq / p.Hkv) / HS;
+  const int groups = slices * p.kvh_count;
+  const int group = blockIdx.x % groups, member = blockIdx.x / groups, members = gridDim.x / groups;
+  const int kvh = p.kvh_base + group % p.kvh_count, slice = group / p.kvh_count;
+  const int tpr = bin_tiles_per_row(nrb, PB);
+  const int total = p.B * tpr;
+  const MetaPtr sched = meta_const(p.sched + query_schedule_offset(nrb, PB));
+  const bool dynamic = slices * p.Hkv <= kDqCounters;
+  const TileDma<32, D / 8, (D == 128 ? 512 : 256)> kdma((size_t)p.Hkv * D * 2);
+  const int w = threadIdx.x >> 6;
+  const DsFragPtrs frags(lds0 + (DsStage<D>::kDs + w * DsStage<D>::kPatch), lane_id());
+  const TrFragOffsets<D / 8, KSlots::kAccum> tp(lds0);
+  for (int pull = member;; pull += members) {
+    if (dynamic) {
+      if (threadIdx.x == 0) next_pull = atomicAdd(&p.dq_counters[slice * p.Hkv + kvh], 1);
+      __syncthreads();
+      pull = uniform(next_pull);
+      __syncthreads();
+    }
+    if (pull >= total) break;
+    const int b = pull % p.B, rank = pull / p.B;
+    const int qt = uniform(sched[(size_t)b * schedule_ints(nrb) + rank]);
+    attn_dq_blocks_item<D, HS>(p, b, kvh, slice, qt, lds0, kdma, frags, tp);
+  }
 }
 
 }  // namespace ct

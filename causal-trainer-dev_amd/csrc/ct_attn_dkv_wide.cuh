@@ -157,7 +157,7 @@ __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
   const int l = lane_id(), j = l & 31, half = l >> 5, w = uniform(threadIdx.x >> 6);
   const int nrb = p.S / 32;
-  const int kvh = blockIdx.x % p.Hkv, entry = blockIdx.x / p.Hkv;
+  const int kvh = p.kvh_base + blockIdx.x % p.kvh_count, entry = blockIdx.x / p.kvh_count;
   if (entry >= uniform(p.dkv_header[0])) return;
   const int2 work_entry = p.dkv_entries[entry];
   const int tile = uniform(work_entry.x), packed = uniform(work_entry.y);

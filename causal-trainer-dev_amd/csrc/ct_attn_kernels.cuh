@@ -57,6 +57,11 @@ struct AttnParams {
   int* dq_counters;  // kDqCounters ints, zeroed by the work-list kernel of the same call
   float* dkv_partials;
   int dkv_max_entries, dkv_max_partials;
+  // KV heads [kvh_base, kvh_base + kvh_count) are what a backward launch works on (all of them
+  // unless dS goes through the workspace, which bounds that region by running the heads in passes)
+  int kvh_base, kvh_count;
+  char* ds;              // dS region of the pass, null when dQ recomputes S and dP
+  size_t ds_row_blocks;  // dS blocks reserved per (query head, batch row)
 };
 
 // ---------------------------------------------------------------------------
@@ -763,6 +768,53 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const bf16* out, const 
 #pragma unroll
       for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
       if (chunk < chunks && chunk % LPR == 0) delta[chunk / LPR] = acc;
+    }
+  }
+}
+
+// The same pass in the form the backward needs when its dK/dV kernel runs first: -delta and
+// -lse / scale, both head-major [B, Hq, S] (the dK/dV kernels add them to their dP and S blocks).
+// A workgroup takes 4 x (256 / lanes per row) consecutive positions of one head; consecutive
+// workgroups take the heads of the same positions, so the rows in flight at a time are one
+// contiguous stretch of `out` and `dout`.
+template <int D>
+__global__ __launch_bounds__(256) void attn_bwd_stats_kernel(const bf16* out, const bf16* dout,
+                                                             const float* lse, float* neg_delta,
+                                                             float* neg_lse_scaled, int B, int S,
+                                                             int Hq, float exponent_scale) {
+  constexpr int LPR = D / 8;          // lanes per row
+  constexpr int RPP = 256 / LPR;      // rows per pass of the workgroup
+  constexpr int kUnroll = 4;
+  constexpr int kTile = kUnroll * RPP;  // 64 (D = 128) or 128 (D = 64) positions: divides S
+  const int tiles_per_row = S / kTile;
+  const long tiles = (long)B * tiles_per_row * Hq;
+  const int r0 = threadIdx.x / LPR, chunk = threadIdx.x % LPR;
+  for (long tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const int h = (int)(tile % Hq);
+    const long rest = tile / Hq;
+    const int st = (int)(rest % tiles_per_row), b = (int)(rest / tiles_per_row);
+    u32x4 a[kUnroll], g[kUnroll];
+    float row_lse[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const size_t row = ((size_t)b * S + st * kTile + r0 + k * RPP) * Hq + h;
+      a[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(out) + row * LPR + chunk);
+      g[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(dout) + row * LPR + chunk);
+      row_lse[k] = lse[row];
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+      const bf16x8 av = as_bf16x8(a[k]), gv = as_bf16x8(g[k]);
+      float acc = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc += (float)av[e] * (float)gv[e];
+#pragma unroll
+      for (int off = LPR / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+      if (chunk == 0) {
+        const size_t stat = ((size_t)b * Hq + h) * S + st * kTile + r0 + k * RPP;
+        neg_delta[stat] = -acc;
+        neg_lse_scaled[stat] = -row_lse[k] / exponent_scale;
+      }
     }
   }
 }

@@ -12,6 +12,10 @@
 //   [6] kv_last  last such tile (INT_MAX / -1 pair when there is none)
 //   [7] q_first  first 32-row query block that has to visit this block (as keys)
 //   [8] q_last   last such block
+//   [9] ds_off   number of (key block, visiting query block) pairs of the key blocks before this
+//                one in the same batch row, i.e. the exclusive prefix sum of
+//                max(0, q_last - q_first + 1): where the dS blocks of this key block start in
+//                the backward's dS region (saturates at INT_MAX)
 // [0], [1] and the "has to visit" predicate follow the reference's block
 // summaries and skip test (src/kernels/efficient_attention.py:313-323,
 // :377-412): two blocks interact iff both hold a nonzero id, their id ranges
@@ -44,6 +48,7 @@ enum MetaSlot {
   kKvLast = 6,
   kQFirst = 7,
   kQLast = 8,
+  kDsOff = 9,
 };
 
 // ints of schedule data per batch row (nrb + nrb/2 + nrb/4 + nrb/4, then ceil(nrb/8) <= nrb/4)
@@ -135,21 +140,96 @@ struct DkvLayout {
 };
 
 // Sum over tiles of the chunk count is at most tiles + total_items / target and the
-// target is at least total_items * kv_heads / kDkvSlots.
-__host__ inline DkvLayout dkv_layout(int B, int S, int Hq, int Hkv, int D) {
+// target is at least total_items * (KV heads that run side by side) / kDkvSlots.
+__host__ inline DkvLayout dkv_layout(int B, int S, int Hq, int Hkv, int D, int kvh_per_pass) {
   DkvLayout L;
   const int tiles = B * (S / kDkvKeys);
-  const int extra = (kDkvSlots + Hkv - 1) / Hkv + 1;
+  const int extra = (kDkvSlots + kvh_per_pass - 1) / kvh_per_pass + 1;
   L.max_entries = tiles + extra;
   L.max_partials = min(2 * extra, L.max_entries);
   auto up = [](size_t v) { return (v + 255) / 256 * 256; };
   L.header = 0;  // 64 ints of dK/dV list header, then kDqCounters work counters of the dQ kernel
   L.entries = (64 + kDqCounters) * sizeof(int);
-  // lse * log2(e), head-major [B, Hq, S] (the caller's delta scratch holds delta the same way)
+  // -lse / scale, head-major [B, Hq, S] (the caller's delta scratch holds -delta the same way)
   L.lse2 = L.entries + up((size_t)L.max_entries * 2 * sizeof(int));
   L.partials = L.lse2 + up((size_t)B * S * Hq * sizeof(float));
-  L.total = L.partials + (size_t)L.max_partials * Hkv * 2 * kDkvKeys * D * sizeof(float);
+  L.total = up(L.partials + (size_t)L.max_partials * Hkv * 2 * kDkvKeys * D * sizeof(float));
   return L;
+}
+
+// ---------------------------------------------------------------------------
+// dS region (backward workspace, after the work list).
+//
+// The dK/dV kernel forms dS = P (dP - delta) for every (key block, visiting query block) pair
+// anyway (its dK product consumes it as bf16). When the workspace has room it also stores these
+// 32 x 32 bf16 blocks, and dQ = scale * dS K becomes a block-sparse product over stored blocks
+// instead of a second evaluation of S and dP: 2 D flops per pair instead of 6 D, paid for with
+// 2 bytes written and 2 bytes read per visited pair.
+// Block (key block rb, query block qb) of query head h, batch row b sits at block index
+//   ((h - first head of the pass) * B + b) * row_blocks + ds_off[rb] + qb - q_first[rb]
+// (kDsBlockBytes each); row_blocks bounds the pairs of one batch row: nrb (nrb + 1) / 2 for plain
+// causal masks (a key block is visited by query blocks at or after it), nrb^2 with visible ends.
+// A block is stored as the dK/dV kernel's lanes hold it: two runs of 64 x 16 bytes; run t, lane
+// (half, key j) holds key j's dS against the 8 query slots 16 half + 8 t + e, and slot s stands
+// for query row 16 ((s >> 3) & 1) + 4 (s >> 4) + (s & 3) + 8 ((s >> 2) & 1) of the block.
+// KV heads are processed in passes of kvh_per_pass heads so that the region stays bounded.
+// ---------------------------------------------------------------------------
+constexpr int kDsBlockBytes = 32 * 32 * 2;
+constexpr size_t kDsRegionDefaultCap = (size_t)16 << 30;  // what ct_attn_bwd_workspace_bytes asks for at most
+constexpr size_t kDsRegionHardCap = (size_t)64 << 30;
+
+CT_DEVICE int ds_slot_row(int s) { return 16 * ((s >> 3) & 1) + 4 * (s >> 4) + (s & 3) + 8 * ((s >> 2) & 1); }
+
+__host__ inline size_t ds_row_blocks(int S, bool has_end) {
+  const size_t nrb = (size_t)S / 32;
+  return has_end ? nrb * nrb : nrb * (nrb + 1) / 2;
+}
+// bytes of dS blocks of one KV head's query heads
+__host__ inline size_t ds_bytes_per_kv_head(int B, int S, int Hq, int Hkv, bool has_end) {
+  return (size_t)(Hq / Hkv) * B * ds_row_blocks(S, has_end) * kDsBlockBytes;
+}
+
+struct BwdPlan {
+  DkvLayout L;
+  bool spill;         // dS goes through the region, dQ from stored blocks
+  int kvh_per_pass;   // KV heads per pass (spill) or all of them
+  size_t ds, ds_bytes, row_blocks, total;
+};
+
+// The plan for a workspace of `bytes` (bytes == 0: the recommended size, dS region capped at
+// kDsRegionDefaultCap but never below one KV head; a KV head beyond kDsRegionHardCap, or
+// allow_spill == false: no region).
+__host__ inline BwdPlan bwd_plan(int B, int S, int Hq, int Hkv, int D, bool has_end, size_t bytes,
+                                 bool allow_spill) {
+  BwdPlan plan;
+  const size_t per_kvh = ds_bytes_per_kv_head(B, S, Hq, Hkv, has_end);
+  plan.row_blocks = ds_row_blocks(S, has_end);
+  plan.spill = false;
+  plan.kvh_per_pass = Hkv;
+  plan.L = dkv_layout(B, S, Hq, Hkv, D, Hkv);
+  plan.ds = plan.L.total;
+  plan.ds_bytes = 0;
+  plan.total = plan.L.total;
+  // (block indices are 32-bit in the kernels' scalar arithmetic before the final widening)
+  const bool indexable = (size_t)(Hq / Hkv) * B * plan.row_blocks < ((size_t)1 << 31);
+  if (!allow_spill || per_kvh > kDsRegionHardCap || !indexable) return plan;
+  for (int kpp = Hkv; kpp >= 1; --kpp) {
+    const DkvLayout L = dkv_layout(B, S, Hq, Hkv, D, kpp);
+    const size_t region = per_kvh * kpp;
+    bool fits;
+    if (bytes == 0) fits = region <= kDsRegionDefaultCap || kpp == 1;
+    else fits = L.total + region <= bytes;
+    if (fits && (size_t)(Hq / Hkv) * kpp * B * plan.row_blocks < ((size_t)1 << 31)) {
+      plan.spill = true;
+      plan.kvh_per_pass = kpp;
+      plan.L = L;
+      plan.ds = L.total;
+      plan.ds_bytes = region;
+      plan.total = L.total + region;
+      return plan;
+    }
+  }
+  return plan;
 }
 
 struct KeyTileBounds {

@@ -55,4 +55,4 @@ extern "C" void ct_set_launch_hook(ct_launch_hook hook, void* user) {
 
 extern "C" const char* ct_last_error(void) { return ct::g_error; }
 
-extern "C" int32_t ct_abi_version(void) { return 2; }
+extern "C" int32_t ct_abi_version(void) { return 3; }

@@ -179,13 +179,28 @@ def _attn_forward(query, key, value, metadata, scale):
     return out, lse
 
 
-def _attn_backward(query, key, value, metadata, out, lse, dout, scale, with_delta=False):
+_DKV_KERNELS = {None: 0, "narrow": _lib.ATTN_BWD_DKV_NARROW, "wide": _lib.ATTN_BWD_DKV_WIDE}
+_DQ_FORMS = {None: 0, "recompute": _lib.ATTN_BWD_DQ_RECOMPUTE, "from_ds": _lib.ATTN_BWD_DQ_FROM_DS}
+
+
+def _attn_backward(query, key, value, metadata, out, lse, dout, scale, with_delta=False, dkv_kernel=None,
+                   dq_form=None, workspace_bytes=None):
     batch, sequence, q_heads, head_dim = query.shape
+    lib = _lib.load()
     dq = torch.empty_like(query)
     dk = torch.empty_like(key)
     dv = torch.empty_like(value)
     delta = torch.empty_like(lse)
-    workspace_bytes = int(_lib.load().ct_attn_bwd_workspace_bytes(batch, sequence, query.shape[2], key.shape[2], head_dim))
+    shape = (batch, sequence, query.shape[2], key.shape[2], head_dim)
+    if workspace_bytes is None:
+        if dq_form == "from_ds":
+            workspace_bytes = int(lib.ct_attn_bwd_workspace_bytes_from_ds(
+                *shape, int(metadata.attention_end is not None)))
+            if workspace_bytes == 0:
+                raise ValueError("dq_form='from_ds' is not available for this shape (dS blocks of one KV head "
+                                 "exceed 64 GiB)")
+        else:
+            workspace_bytes = int(lib.ct_attn_bwd_workspace_bytes(*shape))
     workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=query.device)
     args = _lib.AttnBwdArgs(
         q=query.data_ptr(), k=key.data_ptr(), v=value.data_ptr(),
@@ -196,10 +211,10 @@ def _attn_backward(query, key, value, metadata, out, lse, dout, scale, with_delt
         dq=dq.data_ptr(), dk=dk.data_ptr(), dv=dv.data_ptr(), delta=delta.data_ptr(),
         workspace=workspace.data_ptr(), workspace_bytes=workspace_bytes,
         batch=batch, seq=sequence, q_heads=q_heads, kv_heads=key.shape[2], head_dim=head_dim,
-        scale=scale,
+        scale=scale, variant=_DKV_KERNELS[dkv_kernel] | _DQ_FORMS[dq_form],
     )
     with torch.cuda.device(query.device):
-        _lib.check(_lib.load().ct_attn_bwd(_lib.current_stream(), args))
+        _lib.check(lib.ct_attn_bwd(_lib.current_stream(), args))
     if with_delta:
         return dq, dk, dv, delta.view(batch, q_heads, sequence)
     return dq, dk, dv
@@ -272,19 +287,20 @@ def attention_forward_with_lse(query, key, value, metadata, *, scale=None):
     return _attn_forward(query.contiguous(), key.contiguous(), value.contiguous(), metadata, resolved)
 
 
-def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=None, with_delta=False):
+def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=None, with_delta=False,
+                       dkv_kernel=None, dq_form=None, workspace_bytes=None):
     """Backward only, from the saved residuals: returns ``(dq, dk, dv)``; with ``with_delta`` also the
-    scratch ``delta = rowsum(out * dout)`` as the kernels leave it, head-major ``[B, Hq, S]``."""
+    scratch ``-delta = -rowsum(out * dout)`` as the kernels leave it, head-major ``[B, Hq, S]``.
+
+    ``dkv_kernel`` (``"narrow"`` / ``"wide"``) and ``dq_form`` (``"recompute"`` / ``"from_ds"``) pin a
+    kernel or a form of the backward for this call (``ct_attn_bwd_args.variant``); ``None`` leaves
+    the choice to the library, which is what training code does (dQ recomputes; the dK/dV kernel goes
+    by sequence length). ``workspace_bytes`` overrides the size of the scratch buffer (default: what
+    the library asks for the chosen form)."""
 
     resolved = default_attention_scale(query.shape[-1]) if scale is None else float(scale)
-    return _attn_backward(query, key, value, metadata, out, lse, dout.contiguous(), resolved, with_delta)
-
-
-def set_dkv_variant(variant: int) -> None:
-    """Choose the dK/dV kernel of the backward for head dimension 128, process-wide: 0 two wavefronts
-    per SIMD, 1 the wide one (one wavefront per SIMD, 64 keys), -1 (the default) by sequence length."""
-
-    _lib.check(_lib.load().ct_attn_set_dkv_variant(int(variant)))
+    return _attn_backward(query, key, value, metadata, out, lse, dout.contiguous(), resolved, with_delta,
+                          dkv_kernel, dq_form, workspace_bytes)
 
 
 __all__ = [
@@ -296,7 +312,6 @@ __all__ = [
     "efficient_attention",
     "prepare_attention_metadata",
     "resolve_attention_profile",
-    "set_dkv_variant",
     "tile_bounds_table",
     "validate_attention_profile",
 ]

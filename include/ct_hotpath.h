@@ -65,7 +65,8 @@ void ct_set_launch_hook(ct_launch_hook hook, void* user);
  * tile-bounds buffer; the table is followed by work-sorted tile schedules. */
 #define CT_ATTN_META_WIDTH 12
 
-/* Bytes of the tile-bounds buffer (table + schedules) for [batch, seq] segment ids. */
+/* Bytes of the tile-bounds buffer for [batch, seq] segment ids: the table, the work-sorted
+ * schedules and work bins, and for very long rows a scratch tail that ct_attn_prepare works in. */
 size_t ct_attn_meta_bytes(int32_t batch, int32_t seq);
 
 /*
@@ -127,6 +128,24 @@ typedef struct ct_attn_fwd_args {
  */
 int32_t ct_attn_fwd(void* stream, const ct_attn_fwd_args* args);
 
+/* ct_attn_bwd_args.variant: 0 leaves every choice to the library (what a trainer passes). The
+ * other values pin a kernel or a form of the backward, for tests and measurements; they are
+ * per call, nothing is process-wide. Low 4 bits, the dK/dV kernel at head dimension 128:
+ * NARROW = two wavefronts per SIMD with 32 keys each, WIDE = one wavefront per SIMD with 64
+ * keys, the (dK, dV) sums in the accumulation registers and each step one generated
+ * instruction stream (left open: WIDE from 16384 positions on, NARROW below). Bits 4-7, how dQ
+ * is formed: RECOMPUTE (also what 0 means) = a query-stationary kernel evaluates S and dP a
+ * second time (the reference's _local_attention_dq, src/kernels/efficient_attention.py:985-1267);
+ * FROM_DS = the dK/dV kernel (NARROW) stores its bf16 dS blocks in the workspace and dQ is the
+ * product of those blocks with K: 14 D instead of 18 D executed flops per pair for 4 bytes of
+ * HBM traffic per pair and head; measured at par with RECOMPUTE on packed 4096-token rows and
+ * slower on long rows, hence not the default; needs ct_attn_bwd_workspace_bytes_from_ds. All
+ * give the same results within the operator's tolerances (not bitwise: summation orders differ). */
+#define CT_ATTN_BWD_DKV_NARROW 1
+#define CT_ATTN_BWD_DKV_WIDE 2
+#define CT_ATTN_BWD_DQ_RECOMPUTE 0x10
+#define CT_ATTN_BWD_DQ_FROM_DS 0x20
+
 typedef struct ct_attn_bwd_args {
   const uint16_t* q;
   const uint16_t* k;
@@ -145,41 +164,45 @@ typedef struct ct_attn_bwd_args {
   size_t workspace_bytes;
   int32_t batch, seq, q_heads, kv_heads, head_dim;
   float scale;
+  int32_t variant;              /* 0, or CT_ATTN_BWD_* values or-ed together */
 } ct_attn_bwd_args;
 
-/* Bytes of scratch ct_attn_bwd needs: the dK/dV work list (key tiles whose
- * list of visiting query blocks is long are cut into chunks that run as
- * separate workgroups) and the f32 partial sums of such chunks. 0 for an
- * unsupported shape. No reference counterpart (the reference's dK/dV kernel
- * accumulates in its f32 output window, src/kernels/efficient_attention.py:1545-1549). */
+/* Bytes of scratch ct_attn_bwd needs: the dK/dV work list (key tiles whose list of visiting
+ * query blocks is long are cut into chunks that run as separate workgroups), the f32 partial
+ * sums of such chunks and the row statistics. 0 for an unsupported shape. No reference
+ * counterpart (the reference's dK/dV kernel accumulates in its f32 output window,
+ * src/kernels/efficient_attention.py:1545-1549). */
 size_t ct_attn_bwd_workspace_bytes(int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads,
                                    int32_t head_dim);
 
+/* Bytes of scratch for variant CT_ATTN_BWD_DQ_FROM_DS: the above plus the dS region, 2 KB per
+ * (32-key block, visiting 32-row query block, query head), reserved for the worst case of the
+ * mask family (causal: S/32 (S/32 + 1) / 2 blocks per batch row and head; with attention_end:
+ * (S/32)^2), for all KV heads if that is at most 16 GiB, else for as many KV heads as fit (the
+ * backward then runs its kernels in passes over the KV heads), never less than one KV head; 0
+ * if one KV head alone exceeds 64 GiB (that form is then unavailable). Any workspace between
+ * one KV head's worth and this is used for as many KV heads per pass as it holds. */
+size_t ct_attn_bwd_workspace_bytes_from_ds(int32_t batch, int32_t seq, int32_t q_heads, int32_t kv_heads,
+                                           int32_t head_dim, int32_t has_attention_end);
+
 /*
- * dq, dk, dv from the saved (q, k, v, out, lse) and dout. Four launches:
- * the dK/dV work list; dq per query tile, which also computes
- * delta = rowsum(out * dout) for its rows; dk/dv per key tile; the sum of the
- * chunks of split key tiles (in a fixed order, so the result is
- * deterministic).
+ * dq, dk, dv from the saved (q, k, v, out, lse) and dout. Four launches: the dK/dV work list;
+ * dq per query tile, which also computes the row statistics (-delta = -rowsum(out * dout) and
+ * -lse / scale) for its rows; dk/dv per key tile; the sum of the chunks of split key tiles (in
+ * a fixed order, so the result is deterministic). With CT_ATTN_BWD_DQ_FROM_DS: the row
+ * statistics as a pass of their own, the work list, then per pass of KV heads dk/dv (which
+ * stores its dS blocks) and dq as the product of those blocks with K, and the sum.
  * Replaces: delta at src/kernels/efficient_attention.py:1735-1738,
  * _local_attention_dq (:985-1267), _local_attention_dkv (:1270-1602) and the
  * f32 -> bf16 cast at :1774.
  */
 int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* args);
 
-/* The delta pass as a pass of its own (ct_attn_bwd computes delta inside its dQ kernel; this
- * entry exists so that the HBM-bound pass can be measured and tested by itself). */
+/* The delta pass as a pass of its own, delta[row] = rowsum(out * dout) in row order (the
+ * backward forms it in the private layout its kernels want; this entry exists so that the
+ * HBM-bound pass can be measured and tested by itself). */
 int32_t ct_attn_delta(void* stream, const uint16_t* out, const uint16_t* dout,
                       float* delta, int64_t rows, int32_t head_dim);
-
-/* Chooses the dK/dV kernel ct_attn_bwd runs for head dimension 128 (process-wide; no counterpart
- * in the reference, which has one backward). 0: two wavefronts per SIMD, 32 keys each. 1: one
- * wavefront per SIMD with 64 keys, the (dK, dV) sums in the accumulation registers and each step
- * as one generated instruction stream with the exponent / dS arithmetic and the next item's copies
- * between its own MFMAs. -1 (the default): by sequence length, kernel 1 from 16384 positions on
- * (its looping streams need long segments to pay off), kernel 0 below. Both give the same results
- * within the operator's tolerances (not bitwise: f32 summation order differs). */
-int32_t ct_attn_set_dkv_variant(int32_t variant);
 
 /* ------------------------------------------------------------------------
  * Preparation steps directly in front of the hot paths (they define the

@@ -51,14 +51,18 @@ def _random_ends(rng, ids, blocks_per_row=5):
     return ends
 
 
-def _run_gpu(ct, device, q, k, v, dout, ids, ends, scale):
+# how the backward of _run_gpu is pinned (set by the bwd_variant fixture; empty = the library's choice)
+_BWD = {}
+
+
+def _run_gpu(ct, device, q, k, v, dout, ids, ends, scale, **bwd):
     profile = ct.resolve_attention_profile(q.shape, k.shape, None, has_attention_end=ends is not None)
     metadata = ct.prepare_attention_metadata(
         torch.from_numpy(ids).to(device), mesh=None, profile=profile,
         attention_end=None if ends is None else torch.from_numpy(ends).to(device))
     qd, kd, vd, dod = (t.to(device) for t in (q, k, v, dout))
     out, lse = ct.attention_forward_with_lse(qd, kd, vd, metadata, scale=scale)
-    dq, dk, dv = ct.attention_backward(qd, kd, vd, metadata, out, lse, dod, scale=scale)
+    dq, dk, dv = ct.attention_backward(qd, kd, vd, metadata, out, lse, dod, scale=scale, **(bwd or _BWD))
     torch.cuda.synchronize()
     return tuple(t.cpu() for t in (out, lse, dq, dk, dv))
 
@@ -95,20 +99,25 @@ CASES = [
 ]
 
 
-@pytest.fixture(params=[0, 1], ids=["dkv32", "dkv64"])
-def dkv_variant(request, ct):
-    """Both dK/dV kernels of the backward: two wavefronts of 32 keys per SIMD and one wavefront of
-    64 keys (head dimension 128 only; other dimensions run the first). Tests without this fixture
-    run the default, which chooses by sequence length."""
+@pytest.fixture(params=[("narrow", "recompute"), ("wide", "recompute"), ("narrow", "from_ds")],
+                ids=["dkv32", "dkv64", "from_ds"])
+def bwd_variant(request):
+    """Every form of the backward: dQ from a second evaluation of S and dP beside either dK/dV
+    kernel (two wavefronts of 32 keys per SIMD, or one wavefront of 64 keys: head dimension 128
+    only, other dimensions run the first), and dQ from the dS blocks the narrow dK/dV kernel
+    stores. Tests without this fixture run what the library chooses by itself."""
 
-    ct.set_dkv_variant(request.param)
-    yield request.param
-    ct.set_dkv_variant(-1)
+    _BWD.clear()
+    _BWD.update(dkv_kernel=request.param[0], dq_form=request.param[1])
+    try:
+        yield request.param
+    finally:
+        _BWD.clear()
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B%d_S%d_Hq%d_Hkv%d_D%d_%s%s" % (
     c[0], c[1], c[2], c[3], c[4], "holes" if c[5] else "packed", "_ends" if c[6] else ""))
-def test_forward_backward_match_oracle(ct, gpu, case, dkv_variant):
+def test_forward_backward_match_oracle(ct, gpu, case, bwd_variant):
     batch, seq, q_heads, kv_heads, dim, holes, with_ends = case
     rng = np.random.default_rng(hash(case) % (2 ** 31))
     ids = _layout(rng, batch, seq, holes=holes)
@@ -123,36 +132,53 @@ def test_forward_backward_match_oracle(ct, gpu, case, dkv_variant):
     _check_against_oracle(results, q, k, v, dout, ids, ends, scale)
 
 
-@pytest.mark.parametrize("seq,expected", [(8192, 0), (16384, 1)])
-def test_default_dkv_kernel_goes_by_sequence_length(ct, gpu, seq, expected):
-    """Left to itself the backward runs the wide dK/dV kernel from 16384 positions on and the other
-    one below; each kernel is deterministic, so the default's dK and dV are bitwise those of the
-    kernel it should have chosen (and, the summation order being different, not the other's)."""
+@pytest.mark.parametrize("seq,expected", [(8192, "narrow"), (16384, "wide")])
+def test_default_choices_of_the_backward(ct, gpu, seq, expected):
+    """Left to itself the backward recomputes S and dP in its dQ kernel, beside the wide dK/dV
+    kernel from 16384 positions on and the narrow one below. Every kernel is deterministic, so the
+    default's results are bitwise those of the form it should have chosen (and, the summation
+    orders being different, not the others'). The stored-dS form has to be asked for, with a
+    workspace that holds at least one KV head's blocks."""
 
     rng = np.random.default_rng(seq)
     ids = _layout(rng, 1, seq, max_len=3000)
     q, dout = (_bf16(rng.standard_normal((1, seq, 2, 128))) for _ in range(2))
     k, v = (_bf16(rng.standard_normal((1, seq, 1, 128))) for _ in range(2))
+    library = ct._lib.load()
+    small = int(library.ct_attn_bwd_workspace_bytes(1, seq, 2, 1, 128))
+    assert small < int(library.ct_attn_bwd_workspace_bytes_from_ds(1, seq, 2, 1, 128, 0))
+    runs = {
+        "default": dict(dq_form=None),
+        "from_ds": dict(dq_form="from_ds"),
+        "narrow": dict(dkv_kernel="narrow", dq_form="recompute"),
+        "wide": dict(dkv_kernel="wide", dq_form="recompute"),
+    }
     results = {}
-    try:
-        for variant in (-1, 0, 1):
-            ct.set_dkv_variant(variant)
-            print("seq", seq, "variant", variant, flush=True)
-            results[variant] = _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5)
-    finally:
-        ct.set_dkv_variant(-1)
+    for name, pins in runs.items():
+        print("seq", seq, name, flush=True)
+        results[name] = _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5, **pins)
+    other = "wide" if expected == "narrow" else "narrow"
+    for index in (2, 3, 4):
+        assert torch.equal(results["default"][index], results[expected][index])
+        assert ref.relative_l2(results["narrow"][index], results["wide"][index]) <= 1e-2
+        assert ref.relative_l2(results["from_ds"][index], results["narrow"][index]) <= 1e-2
     for index in (3, 4):
-        assert torch.equal(results[-1][index], results[expected][index])
-        assert not torch.equal(results[-1][index], results[1 - expected][index])
-        assert ref.relative_l2(results[0][index], results[1][index]) <= 1e-2
+        assert not torch.equal(results["default"][index], results[other][index])
+    assert not torch.equal(results["from_ds"][2], results["narrow"][2])
+    with pytest.raises(ct._lib.CtError, match="stored-dS form needs"):
+        _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5, dq_form="from_ds", workspace_bytes=small)
+    with pytest.raises(ct._lib.CtError, match="no stored-dS form"):
+        _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5, dq_form="from_ds", dkv_kernel="wide")
 
 
-@pytest.mark.parametrize("scale", [0.0, -0.09, 1.0])
+@pytest.mark.parametrize("scale", [0.0, 1e-37, -0.09, 1.0])
 @pytest.mark.parametrize("dim", [64, 128])
-def test_any_finite_scale(ct, gpu, dkv_variant, scale, dim):
+def test_any_finite_scale(ct, gpu, bwd_variant, scale, dim):
     """The operator accepts any finite scale (src/kernels/efficient_attention.py:1947-1957): 0 gives
     uniform attention over the allowed keys (dQ and dK exactly 0), a negative one turns the order of
-    the scores around; the dK/dV kernels, which carry the scale in the exponent, must follow."""
+    the scores around; the dK/dV kernels, which carry the scale in the exponent, must follow. A scale
+    so small that lse / scale would overflow (1e-37) behaves like 0: finite results, uniform
+    attention, dQ and dK vanishingly small."""
 
     rng = np.random.default_rng(int(abs(scale) * 100) + dim)
     batch, seq, q_heads, kv_heads = 2, 256, 4, 2
@@ -165,8 +191,12 @@ def test_any_finite_scale(ct, gpu, dkv_variant, scale, dim):
     v = _bf16(rng.standard_normal((batch, seq, kv_heads, dim)))
     dout = _bf16(rng.standard_normal((batch, seq, q_heads, dim)))
     results = _run_gpu(ct, gpu, q, k, v, dout, ids, ends, scale)
-    if scale == 0.0:
-        assert not results[2].any() and not results[3].any()
+    if abs(scale) < 1e-30:
+        if scale == 0.0:
+            assert not results[2].any() and not results[3].any()
+        else:
+            assert all(torch.isfinite(t.float()).all() for t in results)
+            assert float(results[2].float().abs().max()) <= 1e-30 and float(results[3].float().abs().max()) <= 1e-30
         out, lse, _, _, dv = results
         allowed = ref.allowed_from_canonical(ids, ends)
         out_ref, _, _, dv_ref = ref.vanilla_attention_vjp(q, k, v, allowed, dout, scale=scale)
@@ -177,7 +207,7 @@ def test_any_finite_scale(ct, gpu, dkv_variant, scale, dim):
         _check_against_oracle(results, q, k, v, dout, ids, ends, scale)
 
 
-def test_edge_layouts(ct, gpu, dkv_variant):
+def test_edge_layouts(ct, gpu, bwd_variant):
     rng = np.random.default_rng(11)
     batch, seq, q_heads, kv_heads, dim = 4, 256, 4, 2, 128
     ids = np.zeros((batch, seq), np.int32)
@@ -214,7 +244,7 @@ def test_reference_seeded_fixture(ct, gpu):
         assert (grad[:, ids[0] != 2] == 0).all()
 
 
-def test_neighbour_perturbation_leaves_other_segment_bitwise_unchanged(ct, gpu, dkv_variant):
+def test_neighbour_perturbation_leaves_other_segment_bitwise_unchanged(ct, gpu, bwd_variant):
     # reference: tests/kernels/test_efficient_attention_tpu.py:395-424
     rng = np.random.default_rng(21)
     batch, seq, q_heads, kv_heads, dim = 1, 512, 4, 2, 128
@@ -235,7 +265,7 @@ def test_neighbour_perturbation_leaves_other_segment_bitwise_unchanged(ct, gpu, 
         assert torch.equal(a, b)        # fixed summation order: bitwise reproducible
 
 
-def test_zero_cross_segment_mass(ct, gpu, dkv_variant):
+def test_zero_cross_segment_mass(ct, gpu, bwd_variant):
     # V carries a one-hot of the key's segment id: any attention mass that leaks to another
     # segment shows up as a nonzero in a column that must be exactly 0.
     rng = np.random.default_rng(31)
@@ -311,6 +341,11 @@ def test_metadata_matches_oracle_bit_exact(ct, gpu):
                     assert bounds[b, rb, 7] <= queries[0] // 32 and queries[-1] // 32 <= bounds[b, rb, 8]
                 block = ids[b, rb * 32:(rb + 1) * 32]
                 assert bounds[b, rb, 2] == (block[0] if (block == block[0]).all() and block[0] != 0 else 0)
+        # where the dS blocks of a key block start: exclusive prefix sum of its visitors' range lengths
+        for b in range(2):
+            visitors = np.where(bounds[b, :, 8] >= bounds[b, :, 7], bounds[b, :, 8] - bounds[b, :, 7] + 1, 0)
+            np.testing.assert_array_equal(bounds[b, :, 9], np.concatenate(([0], np.cumsum(visitors)[:-1])))
+            assert visitors.sum() <= (1024 // 32) ** 2
         # schedules: permutations, ordered by non-increasing work
         blocks = 1024 // 32
         per_row = 2 * blocks + blocks // 4
@@ -385,7 +420,7 @@ def test_backward_leaves_delta_and_matches_the_pass_on_its_own(ct, gpu):
         torch.testing.assert_close(-delta, expected, atol=1e-4, rtol=1e-5)
 
 
-def test_split_key_tiles_match_oracle(ct, gpu, dkv_variant):
+def test_split_key_tiles_match_oracle(ct, gpu, bwd_variant):
     """One 2048-position segment, one KV head, a small batch: the dK/dV work list is far below
     one compute slot's share, so the chunk target sits at its minimum and the key tiles with the
     longest query lists are split into several chunks whose f32 partial sums the reduce kernel
@@ -490,6 +525,9 @@ def test_million_token_sequence(ct, gpu):
     per_block = ids.reshape(blocks, 32)
     np.testing.assert_array_equal(bounds[:, 1], per_block.max(1))
     np.testing.assert_array_equal(bounds[:, 5:9], _visit_ranges_of_canonical_ids(ids[0], ends[0]))
+    visitors = np.where(bounds[:, 8] >= bounds[:, 7], bounds[:, 8] - bounds[:, 7] + 1, 0).astype(np.int64)
+    np.testing.assert_array_equal(bounds[:, 9], np.minimum(np.concatenate(([0], np.cumsum(visitors)[:-1])),
+                                                           2 ** 31 - 1))
     flat = metadata.tile_bounds.cpu().numpy()
     per_row = 2 * blocks + blocks // 4
     schedules = flat[blocks * 12:blocks * 12 + per_row]
@@ -557,7 +595,7 @@ def _self_contained_window(ids_row, limit):
 
 
 @pytest.mark.parametrize("name", ["packed_small", "llama3_8b", "maskgit", "long_70b"])
-def test_benchmark_shapes(ct, gpu, name, dkv_variant):
+def test_benchmark_shapes(ct, gpu, name, bwd_variant):
     """Full benchmark shapes: size-independent properties everywhere, and the oracle on a
     self-contained window (whole segments) of one KV head with its query group."""
 
@@ -575,43 +613,50 @@ def test_benchmark_shapes(ct, gpu, name, dkv_variant):
         assert (tensor[pad] == 0).all()
     assert (lse[~pad] != 0).any()
 
+    # The oracle on three (batch row, KV head) pairs: the first, the last and one drawn at random
+    # (workgroups, work bins and split chunks place different rows and heads differently).
     group = config.q_heads // config.kv_heads
-    b, kvh = config.batch - 1, config.kv_heads - 1
-    heads = slice(kvh * group, (kvh + 1) * group)
-    start, stop = _self_contained_window(ids[b], 4096)
-    assert stop - start >= 512, "no whole segment short enough for the oracle"
-    window = slice(start, stop)
-    w_ids = ids[b:b + 1, window]
-    w_ends = None if ends is None else ends[b:b + 1, window] - start
-    q = inputs["q"][b:b + 1, window, heads]
-    k = inputs["k"][b:b + 1, window, kvh:kvh + 1]
-    v = inputs["v"][b:b + 1, window, kvh:kvh + 1]
-    dout = inputs["dout"][b:b + 1, window, heads]
-    got = (out[b:b + 1, window, heads], lse[b:b + 1, window, heads], dq[b:b + 1, window, heads],
-           dk[b:b + 1, window, kvh:kvh + 1], dv[b:b + 1, window, kvh:kvh + 1])
-    _check_against_oracle(got, q, k, v, dout, w_ids, w_ends, config.scale)
-
-    # The longest segment of the batch (up to the whole sequence): 64 sampled query rows with
-    # every head of the group for O, LSE and dQ; 64 sampled key rows for dK and dV, which sum
-    # over every query of the segment and every head of the group.
-    b, start, stop = _longest_segment(ids)
-    length = stop - start
-    assert length >= 256
     pick = np.random.default_rng(config.seed + 1)
-    edge = np.array([0, 1, 31, 32, 63, 64, 127, 128, length - 129, length - 65, length - 33, length - 2,
-                     length - 1])
-    edge = edge[(edge >= 0) & (edge < length)]
-    query_rows = np.unique(np.concatenate((edge, pick.choice(length, 64 - len(edge), replace=False))))
-    key_rows = np.unique(np.concatenate((edge, pick.choice(length, 64 - len(edge), replace=False))))
-    seg_ends = (np.arange(length) if ends is None else ends[b, start:stop] - start)
-    want = ref.segment_sampled_rows(
-        inputs["q"][b, start:stop, heads], inputs["k"][b, start:stop, kvh], inputs["v"][b, start:stop, kvh],
-        inputs["dout"][b, start:stop, heads], seg_ends, scale=config.scale, query_rows=query_rows,
-        key_rows=key_rows)
-    print("longest segment", name, b, start, stop, flush=True)
-    rows, cols = start + query_rows, start + key_rows
-    assert float((out[b, rows][:, heads].float() - want[0]).abs().max()) <= O_ATOL
-    assert float((lse[b, rows][:, heads] - want[1]).abs().max()) <= LSE_ATOL
-    assert ref.relative_l2(dq[b, rows][:, heads], want[2]) <= GRAD_RTOL
-    assert ref.relative_l2(dk[b, cols, kvh], want[3]) <= GRAD_RTOL
-    assert ref.relative_l2(dv[b, cols, kvh], want[4]) <= GRAD_RTOL
+    corners = [(0, 0), (config.batch - 1, config.kv_heads - 1),
+               (int(pick.integers(config.batch)), int(pick.integers(config.kv_heads)))]
+    for index, (b, kvh) in enumerate(dict.fromkeys(corners)):
+        heads = slice(kvh * group, (kvh + 1) * group)
+        # a self-contained window (whole segments) of this row
+        start, stop = _self_contained_window(ids[b], 4096)
+        assert stop - start >= 512, "no whole segment short enough for the oracle"
+        window = slice(start, stop)
+        w_ids = ids[b:b + 1, window]
+        w_ends = None if ends is None else ends[b:b + 1, window] - start
+        q = inputs["q"][b:b + 1, window, heads]
+        k = inputs["k"][b:b + 1, window, kvh:kvh + 1]
+        v = inputs["v"][b:b + 1, window, kvh:kvh + 1]
+        dout = inputs["dout"][b:b + 1, window, heads]
+        got = (out[b:b + 1, window, heads], lse[b:b + 1, window, heads], dq[b:b + 1, window, heads],
+               dk[b:b + 1, window, kvh:kvh + 1], dv[b:b + 1, window, kvh:kvh + 1])
+        print("window", name, b, kvh, start, stop, flush=True)
+        _check_against_oracle(got, q, k, v, dout, w_ids, w_ends, config.scale)
+
+        # The longest segment of this row (up to the whole sequence): sampled query rows with every
+        # head of the group for O, LSE and dQ; sampled key rows for dK and dV, which sum over every
+        # query of the segment and every head of the group.
+        _, start, stop = _longest_segment(ids[b:b + 1])
+        length = stop - start
+        assert length >= 64
+        samples = 64 if index == 0 else 32
+        edge = np.array([0, 1, 31, 32, 63, 64, 127, 128, length - 129, length - 65, length - 33, length - 2,
+                         length - 1])
+        edge = edge[(edge >= 0) & (edge < length)]
+        query_rows = np.unique(np.concatenate((edge, pick.choice(length, samples - len(edge), replace=False))))
+        key_rows = np.unique(np.concatenate((edge, pick.choice(length, samples - len(edge), replace=False))))
+        seg_ends = (np.arange(length) if ends is None else ends[b, start:stop] - start)
+        want = ref.segment_sampled_rows(
+            inputs["q"][b, start:stop, heads], inputs["k"][b, start:stop, kvh], inputs["v"][b, start:stop, kvh],
+            inputs["dout"][b, start:stop, heads], seg_ends, scale=config.scale, query_rows=query_rows,
+            key_rows=key_rows)
+        print("longest segment", name, b, kvh, start, stop, flush=True)
+        rows, cols = start + query_rows, start + key_rows
+        assert float((out[b, rows][:, heads].float() - want[0]).abs().max()) <= O_ATOL
+        assert float((lse[b, rows][:, heads] - want[1]).abs().max()) <= LSE_ATOL
+        assert ref.relative_l2(dq[b, rows][:, heads], want[2]) <= GRAD_RTOL
+        assert ref.relative_l2(dk[b, cols, kvh], want[3]) <= GRAD_RTOL
+        assert ref.relative_l2(dv[b, cols, kvh], want[4]) <= GRAD_RTOL

@@ -28,8 +28,25 @@ def test_size_queries_need_no_gpu(ct):
     bins = sum(33 + 4 * ((nrb + pb - 1) // pb) for pb in (2, 4, 8))
     assert library.ct_attn_meta_bytes(4, 4096) == (4 * (nrb * 12 + 2 * nrb + nrb // 4) + bins) * 4
     assert library.ct_attn_meta_bytes(0, 128) == 0
-    assert 0 < library.ct_attn_bwd_workspace_bytes(4, 4096, 32, 8, 128) < 1 << 30
+    # the backward's scratch: the work list, statistics and partial sums alone are small ...
+    least = library.ct_attn_bwd_workspace_bytes(4, 4096, 32, 8, 128)
+    assert 0 < least < 1 << 30
     assert library.ct_attn_bwd_workspace_bytes(4, 4000, 32, 8, 128) == 0
+    assert library.ct_attn_bwd_workspace_bytes_from_ds(4, 4000, 32, 8, 128, 0) == 0
+    # ... the stored-dS form adds 2 KB per (key block, query block at or after it) pair of every
+    # batch row and query head (nrb^2 pairs with visible ends)
+    causal = library.ct_attn_bwd_workspace_bytes_from_ds(4, 4096, 32, 8, 128, 0)
+    hybrid = library.ct_attn_bwd_workspace_bytes_from_ds(4, 4096, 32, 8, 128, 1)
+    assert causal - least == 4 * 32 * (nrb * (nrb + 1) // 2) * 2048
+    assert hybrid - least == 4 * 32 * nrb * nrb * 2048
+    # the region is capped at 16 GiB but never below one KV head's blocks: 64 query heads over 8 KV heads
+    # at S = 32768 take 8.6 GB per KV head, so the backward runs in 8 passes of one KV head
+    long_blocks = (32768 // 32) * (32768 // 32 + 1) // 2
+    long_total = library.ct_attn_bwd_workspace_bytes_from_ds(1, 32768, 64, 8, 128, 0)
+    long_least = library.ct_attn_bwd_workspace_bytes(1, 32768, 64, 8, 128)
+    assert 8 * long_blocks * 2048 <= long_total - long_least + (1 << 30) and long_total < 10 << 30
+    # one KV head beyond 64 GiB: that form is not available
+    assert library.ct_attn_bwd_workspace_bytes_from_ds(1, 1 << 20, 2, 1, 64, 1) == 0
     shape = ct._lib.CutceShape(16384, 4096, 128256)
     fwd = library.ct_cutce_fwd_workspace_bytes(ctypes.byref(shape))
     full = library.ct_cutce_bwd_workspace_bytes(ctypes.byref(shape))
