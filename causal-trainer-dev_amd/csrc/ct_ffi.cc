@@ -40,6 +40,10 @@ ffi::Error AttnPrepare(hipStream_t stream, ffi::Buffer<ffi::S32> segment_ids,
                        bool has_end) {
   const auto dims = segment_ids.dimensions();
   if (dims.size() != 2) return ffi::Error::InvalidArgument("segment_ids must be [batch, sequence]");
+  // ct_attn_prepare takes no buffer size: the table, its schedules and (for very long rows) the
+  // scratch tail the kernels work in must all fit the result the caller asked XLA for
+  if (tile_meta->size_bytes() < ct_attn_meta_bytes((int32_t)dims[0], (int32_t)dims[1]))
+    return ffi::Error::InvalidArgument("tile_meta is smaller than ct_attn_meta_bytes(batch, sequence)");
   return status_to_error(ct_attn_prepare(stream, segment_ids.typed_data(),
                                          has_end ? attention_end.typed_data() : nullptr,
                                          (int32_t)dims[0], (int32_t)dims[1], tile_meta->typed_data()));
@@ -170,6 +174,44 @@ ffi::Error CutceBwd(hipStream_t stream, ffi::Buffer<ffi::BF16> hidden, ffi::Buff
     a.logits_cache_bytes = logits_cache.size_bytes();
   }
   return status_to_error(ct_cutce_bwd(stream, &a));
+}
+
+// ---- preparation steps in front of the hot paths (bit-exact integer kernels) ------------------
+
+// An absent optional operand is passed as any int32 array of the right shape plus a false flag.
+ffi::Error CanonicalizeSegmentIds(hipStream_t stream, ffi::Buffer<ffi::S32> attention_mask,
+                                  ffi::Buffer<ffi::S32> segment_ids, ffi::ResultBuffer<ffi::S32> canonical,
+                                  bool has_segments) {
+  const auto dims = attention_mask.dimensions();
+  if (dims.size() != 2) return ffi::Error::InvalidArgument("attention_mask must be [batch, sequence]");
+  return status_to_error(ct_canonicalize_segment_ids(stream, attention_mask.typed_data(),
+                                                     has_segments ? segment_ids.typed_data() : nullptr,
+                                                     (int32_t)dims[0], (int32_t)dims[1], canonical->typed_data()));
+}
+
+ffi::Error ShiftedTargets(hipStream_t stream, ffi::Buffer<ffi::S32> input_ids, ffi::Buffer<ffi::S32> attention_mask,
+                          ffi::Buffer<ffi::S32> segment_ids, ffi::Buffer<ffi::S32> assistant_mask,
+                          ffi::Buffer<ffi::F32> loss_mask, ffi::Buffer<ffi::S32> labels,
+                          ffi::ResultBuffer<ffi::S32> targets, ffi::ResultBuffer<ffi::F32> weights,
+                          ffi::ResultBuffer<ffi::U8> scratch, bool has_mask, bool has_segments, bool has_assistant,
+                          bool has_loss_mask, bool has_labels, int32_t ignore_index) {
+  const auto dims = input_ids.dimensions();
+  if (dims.size() != 2) return ffi::Error::InvalidArgument("input_ids must be [batch, sequence]");
+  ct_shifted_targets_args a = {};
+  a.input_ids = input_ids.typed_data();
+  a.attention_mask = has_mask ? attention_mask.typed_data() : nullptr;
+  a.segment_ids = has_segments ? segment_ids.typed_data() : nullptr;
+  a.assistant_mask = has_assistant ? assistant_mask.typed_data() : nullptr;
+  a.loss_mask = has_loss_mask ? loss_mask.typed_data() : nullptr;
+  a.labels = has_labels ? labels.typed_data() : nullptr;
+  a.targets = targets->typed_data();
+  a.weights = weights->typed_data();
+  a.scratch = scratch->untyped_data();
+  a.scratch_bytes = scratch->size_bytes();
+  a.batch = (int32_t)dims[0];
+  a.seq = (int32_t)dims[1];
+  a.ignore_index = ignore_index;
+  return status_to_error(ct_shifted_targets_and_weights(stream, &a));
 }
 
 // ---- decoder-layer neighbours and the logits-level loss ----------------------------------
@@ -341,6 +383,31 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_cutce_bwd, CutceBwd,
                                   .Ret<ffi::Buffer<ffi::U8>>()
                                   .Attr<bool>("sparse_compaction")
                                   .Attr<bool>("head_trainable"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_canonicalize_segment_ids, CanonicalizeSegmentIds,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::S32>>()
+                                  .Attr<bool>("has_segments"));
+
+XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_shifted_targets, ShiftedTargets,
+                              ffi::Ffi::Bind()
+                                  .CT_STREAM.Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Arg<ffi::Buffer<ffi::F32>>()
+                                  .Arg<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::S32>>()
+                                  .Ret<ffi::Buffer<ffi::F32>>()
+                                  .Ret<ffi::Buffer<ffi::U8>>()
+                                  .Attr<bool>("has_mask")
+                                  .Attr<bool>("has_segments")
+                                  .Attr<bool>("has_assistant")
+                                  .Attr<bool>("has_loss_mask")
+                                  .Attr<bool>("has_labels")
+                                  .Attr<int32_t>("ignore_index"));
 
 XLA_FFI_DEFINE_HANDLER_SYMBOL(ct_ffi_position_ids, PositionIds,
                               ffi::Ffi::Bind()

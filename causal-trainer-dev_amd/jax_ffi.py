@@ -9,6 +9,13 @@ Reference-side glue with the reference's operator interfaces:
   pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weights, *, mesh,
       sparse_compaction=False, lm_head_trainable=True, local_chunk_size=0)
                                                  src/causal_trainer/kernels/cut_cross_entropy.py:524-670, :828-958
+  canonicalize_segment_ids, make_position_ids, rotary_cos_sin, apply_rotary_cos_sin,
+      apply_rotary_embedding                     src/causal_trainer/modeling/rotary.py:13-50, :63-234
+  rms_norm(x, scale, eps, compute_dtype)         src/causal_trainer/modeling/architecture.py:155-162
+  shifted_targets_and_weights (= _shifted_targets_and_weights)
+                                                 src/causal_trainer/training/losses.py:21-85
+  pallas_fused_sparse_cross_entropy(logits, targets, weights, *, mesh)
+                                                 src/causal_trainer/kernels/cross_entropy.py:600-643
 
 so that the call sites at src/causal_trainer/modeling/attention.py:435-444,
 src/causal_trainer/modeling/architecture.py:691-696 and
@@ -62,6 +69,9 @@ HANDLERS = {
     "ct_ffi_attn_bwd": Handler(9, 5, ("scale", "has_end")),
     "ct_ffi_cutce_fwd": Handler(4, 5, ("sparse_compaction",)),
     "ct_ffi_cutce_bwd": Handler(7, 3, ("sparse_compaction", "head_trainable")),
+    "ct_ffi_canonicalize_segment_ids": Handler(2, 1, ("has_segments",)),
+    "ct_ffi_shifted_targets": Handler(6, 3, ("has_mask", "has_segments", "has_assistant", "has_loss_mask",
+                                             "has_labels", "ignore_index")),
     "ct_ffi_position_ids": Handler(2, 1, ()),
     "ct_ffi_rotary_cos_sin": Handler(2, 2, ()),
     "ct_ffi_apply_rotary": Handler(4, 2, ("rope_style", "inverse", "q_scale")),
@@ -420,6 +430,299 @@ def pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weig
                           bool(lm_head_trainable), bool(sparse_compaction), local_chunk_size)
 
 
+# ------------------------------------------------------------------------------------------
+# preparation steps in front of the hot paths (integer kernels, nothing to differentiate)
+# ------------------------------------------------------------------------------------------
+def canonicalize_segment_ids(attention_mask, segment_ids=None):
+    """One-based ids of contiguous valid runs, zero for padding (int32 ``[batch, sequence]``)."""
+
+    import jax.numpy as jnp
+
+    valid = jnp.asarray(attention_mask, dtype=jnp.bool_)
+    if valid.ndim != 2:
+        raise ValueError(f"attention_mask must have shape [batch, sequence], got {valid.shape}")
+    mask = valid.astype(jnp.int32)
+    has_segments = segment_ids is not None
+    if has_segments:
+        labels = jnp.asarray(segment_ids, dtype=jnp.int32)
+        if labels.shape != valid.shape:
+            raise ValueError(f"segment_ids must have shape {valid.shape}, got {labels.shape}")
+    else:
+        labels = mask                                  # placeholder of the right shape, not read
+    if valid.size == 0:
+        return jnp.zeros(valid.shape, jnp.int32)
+    (canonical,) = _call("ct_ffi_canonicalize_segment_ids", [_struct(valid.shape, jnp.int32)], mask, labels,
+                         has_segments=has_segments)
+    return canonical
+
+
+def shifted_targets_and_weights(input_ids, attention_mask, segment_ids=None, assistant_mask=None, loss_mask=None,
+                                labels=None, *, ignore_index: int = -100):
+    """Safe shifted targets (int32) and target-position loss weights (f32), ``[batch, sequence - 1]`` each."""
+
+    import jax.numpy as jnp
+
+    tokens = jnp.asarray(input_ids, dtype=jnp.int32)
+    if tokens.ndim != 2:
+        raise ValueError(f"input_ids must have shape [batch, sequence], got {tokens.shape}")
+
+    def optional(value, name, convert):
+        if value is None:
+            return tokens, False                       # placeholder of the right shape, not read
+        array = convert(jnp.asarray(value))
+        if array.shape != tokens.shape:
+            raise ValueError(f"{name} must have shape {tokens.shape}, got {array.shape}")
+        return array, True
+
+    label_array, has_labels = optional(labels, "labels", lambda a: a.astype(jnp.int32))
+    # validity is "mask == 1" (losses.py:49)
+    mask_array, has_mask = optional(attention_mask, "attention_mask", lambda a: (a == 1).astype(jnp.int32))
+    segment_array, has_segments = optional(segment_ids, "segment_ids", lambda a: a.astype(jnp.int32))
+    assistant_array, has_assistant = optional(assistant_mask, "assistant_mask", lambda a: (a != 0).astype(jnp.int32))
+    if loss_mask is None:
+        loss_array, has_loss_mask = jnp.zeros(tokens.shape, jnp.float32), False
+    else:
+        loss_array, has_loss_mask = jnp.asarray(loss_mask, dtype=jnp.float32), True
+        if loss_array.shape != tokens.shape:
+            raise ValueError(f"loss_mask must have shape {tokens.shape}, got {loss_array.shape}")
+    batch, sequence = tokens.shape
+    if sequence < 2:
+        raise ValueError("input_ids needs at least two positions to form a prediction edge")
+    if has_segments and not has_mask:                  # canonical runs need a validity mask: every token valid
+        mask_array, has_mask = jnp.ones(tokens.shape, jnp.int32), True
+    scratch = max(16, int(_lib.load().ct_shifted_targets_scratch_bytes(batch, sequence)))
+    targets, weights, _ = _call(
+        "ct_ffi_shifted_targets",
+        [_struct((batch, sequence - 1), jnp.int32), _struct((batch, sequence - 1), jnp.float32),
+         _struct((scratch,), jnp.uint8)],
+        tokens, mask_array, segment_array, assistant_array, loss_array, label_array,
+        has_mask=has_mask, has_segments=has_segments, has_assistant=has_assistant, has_loss_mask=has_loss_mask,
+        has_labels=has_labels, ignore_index=np.int32(ignore_index))
+    return targets, weights
+
+
+# ------------------------------------------------------------------------------------------
+# decoder-layer neighbours of attention
+# ------------------------------------------------------------------------------------------
+_ROPE_STYLES = {"gpt-j": 0, "gpt-neox": 1}
+
+
+def _make_position_ids_precanonicalized(attention_mask, segment_ids):
+    import jax.numpy as jnp
+
+    valid = jnp.asarray(attention_mask, dtype=jnp.bool_)
+    if valid.ndim != 2:
+        raise ValueError(f"attention_mask must have shape [batch, sequence], got {valid.shape}")
+    segments = jnp.asarray(segment_ids, dtype=jnp.int32)
+    if segments.shape != valid.shape:
+        raise ValueError(f"segment_ids must have shape {valid.shape}, got {segments.shape}")
+    if valid.size == 0:
+        return jnp.zeros(valid.shape, jnp.int32)
+    (positions,) = _call("ct_ffi_position_ids", [_struct(valid.shape, jnp.int32)], valid.astype(jnp.int32), segments)
+    return positions
+
+
+def make_position_ids(attention_mask, segment_ids=None):
+    """Zero-based positions that reset at every packed segment (int32 ``[batch, sequence]``)."""
+
+    import jax.numpy as jnp
+
+    valid = jnp.asarray(attention_mask, dtype=jnp.bool_)
+    if valid.ndim != 2:
+        raise ValueError(f"attention_mask must have shape [batch, sequence], got {valid.shape}")
+    return _make_position_ids_precanonicalized(valid, canonicalize_segment_ids(valid, segment_ids))
+
+
+def rotary_cos_sin(position_ids, inv_freq, dtype):
+    """Per-token cos / sin tables ``[batch, sequence, rotary_dim / 2]``: f32 angles, one cast to bf16."""
+
+    import jax.numpy as jnp
+
+    positions = jnp.asarray(position_ids)
+    if positions.ndim != 2:
+        raise ValueError(f"position_ids must have shape [batch, sequence], got {positions.shape}")
+    frequencies = jnp.asarray(inv_freq, dtype=jnp.float32)
+    if frequencies.ndim != 1 or frequencies.shape[0] == 0:
+        raise ValueError(f"inv_freq must be a non-empty vector, got {frequencies.shape}")
+    if jnp.dtype(dtype) != jnp.bfloat16:
+        raise ValueError("the MI355X path computes rotary tables in bfloat16 only")
+    table = _struct(positions.shape + (frequencies.shape[0],), jnp.bfloat16)
+    cosine, sine = _call("ct_ffi_rotary_cos_sin", [table, table], positions.astype(jnp.int32), frequencies)
+    return cosine, sine
+
+
+@functools.lru_cache(maxsize=1)
+def _apply_rotary_impl():
+    import jax
+    import jax.numpy as jnp
+
+    def rotate(query, key, cosine, sine, style, q_scale, inverse):
+        return _call("ct_ffi_apply_rotary", [_struct(query.shape, jnp.bfloat16), _struct(key.shape, jnp.bfloat16)],
+                     query, key, cosine, sine, rope_style=np.int32(style), inverse=bool(inverse),
+                     q_scale=np.float32(q_scale))
+
+    # the rotation is linear in (query, key): its VJP is the transposed rotation of the cotangents
+    @functools.partial(jax.custom_vjp, nondiff_argnums=(4, 5))
+    def apply(query, key, cosine, sine, style, q_scale):
+        return tuple(rotate(query, key, cosine, sine, style, q_scale, False))
+
+    def apply_fwd(query, key, cosine, sine, style, q_scale):
+        return tuple(rotate(query, key, cosine, sine, style, q_scale, False)), (cosine, sine)
+
+    def apply_bwd(style, q_scale, residual, cotangents):
+        cosine, sine = residual
+        dq, dk = cotangents
+        dq_in, dk_in = rotate(dq.astype(jnp.bfloat16), dk.astype(jnp.bfloat16), cosine, sine, style, q_scale, True)
+        return dq_in, dk_in, None, None
+
+    apply.defvjp(apply_fwd, apply_bwd)
+    return apply
+
+
+def apply_rotary_cos_sin(query, key, cosine, sine, *, rope_style: str = "gpt-j", q_scale: float = 1.0):
+    """Partial RoPE of Q and K ``[batch, sequence, heads, head_dim]`` from precomputed tables.
+    ``q_scale`` (not in the reference signature, default off) also applies the attention operator's
+    bf16 pre-scale of Q in the same pass; call ``efficient_attention`` with scale 1 then."""
+
+    import jax.numpy as jnp
+
+    if query.ndim != 4 or key.ndim != 4:
+        raise ValueError("query and key must have shape [batch, sequence, heads, head_dim]")
+    if query.shape[:2] != key.shape[:2] or query.shape[-1] != key.shape[-1]:
+        raise ValueError(f"incompatible query/key shapes: {query.shape} and {key.shape}")
+    cosine, sine = jnp.asarray(cosine), jnp.asarray(sine)
+    if cosine.shape != sine.shape:
+        raise ValueError(f"cosine and sine shapes differ: {cosine.shape} and {sine.shape}")
+    if cosine.ndim != 3 or cosine.shape[:2] != query.shape[:2]:
+        raise ValueError("cosine and sine must have shape "
+                         f"[{query.shape[0]}, {query.shape[1]}, rotary_dim / 2], got {cosine.shape}")
+    rotary_dim = cosine.shape[-1] * 2
+    if rotary_dim <= 0 or rotary_dim > query.shape[-1] or rotary_dim % 2:
+        raise ValueError(f"invalid rotary dimension {rotary_dim} for head_dim={query.shape[-1]}")
+    if rope_style not in _ROPE_STYLES:
+        raise ValueError("rope_style must be 'gpt-j' or 'gpt-neox'")
+    if query.dtype != jnp.bfloat16 or key.dtype != jnp.bfloat16:
+        raise ValueError("the MI355X path rotates bfloat16 query and key only")
+    return _apply_rotary_impl()(query, key, cosine.astype(jnp.bfloat16), sine.astype(jnp.bfloat16),
+                                _ROPE_STYLES[rope_style], float(q_scale))
+
+
+def apply_rotary_embedding(query, key, position_ids, inv_freq, *, rope_style: str = "gpt-j"):
+    """Partial RoPE of Q and K from positions (``[sequence]`` or ``[batch, sequence]``) and inverse frequencies."""
+
+    import jax.numpy as jnp
+
+    if query.ndim != 4 or key.ndim != 4:
+        raise ValueError("query and key must have shape [batch, sequence, heads, head_dim]")
+    if query.shape[:2] != key.shape[:2] or query.shape[-1] != key.shape[-1]:
+        raise ValueError(f"incompatible query/key shapes: {query.shape} and {key.shape}")
+    positions = jnp.asarray(position_ids)
+    if positions.ndim == 1:
+        positions = jnp.broadcast_to(positions[None, :], query.shape[:2])
+    if positions.shape != query.shape[:2]:
+        raise ValueError(f"position_ids must have shape {query.shape[:2]}, got {positions.shape}")
+    inv_freq = jnp.asarray(inv_freq, dtype=jnp.float32)
+    rotary_dim = inv_freq.shape[0] * 2
+    if rotary_dim <= 0 or rotary_dim > query.shape[-1] or rotary_dim % 2:
+        raise ValueError(f"invalid rotary dimension {rotary_dim} for head_dim={query.shape[-1]}")
+    cosine, sine = rotary_cos_sin(positions, inv_freq, query.dtype)
+    return apply_rotary_cos_sin(query, key, cosine, sine, rope_style=rope_style)
+
+
+@functools.lru_cache(maxsize=1)
+def _rms_norm_impl():
+    import jax
+    import jax.numpy as jnp
+
+    @functools.partial(jax.custom_vjp, nondiff_argnums=(2,))
+    def norm(x, scale, eps):
+        (y,) = _call("ct_ffi_rms_norm_fwd", [_struct(x.shape, jnp.bfloat16)], x, scale, eps=np.float32(eps))
+        return y
+
+    def norm_fwd(x, scale, eps):
+        return norm(x, scale, eps), (x, scale)
+
+    def norm_bwd(eps, residual, dy):
+        x, scale = residual
+        hidden = x.shape[-1]
+        workspace = int(_lib.load().ct_rms_norm_bwd_workspace_bytes(hidden))
+        dx, dscale, _ = _call(
+            "ct_ffi_rms_norm_bwd",
+            [_struct(x.shape, jnp.bfloat16), _struct((hidden,), jnp.float32), _struct((max(workspace, 16),), jnp.uint8)],
+            x, scale, dy.astype(jnp.bfloat16), eps=np.float32(eps))
+        return dx, dscale.astype(scale.dtype)
+
+    norm.defvjp(norm_fwd, norm_bwd)
+    return norm
+
+
+def rms_norm(x, scale, eps: float, compute_dtype):
+    """RMS normalisation over the last axis with f32 statistics and a learned scale (bf16 in, bf16 out)."""
+
+    import jax.numpy as jnp
+
+    x, scale = jnp.asarray(x), jnp.asarray(scale)
+    if jnp.dtype(compute_dtype) != jnp.bfloat16 or x.dtype != jnp.bfloat16:
+        raise ValueError("the MI355X path normalises bfloat16 activations with a bfloat16 compute dtype")
+    if scale.ndim != 1 or scale.shape[0] != x.shape[-1]:
+        raise ValueError(f"scale must have shape ({x.shape[-1]},), got {scale.shape}")
+    if x.size == 0:
+        return x
+    return _rms_norm_impl()(x, scale.astype(jnp.bfloat16), float(eps))
+
+
+# ------------------------------------------------------------------------------------------
+# sparse cross-entropy on materialised logits (the trainer's non-fused loss backend)
+# ------------------------------------------------------------------------------------------
+@functools.lru_cache(maxsize=1)
+def _sparse_ce_impl():
+    import jax
+    import jax.numpy as jnp
+
+    def forward(logits, targets, weights):
+        rows = _struct((logits.shape[0],), jnp.float32)
+        return _call("ct_ffi_sparse_ce_fwd", [rows, rows], logits, targets, weights)
+
+    @jax.custom_vjp
+    def loss(logits, targets, weights):
+        return forward(logits, targets, weights)[0]
+
+    def loss_fwd(logits, targets, weights):
+        per_row, lse = forward(logits, targets, weights)
+        return per_row, (logits, targets, weights, lse)
+
+    def loss_bwd(residual, dy):
+        logits, targets, weights, lse = residual
+        (dlogits,) = _call("ct_ffi_sparse_ce_bwd", [_struct(logits.shape, logits.dtype)], logits, targets, weights,
+                           lse, dy.astype(jnp.float32))
+        return dlogits, None, None
+
+    loss.defvjp(loss_fwd, loss_bwd)
+    return loss
+
+
+def pallas_fused_sparse_cross_entropy(logits, targets, weights, *, mesh):
+    """Per-token weighted CE ``[batch, sequence]`` (f32) of logits ``[batch, sequence, vocab]`` (bf16 or
+    f32); rows with target -100 or weight 0 contribute nothing and are not read."""
+
+    import jax.numpy as jnp
+
+    logits = jnp.asarray(logits)
+    if logits.ndim != 3 or targets.shape != logits.shape[:-1] or weights.shape != targets.shape:
+        raise ValueError("Pallas CE expects logits [batch, sequence, vocab] and matching target/weight rows")
+    _require_one_device(mesh, "pallas_fused_sparse_cross_entropy")
+    if logits.dtype not in (jnp.bfloat16, jnp.float32):
+        raise ValueError("logits must be bfloat16 or float32")
+    leading = logits.shape[:-1]
+    if logits.size == 0:
+        return jnp.zeros(leading, jnp.float32)
+    flat = _sparse_ce_impl()(logits.reshape(-1, logits.shape[-1]), jnp.asarray(targets, jnp.int32).reshape(-1),
+                             jnp.asarray(weights, jnp.float32).reshape(-1))
+    return flat.reshape(leading)
+
+
 __all__ = ["AttentionKernelProfile", "AttentionMetadata", "HANDLERS", "LOGITS_CACHE_LIMIT_BYTES",
-           "backward_workspace_bytes", "efficient_attention", "pallas_cut_linear_cross_entropy",
-           "prepare_attention_metadata", "register", "resolve_attention_profile"]
+           "apply_rotary_cos_sin", "apply_rotary_embedding", "backward_workspace_bytes", "canonicalize_segment_ids",
+           "efficient_attention", "make_position_ids", "pallas_cut_linear_cross_entropy",
+           "pallas_fused_sparse_cross_entropy", "prepare_attention_metadata", "register", "resolve_attention_profile",
+           "rms_norm", "rotary_cos_sin", "shifted_targets_and_weights"]

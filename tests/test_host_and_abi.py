@@ -190,7 +190,7 @@ def test_jax_binding_matches_the_ffi_handlers_and_the_documentation(ct):
     from causal_trainer_dev_amd import jax_ffi
 
     in_source = _ffi_handlers_in_source()
-    assert len(in_source) == 12
+    assert len(in_source) == 14
     assert {name: tuple(handler) for name, handler in jax_ffi.HANDLERS.items()} == in_source
     documented = set(re.findall(r"`(ct_ffi_\w+)`", (ROOT / "INTEGRATION.md").read_text()))
     assert documented == set(in_source)
@@ -206,8 +206,9 @@ def test_jax_binding_matches_the_ffi_handlers_and_the_documentation(ct):
         assert isinstance(site.args[1], ast.List) and len(site.args[1].elts) == results, name
         assert len(site.args) - 2 == operands, name
         assert tuple(keyword.arg for keyword in site.keywords) == attributes, name
+    # every registered handler has a caller: no symbol is handed to a maintainer without its glue
     used = {site.args[0].value for site in sites}
-    assert {"ct_ffi_attn_prepare", "ct_ffi_attn_fwd", "ct_ffi_attn_bwd", "ct_ffi_cutce_fwd", "ct_ffi_cutce_bwd"} <= used
+    assert used == set(in_source)
 
     # the operators keep the reference's signatures (efficient_attention.py:326-331, :1890-1900;
     # cut_cross_entropy.py:828-838)
@@ -228,6 +229,33 @@ def test_jax_binding_matches_the_ffi_handlers_and_the_documentation(ct):
         ("targets", "POSITIONAL_OR_KEYWORD", empty), ("weights", "POSITIONAL_OR_KEYWORD", empty),
         ("mesh", "KEYWORD_ONLY", empty), ("sparse_compaction", "KEYWORD_ONLY", False),
         ("lm_head_trainable", "KEYWORD_ONLY", True), ("local_chunk_size", "KEYWORD_ONLY", 0)]
+    # the rows either side of the two paths (rotary.py:13-16, :63-66, :132-136, :160-167, :207-214;
+    # architecture.py:155; losses.py:21-30; cross_entropy.py:600-606)
+    assert parameters(jax_ffi.canonicalize_segment_ids) == [
+        ("attention_mask", "POSITIONAL_OR_KEYWORD", empty), ("segment_ids", "POSITIONAL_OR_KEYWORD", None)]
+    assert parameters(jax_ffi.make_position_ids) == parameters(jax_ffi.canonicalize_segment_ids)
+    assert parameters(jax_ffi.rotary_cos_sin) == [
+        ("position_ids", "POSITIONAL_OR_KEYWORD", empty), ("inv_freq", "POSITIONAL_OR_KEYWORD", empty),
+        ("dtype", "POSITIONAL_OR_KEYWORD", empty)]
+    assert parameters(jax_ffi.apply_rotary_cos_sin)[:5] == [
+        ("query", "POSITIONAL_OR_KEYWORD", empty), ("key", "POSITIONAL_OR_KEYWORD", empty),
+        ("cosine", "POSITIONAL_OR_KEYWORD", empty), ("sine", "POSITIONAL_OR_KEYWORD", empty),
+        ("rope_style", "KEYWORD_ONLY", "gpt-j")]
+    assert parameters(jax_ffi.apply_rotary_embedding) == [
+        ("query", "POSITIONAL_OR_KEYWORD", empty), ("key", "POSITIONAL_OR_KEYWORD", empty),
+        ("position_ids", "POSITIONAL_OR_KEYWORD", empty), ("inv_freq", "POSITIONAL_OR_KEYWORD", empty),
+        ("rope_style", "KEYWORD_ONLY", "gpt-j")]
+    assert parameters(jax_ffi.rms_norm) == [
+        ("x", "POSITIONAL_OR_KEYWORD", empty), ("scale", "POSITIONAL_OR_KEYWORD", empty),
+        ("eps", "POSITIONAL_OR_KEYWORD", empty), ("compute_dtype", "POSITIONAL_OR_KEYWORD", empty)]
+    assert parameters(jax_ffi.shifted_targets_and_weights) == [
+        ("input_ids", "POSITIONAL_OR_KEYWORD", empty), ("attention_mask", "POSITIONAL_OR_KEYWORD", empty),
+        ("segment_ids", "POSITIONAL_OR_KEYWORD", None), ("assistant_mask", "POSITIONAL_OR_KEYWORD", None),
+        ("loss_mask", "POSITIONAL_OR_KEYWORD", None), ("labels", "POSITIONAL_OR_KEYWORD", None),
+        ("ignore_index", "KEYWORD_ONLY", -100)]
+    assert parameters(jax_ffi.pallas_fused_sparse_cross_entropy) == [
+        ("logits", "POSITIONAL_OR_KEYWORD", empty), ("targets", "POSITIONAL_OR_KEYWORD", empty),
+        ("weights", "POSITIONAL_OR_KEYWORD", empty), ("mesh", "KEYWORD_ONLY", empty)]
     assert jax_ffi.AttentionMetadata._fields[:5] == (
         "query_segment_ids", "kv_segment_ids", "q_block_segments", "kv_block_segments", "attention_end")
     assert jax_ffi.AttentionMetadata._fields[5:] == ("tile_bounds",)
