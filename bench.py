@@ -63,6 +63,11 @@ def parse_args():
     parser.add_argument("--cutce-cached-only", action="store_true",
                         help="only time cut-CE with the logits cache")
     parser.add_argument("--no-shapes", action="store_true", help="skip the other attention shapes")
+    parser.add_argument("--only-shape", default=None, metavar="NAME",
+                        help="counter runs: only the attention step at this named shape (llama3_8b, maskgit, "
+                             "long_70b, packed_small), a reduced JSON line")
+    parser.add_argument("--only-cutce", action="store_true",
+                        help="counter runs: only cut-CE without the logits cache, a reduced JSON line")
     parser.add_argument("--preamble-steps", type=int, default=300,
                         help="untimed attention steps before the warm-up (clock ramp)")
     return parser.parse_args()
@@ -292,6 +297,65 @@ def bench_attention(ct, torch, steps, warmup, preamble_steps):
     }
 
 
+def step_time_distribution(torch, step, steps, warmup, preamble=0):
+    """Median, minimum and maximum over `steps` steps, each bracketed by its own pair of stream events
+    (recorded on torch's current stream, which is the stream the library launches on), after the
+    same preamble and warm-up as the timed region. Not the headline: the events sit between the
+    steps, so consecutive steps cannot overlap their launch overhead as they do in the timed region."""
+
+    gc.collect()
+    gc.disable()
+    try:
+        for _ in range(preamble + warmup):
+            step()
+        events = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+        events[0].record()
+        for index in range(steps):
+            step()
+            events[index + 1].record()
+        torch.cuda.synchronize()
+    finally:
+        gc.enable()
+    times = sorted(events[i].elapsed_time(events[i + 1]) for i in range(steps))
+    return {"median_ms": times[len(times) // 2], "min_ms": times[0], "max_ms": times[-1], "steps": steps}
+
+
+def bench_forward_backward_split(ct, torch, config, attention, steps, warmup, preamble_steps):
+    """The forward alone and the backward alone at the headline shape (same inputs, the backward from
+    one saved (O, LSE) pair), each as a timed region of its own, and the distribution of the whole
+    step over the timed steps."""
+
+    inputs = attention["inputs"]
+    profile = ct.resolve_attention_profile(inputs["q"].shape, inputs["k"].shape, None,
+                                           has_attention_end=inputs["attention_end"] is not None)
+    metadata = ct.prepare_attention_metadata(inputs["segment_ids"], mesh=None, profile=profile,
+                                             attention_end=inputs["attention_end"])
+    q, k, v, dout = inputs["q"], inputs["k"], inputs["v"], inputs["dout"]
+    out, lse = ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
+
+    def forward():
+        ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
+
+    def backward():
+        ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=config.scale)
+
+    def both():
+        o, l = ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
+        ct.attention_backward(q, k, v, metadata, o, l, dout, scale=config.scale)
+
+    result = {}
+    no_events = lambda: ct.profiling.KernelTimer(only=())  # a timer that records nothing
+    for name, function, flops in (("forward", forward, attention["flops"]["fwd"]),
+                                  ("backward", backward, attention["flops"]["bwd"])):
+        # (as many untimed launches of the half as the preamble has halves of full steps)
+        elapsed, _ = timed_region(torch, function, steps, warmup, no_events, preamble=2 * preamble_steps)
+        ms = elapsed / steps * 1e3
+        result[name] = {"ms": ms, "mask_aware_tflops": flops / (ms * 1e-3) / 1e12,
+                        "distribution": step_time_distribution(torch, function, steps, warmup, 2 * preamble_steps)}
+    result["step_distribution"] = step_time_distribution(torch, both, steps, warmup, preamble_steps)
+    return result
+
+
 def bench_backward_forms(ct, torch, config, attention, steps, warmup, preamble_steps):
     """The same step with the other forms of the backward pinned (ct_attn_bwd_args.variant), for the
     record: dQ from dS blocks that the dK/dV kernel stores, and the wide dK/dV kernel."""
@@ -374,11 +438,24 @@ def bench_cutce(ct, torch, steps, warmup, logits_cache=True):
     gemm = 2 * active * config.hidden * config.vocab
     per_kernel_flops = {"cutce_stats_kernel": gemm, "cutce_dhidden_kernel": gemm, "cutce_dhead_kernel": gemm,
                         "cutce_dlogits_kernel": gemm, "cutce_grads_kernel": 2 * gemm}  # dHidden + dHead in one launch
+    # the HBM-bound passes over per-row statistics: the merge of the per-chunk (max, sum exp, target
+    # logit) partials into lse and the loss terms reads 12 bytes per (vocabulary chunk of 1024, active
+    # row) and the weights, and writes lse; the row packing copies the active hidden rows
+    chunks = -(-(-(-config.vocab // 256)) // 4)
+    per_kernel_bytes = {
+        "cutce_merge_kernel": chunks * active * 12 + 8 * active + 8 * config.rows,
+        "cutce_pack_rows_kernel": 2 * active * config.hidden * 2,
+    }
+    if logits_cache:
+        per_kernel_bytes["cutce_dlogits_cached_kernel"] = (-(-active // 256) * 256) * config.vocab * 6
     table = []
     for name, durations in kernels.items():
         entry = {"kernel": name, "launches": len(durations), "avg_ms": mean(durations)}
         if name in per_kernel_flops:
             entry["algorithmic_tflops"] = per_kernel_flops[name] / (entry["avg_ms"] * 1e-3) / 1e12
+        if name in per_kernel_bytes:
+            entry["algorithmic_gbps"] = per_kernel_bytes[name] / (entry["avg_ms"] * 1e-3) / 1e9
+            entry["frac_hbm_peak"] = entry["algorithmic_gbps"] / PEAK_HBM_GBPS
         table.append(entry)
     nll, weight_sum = state["loss"]
     gemms = [e for e in table if "algorithmic_tflops" in e]
@@ -575,6 +652,22 @@ def main():
         return 2
     ct._lib.load()
 
+    if args.only_shape or args.only_cutce:
+        # one workload for a run under a counter profiler: few steps, no clock-ramp preamble
+        if args.only_cutce:
+            entry = bench_cutce(ct, torch, args.cutce_steps or min(args.steps, 10), min(args.warmup, 3),
+                                logits_cache=False)
+            entry.pop("inputs", None)
+        else:
+            W = ct.workloads
+            config = W.ATTENTION_CONFIGS[args.only_shape]
+            step, _, pairs = attention_step_for(ct, config, W.make_attention_inputs(config, "cuda"))
+            elapsed, kernels, _ = timed_with_table(torch, ct, step, args.steps, args.warmup)
+            entry = {"shape": args.only_shape, "allowed_pairs": pairs, "ms_per_step": elapsed / args.steps * 1e3,
+                     "kernels": kernel_table(config, pairs, kernels)}
+        print(json.dumps(entry))
+        return 0
+
     attention = bench_attention(ct, torch, args.steps, args.warmup, args.preamble_steps)
     config = attention["config"]
     dominant = max((k for k in attention["kernels"] if "algorithmic_tflops" in k),
@@ -618,6 +711,8 @@ def main():
         # the same step replayed from a captured HIP graph (not the headline: `value` is the eager step)
         "graph_replay_ms_per_step": attention["graph_replay_ms_per_step"],
     }
+    result["forward_backward"] = bench_forward_backward_split(ct, torch, config, attention, args.steps, args.warmup,
+                                                              args.preamble_steps)
     result["backward_forms"] = bench_backward_forms(ct, torch, config, attention, min(args.steps, 50),
                                                     min(args.warmup, 10), args.preamble_steps)
     result["delta_pass"] = bench_delta_pass(ct, torch, config, attention["inputs"]["q"])

@@ -330,56 +330,87 @@ __global__ __launch_bounds__(256) void cutce_stats_kernel(CutceParams p, float* 
 // ---------------------------------------------------------------------------
 // merge + finalize
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void cutce_merge_kernel(CutceParams p, const float* part,
-                                                          int chunks, float* lse_out,
-                                                          double* block_sums) {
-  __shared__ double red[2][4];
-  const int tid = threadIdx.x;
-  const int slot = blockIdx.x * 256 + tid;
+// A workgroup merges the per-chunk partials of kMergeSlots row slots: kMergeParts threads per slot
+// each walk every kMergeParts-th vocabulary chunk (so a row's chain of dependent loads is an
+// eighth as long and eight times as many loads are in flight: the pass is bound by the bytes of
+// the partials, not by their latency), then the parts are combined in a fixed order.
+constexpr int kMergeSlots = 32, kMergeParts = 8;
+__global__ __launch_bounds__(kMergeSlots * kMergeParts) void cutce_merge_kernel(CutceParams p, const float* part,
+                                                                                int chunks, float* lse_out,
+                                                                                double* block_sums) {
+  __shared__ float exch[kMergeParts][kMergeSlots][3];
+  __shared__ double red[2][kMergeSlots];
+  const int tid = threadIdx.x, lane_slot = tid % kMergeSlots, piece = tid / kMergeSlots;
+  const int slot = blockIdx.x * kMergeSlots + lane_slot;
   const int n_act = p.header->n_act;
   double loss = 0.0, wsum = 0.0;
-  if (slot < p.N) {
+  if (piece == 0 && slot < p.N) {
     const float wi = p.weights[slot];
     wsum = (double)wi;
     if (wi == 0.f) lse_out[slot] = 0.f;
   }
+  int row = 0;
+  float wr = 0.f;
   if (slot < n_act) {
-    const int row = p.idx[slot];
-    const float wr = p.weights[row];
+    row = p.idx[slot];
+    wr = p.weights[row];
+  }
+  float m = kNegInfF, s = 0.f, t = 0.f;
+  if (wr != 0.f) {
+    for (int c = piece; c < chunks; c += kMergeParts) {
+      const float* e = part + ((size_t)c * p.n_pad + slot) * 3;
+      merge_stats(m, s, e[0], e[1]);
+      t += e[2];
+    }
+  }
+  exch[piece][lane_slot][0] = m;
+  exch[piece][lane_slot][1] = s;
+  exch[piece][lane_slot][2] = t;
+  __syncthreads();
+  if (piece == 0) {
     if (wr != 0.f) {
-      float m = kNegInfF, s = 0.f, t = 0.f;
-      for (int c = 0; c < chunks; ++c) {
-        const float* e = part + ((size_t)c * p.n_pad + slot) * 3;
-        merge_stats(m, s, e[0], e[1]);
-        t += e[2];
+      for (int k = 1; k < kMergeParts; ++k) {
+        merge_stats(m, s, exch[k][lane_slot][0], exch[k][lane_slot][1]);
+        t += exch[k][lane_slot][2];
       }
       const float lse = (__log2f(s) + m) * kLn2;
       lse_out[row] = lse;
       loss = (double)wr * ((double)lse - (double)t);
     }
-  }
-  for (int off = 32; off > 0; off >>= 1) {
-    loss += __shfl_xor(loss, off, 64);
-    wsum += __shfl_xor(wsum, off, 64);
-  }
-  if ((tid & 63) == 0) {
-    red[0][tid >> 6] = loss;
-    red[1][tid >> 6] = wsum;
+    red[0][lane_slot] = loss;
+    red[1][lane_slot] = wsum;
   }
   __syncthreads();
   if (tid == 0) {
-    block_sums[2 * blockIdx.x + 0] = red[0][0] + red[0][1] + red[0][2] + red[0][3];
-    block_sums[2 * blockIdx.x + 1] = red[1][0] + red[1][1] + red[1][2] + red[1][3];
+    double loss_sum = 0.0, weight_sum = 0.0;
+    for (int k = 0; k < kMergeSlots; ++k) {  // fixed order
+      loss_sum += red[0][k];
+      weight_sum += red[1][k];
+    }
+    block_sums[2 * blockIdx.x + 0] = loss_sum;
+    block_sums[2 * blockIdx.x + 1] = weight_sum;
   }
 }
 
 __global__ __launch_bounds__(64) void cutce_finalize_kernel(const double* block_sums, int blocks,
                                                             float* nll_sum, float* weight_sum) {
-  if (threadIdx.x != 0) return;
+  // lane l adds the blocks l, l + 64, ... in order, then the lanes are added in order: the
+  // result does not depend on timing
+  __shared__ double red[2][64];
   double loss = 0.0, wsum = 0.0;
-  for (int b = 0; b < blocks; ++b) {
+  for (int b = threadIdx.x; b < blocks; b += 64) {
     loss += block_sums[2 * b];
     wsum += block_sums[2 * b + 1];
+  }
+  red[0][threadIdx.x] = loss;
+  red[1][threadIdx.x] = wsum;
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  loss = 0.0;
+  wsum = 0.0;
+  for (int k = 0; k < 64; ++k) {
+    loss += red[0][k];
+    wsum += red[1][k];
   }
   *nll_sum = (float)loss;
   *weight_sum = (float)wsum;
@@ -710,7 +741,7 @@ static FwdLayout fwd_layout(const ct_cutce_shape& s) {
   L.idx = align_up(sizeof(CutceHeader), 256);
   L.part = L.idx + align_up((size_t)n_pad * sizeof(int), 256);
   L.sums = L.part + align_up((size_t)stats_chunks(s.vocab) * n_pad * 3 * sizeof(float), 256);
-  L.total = L.sums + align_up((size_t)(n_pad / kGemmTile) * 2 * sizeof(double), 256);
+  L.total = L.sums + align_up((size_t)(n_pad / kMergeSlots) * 2 * sizeof(double), 256);
   return L;
 }
 
@@ -870,12 +901,13 @@ static int32_t cutce_fwd_on(void* stream_, const ct_cutce_fwd_args* a, void* ws_
                        chunks, static_cast<float*>(nullptr));
   if ((rc = scope2.done())) return rc;
 
+  const int merge_blocks = p.n_pad / kMergeSlots;
   LaunchScope scope3("cutce_merge_kernel", stream);
-  hipLaunchKernelGGL(cutce_merge_kernel, dim3(row_blocks), dim3(256), 0, stream, p, part, chunks,
-                     a->lse, sums);
+  hipLaunchKernelGGL(cutce_merge_kernel, dim3(merge_blocks), dim3(kMergeSlots * kMergeParts), 0, stream, p, part,
+                     chunks, a->lse, sums);
   if ((rc = scope3.done())) return rc;
   LaunchScope scope4("cutce_finalize_kernel", stream);
-  hipLaunchKernelGGL(cutce_finalize_kernel, dim3(1), dim3(64), 0, stream, sums, row_blocks,
+  hipLaunchKernelGGL(cutce_finalize_kernel, dim3(1), dim3(64), 0, stream, sums, merge_blocks,
                      a->nll_sum, a->weight_sum);
   return scope4.done();
 }

@@ -145,6 +145,65 @@ def private_accumulators(assembly: str, kernel: str) -> list[str]:
     return problems
 
 
+def block_mix(assembly: str, kernel: str) -> list[dict]:
+    """Instruction mix of every basic block of `kernel` (the first function whose label contains the
+    name): a list of {"label", "valu", "exp", "max3", "mfma", "salu", "lds", "vmem"} in program order.
+    "valu" counts vector ALU instructions other than MFMA (v_exp and v_max3 included; they are also
+    counted on their own). Used to hold the steady-state paths of the attention kernels to an
+    instruction budget per MFMA."""
+
+    blocks, inside, found = [], False, False
+    current = None
+
+    def start(label):
+        nonlocal current
+        current = {"label": label, "valu": 0, "exp": 0, "max3": 0, "mfma": 0, "salu": 0, "lds": 0, "vmem": 0}
+        blocks.append(current)
+
+    for line in assembly.splitlines():
+        text = line.strip()
+        fallthrough = re.match(r"; %bb\.(\d+):", text)
+        if fallthrough and inside:
+            start("%bb." + fallthrough.group(1))  # a block entered by falling through has no label of its own
+            continue
+        if not text or text.startswith((";", "//")):
+            continue
+        function = re.match(r"([A-Za-z_][\w$]*):", text)
+        if function and not text.startswith(".L"):
+            if found and inside:
+                break                      # next function: done
+            inside = kernel in function.group(1)
+            if inside:
+                found = True
+                start("entry")
+            continue
+        if not inside:
+            continue
+        if text.startswith(".Lfunc_end"):
+            break
+        if re.match(r"\.LBB\w+:", text):
+            start(text.split(":")[0])
+            continue
+        if text.startswith("."):
+            continue
+        op = text.split()[0]
+        if op.startswith("v_mfma"):
+            current["mfma"] += 1
+        elif op.startswith("v_"):
+            current["valu"] += 1
+            if op.startswith("v_exp"):
+                current["exp"] += 1
+            if op.startswith("v_max3"):
+                current["max3"] += 1
+        elif op.startswith("ds_"):
+            current["lds"] += 1
+        elif op.startswith(("global_", "scratch_", "buffer_", "flat_")):
+            current["vmem"] += 1
+        elif op.startswith("s_"):
+            current["salu"] += 1
+    return blocks
+
+
 def device_assembly(source: Path, flags) -> str:
     from . import build as recipe
 

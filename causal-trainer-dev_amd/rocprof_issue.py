@@ -26,8 +26,10 @@ import os
 
 from .rocprof_traffic import _short
 
-# resident wavefronts per SIMD of the kernels reported
-WAVES_PER_SIMD = {"attn_fwd_kernel": 2, "attn_dq_kernel": 2, "attn_dkv_kernel": 2}
+# resident wavefronts per SIMD of the kernels reported (launch bounds and register use fix them)
+WAVES_PER_SIMD = {"attn_fwd_kernel": 2, "attn_dq_kernel": 2, "attn_dkv_kernel": 2, "attn_dkv_wide_kernel": 1,
+                  "attn_dq_blocks_kernel": 4, "cutce_stats_kernel": 1, "cutce_dlogits_kernel": 1,
+                  "cutce_grads_kernel": 1, "cutce_dhidden_kernel": 1, "cutce_dhead_kernel": 1}
 
 
 def read_counters(folders) -> dict[str, dict[str, float]]:
@@ -46,8 +48,38 @@ def read_counters(folders) -> dict[str, dict[str, float]]:
             for kernel, counters in sums.items()}
 
 
+XCDS = 8  # GRBM_GUI_ACTIVE is reported as the sum over the accelerator dies
+
+
+def shader_clocks(folders) -> dict[str, tuple[float, float, float, int]]:
+    """kernel -> (mean, lowest, highest shader clock in GHz, dispatches) from a pass that collected
+    GRBM_GUI_ACTIVE (busy cycles of the graphics engine, summed over the dies) together with each
+    dispatch's start / end timestamps (ns). The counter window is wider than the kernel by a fixed
+    amount; the smallest value any dispatch of the pass reads (a microsecond-scale kernel) is taken
+    as that amount and subtracted, which leaves a few per cent of error on kernels under a millisecond
+    and none that matters above."""
+
+    samples = []
+    for folder in folders:
+        for path in sorted(glob.glob(os.path.join(folder, "**", "*counter_collection.csv"), recursive=True)):
+            with open(path, newline="") as handle:
+                for row in csv.DictReader(handle):
+                    if row["Counter_Name"] != "GRBM_GUI_ACTIVE":
+                        continue
+                    span = float(row["End_Timestamp"]) - float(row["Start_Timestamp"])
+                    if span > 0.0:
+                        samples.append((_short(row["Kernel_Name"]), float(row["Counter_Value"]), span))
+    if not samples:
+        return {}
+    window = min(cycles for _, cycles, _ in samples)
+    per_kernel = collections.defaultdict(list)
+    for kernel, cycles, span in samples:
+        per_kernel[kernel].append((cycles - window) / XCDS / span)
+    return {kernel: (sum(v) / len(v), min(v), max(v), len(v)) for kernel, v in per_kernel.items()}
+
+
 def summarize(counters: dict[str, dict[str, float]]) -> list[str]:
-    lines = ["%-18s %9s %9s %9s %9s %9s | %s" % ("kernel", "MFMA", "VALU", "LDS", "wait any", "wait LDS",
+    lines = ["%-22s %9s %9s %9s %9s %9s | %s" % ("kernel", "MFMA", "VALU", "LDS", "wait any", "wait LDS",
                                                   "instructions per MFMA: VALU (other than MFMA), LDS, SALU")]
     for kernel, waves in WAVES_PER_SIMD.items():
         c = counters.get(kernel)
@@ -60,7 +92,7 @@ def summarize(counters: dict[str, dict[str, float]]) -> list[str]:
             # the VALU counter includes the MFMA instructions' own issue; report the rest
             valu_time *= (c["SQ_INSTS_VALU"] - mfma) / c["SQ_INSTS_VALU"]
         per = lambda name: (c.get(name, 0.0) - (mfma if name == "SQ_INSTS_VALU" else 0.0)) / mfma if mfma else float("nan")
-        lines.append("%-18s %8.1f%% %8.1f%% %8.1f%% %8.1f%% %8.1f%% | %.1f, %.1f, %.1f" % (
+        lines.append("%-22s %8.1f%% %8.1f%% %8.1f%% %8.1f%% %8.1f%% | %.1f, %.1f, %.1f" % (
             kernel, 100 * c.get("SQ_VALU_MFMA_BUSY_CYCLES", 0.0) / simd_cycles, 100 * valu_time / simd_cycles,
             100 * 4.0 * c.get("SQ_ACTIVE_INST_LDS", 0.0) / simd_cycles,
             100 * 4.0 * c.get("SQ_WAIT_INST_ANY", 0.0) / waves / simd_cycles,
@@ -75,13 +107,21 @@ def main() -> None:
     parser.add_argument("--out", default=None)
     parser.add_argument("--command", default="")
     args = parser.parse_args()
-    lines = ["Issue-slot shares of the attention kernels (fractions of SIMD time; MFMA = matrix pipe busy, VALU = vector",
+    lines = ["Issue-slot shares of the MFMA kernels (fractions of SIMD time; MFMA = matrix pipe busy, VALU = vector",
              "ALU instructions other than MFMA executing, LDS = LDS instructions executing, wait = a wavefront waits",
              "for an instruction to issue; shares of different classes can overlap in time)"]
     if args.command:
         lines.append("command: " + args.command)
     lines.append("")
     lines += summarize(read_counters(args.folders))
+    clocks = shader_clocks(args.folders)
+    if clocks:
+        lines += ["", "shader clock during the kernel (GRBM_GUI_ACTIVE / dies / dispatch duration; the part's peak",
+                  "figures are quoted at 2.4 GHz): mean [lowest .. highest] GHz over the dispatches"]
+        for kernel in WAVES_PER_SIMD:
+            if kernel in clocks:
+                mean, low, high, count = clocks[kernel]
+                lines.append("%-22s %.2f [%.2f .. %.2f] over %d" % (kernel, mean, low, high, count))
     text = "\n".join(lines) + "\n"
     if args.out:
         with open(args.out, "w") as handle:

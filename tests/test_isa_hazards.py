@@ -79,3 +79,45 @@ def test_library_sources_have_no_scalar_base_hazard(ct):
 
     findings = isa_hazards.scan_library()
     assert findings and all(not problems for problems in findings.values()), findings
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None, reason="needs hipcc")
+def test_steady_state_paths_keep_their_instruction_budget(ct):
+    """Vector ALU instructions per MFMA on the paths an all-allowed key tile takes, read off the
+    compiled head-dimension-128 kernels. What the arithmetic alone needs per score is fma + exp2 + add
+    (+ half a max3 and half a bf16 packing) in the forward, and add, mul, exp2, add, mul (+ a
+    packing each for P and dS) in the backward: 4.0, 3.5 and 3.5 per MFMA. The kernels with two
+    wavefronts per SIMD add the rebuilding of their swizzled fragment addresses per tile (their 16
+    pointers do not fit beside the accumulators), which is the rest. The bounds hold these paths
+    where they are; masked tiles and the per-item prologue and epilogue come on top (measured
+    averages at short packed segments: 7.1, 5.9, 5.5; at long ones 4.8, 4.4)."""
+
+    from causal_trainer_dev_amd import build as recipe
+    from causal_trainer_dev_amd import isa_hazards
+
+    assembly = isa_hazards.device_assembly(recipe.CSRC / "ct_attn.hip", recipe.HIP_FLAGS)
+
+    # forward: per key tile one maximum pass (16 v_max3) and one exponent pass (32 v_exp) per wavefront,
+    # both in blocks of their own, 32 MFMAs in the generated sequences
+    forward = isa_hazards.block_mix(assembly, "attn_fwd_kernelILi128ELi4E")
+    max_passes = [b for b in forward if b["max3"] >= 16 and b["mfma"] == 0 and b["exp"] == 0]
+    exp_passes = [b for b in forward if b["exp"] >= 32 and b["mfma"] == 0]
+    assert max_passes and exp_passes
+    per_tile = max(b["valu"] for b in max_passes) + max(b["valu"] for b in exp_passes)
+    assert per_tile / 32 <= 4.6, per_tile
+
+    # dQ and dK/dV: the blocks of the key-tile loop that hold the MFMA sequences also hold the
+    # exponent / dS arithmetic of an all-allowed tile (masking sits in blocks of its own)
+    def loop_ratio(kernel, mfmas_per_step, stores_per_block=0):
+        blocks = [b for b in isa_hazards.block_mix(assembly, kernel) if b["mfma"]]
+        assert blocks and sum(b["mfma"] for b in blocks) % mfmas_per_step == 0
+        assert all(b["vmem"] <= stores_per_block for b in blocks)      # no spill traffic on these paths
+        return (sum(b["valu"] for b in blocks) / sum(b["mfma"] for b in blocks),
+                sum(b["salu"] for b in blocks) / sum(b["mfma"] for b in blocks))
+
+    dq_valu, dq_salu = loop_ratio("attn_dq_kernelILi128ELi4E", 48)
+    dkv_valu, dkv_salu = loop_ratio("attn_dkv_kernelILi128ELb0E", 32)
+    stored_valu, _ = loop_ratio("attn_dkv_kernelILi128ELb1E", 32, stores_per_block=2)   # + the dS store
+    assert dq_valu <= 4.0 and dkv_valu <= 5.2 and stored_valu <= 5.3, (dq_valu, dkv_valu, stored_valu)
+    # scalar instructions of those blocks: bounds, branches, copy bookkeeping
+    assert dq_salu <= 2.0 and dkv_salu <= 2.2, (dq_salu, dkv_salu)
