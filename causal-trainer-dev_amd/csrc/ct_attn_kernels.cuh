@@ -372,6 +372,124 @@ CT_DEVICE void qk_sequence_128(const RowFragOffsets<16>& ro, const bf16x8* qf, f
                : "memory", CT_ATTN_ASM_SCRATCH);
 }
 
+// Forward, interleaved form (see gen_attn_asm.py): statements on registers that only they name:
+// the score buffers v[112:143] ("a") and v[144:175] ("b"), a fragment ring v[176:191] and the
+// output accumulator O^T in a[0:63]. NAME = a: the scores of the current key tile are in a, P^T of
+// the tile before in the first half of b, and the next tile's scores go to b; NAME = b the other
+// way round. Every statement lists all of these registers as clobbered, so the compiler keeps no
+// value of its own there across one, and a static check of the compiled kernel
+// (isa_hazards.private_registers) proves that it uses none of them between statements either.
+// A wavefront's share of a step's global -> LDS copies, for the statement that issues them: the
+// sources (wave-uniform addresses of the V tile and the K tile), this thread's two byte offsets
+// into a tile (a tile is two pieces of 1 KB per wavefront), and the LDS destinations (the V
+// pieces, then the K pieces).
+struct FwdCopies {
+  unsigned long long v_source, k_source;
+  unsigned lane_off[2];
+  unsigned dst[4];
+};
+#define CT_FWD_TR_PTRS(to)                                                                              \
+  [lo0] "v"(to.ptr[0][0]), [lo1] "v"(to.ptr[0][1]), [lo2] "v"(to.ptr[0][2]), [lo3] "v"(to.ptr[0][3]), \
+      [hi0] "v"(to.ptr[1][0]), [hi1] "v"(to.ptr[1][1]), [hi2] "v"(to.ptr[1][2]), [hi3] "v"(to.ptr[1][3])
+#define CT_FWD_ROW_PTRS(ro, qf)                                                                          \
+  [rp0] "v"(ro.ptr[0]), [rp1] "v"(ro.ptr[1]), [rp2] "v"(ro.ptr[2]), [rp3] "v"(ro.ptr[3]),               \
+      [rp4] "v"(ro.ptr[4]), [rp5] "v"(ro.ptr[5]), [rp6] "v"(ro.ptr[6]), [rp7] "v"(ro.ptr[7]),           \
+      [q0] "v"(qf[0]), [q1] "v"(qf[1]), [q2] "v"(qf[2]), [q3] "v"(qf[3]), [q4] "v"(qf[4]), [q5] "v"(qf[5]), \
+      [q6] "v"(qf[6]), [q7] "v"(qf[7])
+#define CT_FWD_STATEMENTS(NAME, UPPER)                                                                        \
+  /* first half of the PV product | maximum of the scores (times log2 e, over the lane pair) */              \
+  template <int V_OFF>                                                                                        \
+  CT_DEVICE float fwd_max_##NAME(const TrFragOffsets<16, KSlots::kAccum>& to, const FwdCopies& cp) {         \
+    float mx, tmp;                                                                                            \
+    asm volatile(CT_FWD_MAX_##UPPER                                                                           \
+                 : [mx] "=&v"(mx), [tmp] "=&v"(tmp)                                                           \
+                 : CT_FWD_TR_PTRS(to), [c] "s"(kLog2e), [voff] "i"(V_OFF), [vsrc] "s"(cp.v_source),           \
+                   [ksrc] "s"(cp.k_source), [off0] "v"(cp.lane_off[0]), [off1] "v"(cp.lane_off[1]),           \
+                   [d0] "s"(cp.dst[0]), [d1] "s"(cp.dst[1]), [d2] "s"(cp.dst[2]), [d3] "s"(cp.dst[3])          \
+                 : "memory", "m0", CT_FWD_PRIVATE);                                                           \
+    return mx;                                                                                                \
+  }                                                                                                           \
+  /* second half of the PV product | first exponentials */                                                    \
+  template <int V_OFF>                                                                                        \
+  CT_DEVICE void fwd_exp_a_##NAME(const TrFragOffsets<16, KSlots::kAccum>& to, float m, float& psum) {       \
+    asm volatile(CT_FWD_EXP_A_##UPPER                                                                         \
+                 : [psum] "+v"(psum)                                                                          \
+                 : CT_FWD_TR_PTRS(to), [m] "v"(m), [c] "s"(kLog2e), [voff] "i"(V_OFF)                         \
+                 : "memory", CT_FWD_PRIVATE);                                                                 \
+  }                                                                                                           \
+  /* scores of the next tile | the other exponentials */                                                      \
+  template <int K_OFF>                                                                                        \
+  CT_DEVICE void fwd_exp_b_##NAME(const RowFragOffsets<16>& ro, const bf16x8* qf, float m, float& psum) {    \
+    asm volatile(CT_FWD_EXP_B_##UPPER                                                                         \
+                 : [psum] "+v"(psum)                                                                          \
+                 : CT_FWD_ROW_PTRS(ro, qf), [m] "v"(m), [c] "s"(kLog2e), [koff] "i"(K_OFF)                    \
+                 : "memory", CT_FWD_PRIVATE);                                                                 \
+  }                                                                                                           \
+  CT_DEVICE float fwd_max_only_##NAME() {                                                                     \
+    float mx, tmp;                                                                                            \
+    asm volatile(CT_FWD_MAX_ONLY_##UPPER                                                                      \
+                 : [mx] "=&v"(mx), [tmp] "=&v"(tmp)                                                           \
+                 : [c] "s"(kLog2e)                                                                            \
+                 : "memory", CT_FWD_PRIVATE);                                                                 \
+    return mx;                                                                                                \
+  }                                                                                                           \
+  CT_DEVICE void fwd_exp_only_##NAME(float m, float& psum) {                                                  \
+    asm volatile(CT_FWD_EXP_ONLY_##UPPER                                                                      \
+                 : [psum] "+v"(psum)                                                                          \
+                 : [m] "v"(m), [c] "s"(kLog2e)                                                                \
+                 : "memory", CT_FWD_PRIVATE);                                                                 \
+  }                                                                                                           \
+  template <int V_OFF>                                                                                        \
+  CT_DEVICE void fwd_pv_##NAME(const TrFragOffsets<16, KSlots::kAccum>& to) {                                \
+    asm volatile(CT_FWD_PV_##UPPER : : CT_FWD_TR_PTRS(to), [voff] "i"(V_OFF) : "memory", CT_FWD_PRIVATE);     \
+  }                                                                                                           \
+  template <int V_OFF>                                                                                        \
+  CT_DEVICE void fwd_pv_late_##NAME(const TrFragOffsets<16, KSlots::kAccum>& to) {                           \
+    asm volatile(CT_FWD_PV_LATE_##UPPER : : CT_FWD_TR_PTRS(to), [voff] "i"(V_OFF) : "memory", CT_FWD_PRIVATE); \
+  }                                                                                                           \
+  /* scores of the next tile into the other buffer */                                                         \
+  template <int K_OFF>                                                                                        \
+  CT_DEVICE void fwd_qk_##NAME(const RowFragOffsets<16>& ro, const bf16x8* qf) {                             \
+    asm volatile(CT_FWD_QK_##UPPER : : CT_FWD_ROW_PTRS(ro, qf), [koff] "i"(K_OFF) : "memory", CT_FWD_PRIVATE); \
+  }                                                                                                           \
+  /* -inf where the key's offset in the tile exceeds rel (per lane) */                                        \
+  CT_DEVICE void fwd_mask_causal_##NAME(int rel) {                                                            \
+    asm volatile(CT_FWD_MASK_CAUSAL_##UPPER                                                                   \
+                 :                                                                                            \
+                 : [rel] "v"(rel), [ninf] "v"(kNegInf)                                                        \
+                 : "memory", "vcc", CT_FWD_PRIVATE);                                                          \
+  }                                                                                                           \
+  /* -inf where bit r of bits0 / bits1 (register r of key block 0 / 1) is clear */                            \
+  CT_DEVICE void fwd_mask_bits_##NAME(unsigned bits0, unsigned bits1) {                                       \
+    int tmp;                                                                                                  \
+    asm volatile(CT_FWD_MASK_BITS_##UPPER                                                                     \
+                 : [tmp] "=&v"(tmp)                                                                           \
+                 : [bits0] "v"(bits0), [bits1] "v"(bits1), [ninf] "v"(kNegInf)                                \
+                 : "memory", "vcc", CT_FWD_PRIVATE);                                                          \
+  }
+CT_FWD_STATEMENTS(a, A)
+CT_FWD_STATEMENTS(b, B)
+
+// The output accumulator in a[0:63]: cleared, multiplied by the row's factor (one per lane), and
+// read out as the four 32-column blocks of O^T.
+CT_DEVICE void fwd_acc_zero() { asm volatile(CT_FWD_ACC_ZERO : : : "memory", CT_FWD_PRIVATE); }
+CT_DEVICE void fwd_acc_scale(float alpha) {
+  asm volatile(CT_FWD_ACC_SCALE : : [alpha] "v"(alpha) : "memory", CT_FWD_PRIVATE);
+}
+template <int INDEX>
+CT_DEVICE f32x16 fwd_acc_read() {
+  float v[16];
+  asm volatile(CT_DKVW_READ
+               : "=v"(v[0]), "=v"(v[1]), "=v"(v[2]), "=v"(v[3]), "=v"(v[4]), "=v"(v[5]), "=v"(v[6]), "=v"(v[7]),
+                 "=v"(v[8]), "=v"(v[9]), "=v"(v[10]), "=v"(v[11]), "=v"(v[12]), "=v"(v[13]), "=v"(v[14]), "=v"(v[15])
+               : "i"(16 * INDEX)
+               : "memory");
+  f32x16 out;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) out[e] = v[e];
+  return out;
+}
+
 // dQ kernel, one 32-key half of a key tile (see gen_attn_asm.py): S^T and dP^T of the half, and
 // the half's contribution to dQ^T. K_OFF / V_OFF are the byte offsets of the half's K and V rows.
 template <int K_OFF, int V_OFF>
@@ -399,6 +517,25 @@ CT_DEVICE void dq_acc_half_128(const TrFragOffsets<16, KSlots::kAccum>& to, bf16
 // ---------------------------------------------------------------------------
 // Forward
 //
+// One workgroup of 8 wavefronts per compute unit (wavefronts w and w + 4 share a SIMD), each with
+// 32 query rows of one head. Two forms of the key-tile loop:
+//
+// D = 128, interleaved (attn_fwd_item). Per key tile t a wavefront has three pieces of work: the
+// softmax arithmetic of tile t (vector ALU), O += V(t-1)^T P(t-1)^T and S(t+1)^T = K(t+1) Q^T
+// (32 MFMAs). They are independent of each other, so the arithmetic is issued between the MFMAs
+// of the same wavefront (three asm statements per tile, see gen_attn_asm.py): about five vector
+// instructions fit behind an MFMA without delaying the next one, and the matrix pipe does not
+// wait for a separate arithmetic phase. The first and the last tile of a query tile, tiles that a
+// wavefront's rows do not see, and tiles on which the running maximum has to move take the same
+// pieces one after the other (same instructions on the same registers: same bits). The scores
+// never leave the registers that those statements name.
+// LDS holds 2 stages; stage s = V rows of tile s and K rows of tile s + 2, exactly what the step
+// of tile s + 1 reads. The copies for stage t are issued at the start of the step of tile t, into
+// the buffer that the step before has finished with, and awaited at its end, in front of the one
+// workgroup barrier per step. Segment ids of the key tiles go through a ring of 4 slots (tile t
+// in slot t % 4, copied together with its K rows, read in the step of tile t).
+//
+// Other head sizes, phased (attn_fwd_item_phased):
 // One workgroup of 8 wavefronts per compute unit: wavefronts w and w + 4 share
 // a SIMD. Per key tile a wavefront alternates between a VALU phase (softmax of
 // the tile's scores) and an MFMA phase (O += V^T P of this tile, then the
@@ -458,6 +595,41 @@ struct VkFetcher {
     if (s <= last) issue_v(s, stage);
     if (s + 1 <= last) issue_k(s + 1, stage, lds0);
   }
+  // Stage s = V(s), K(s + 2) as the operands of a statement that issues this wavefront's copies
+  // itself. A K tile past `last` is replaced by tile `last` (copied to where nothing reads it):
+  // the statement has no branches.
+  static constexpr int kPasses = decltype(dma)::kPasses;
+  // this thread's offsets and this wavefront's LDS destinations for copies into `stage`
+  CT_DEVICE FwdCopies stage_destinations(lds_addr stage) const {
+    static_assert(kPasses == 2, "two pieces per tile and wavefront");
+    const int wave = uniform(threadIdx.x >> 6);
+    FwdCopies c;
+#pragma unroll
+    for (int n = 0; n < kPasses; ++n) {
+      c.lane_off[n] = dma.lane_off[n];
+      c.dst[n] = uniform((int)(unsigned)(uintptr_t)(stage + VkStage<D>::kV + (n * kFwdWaves * 64 + wave * 64) * 16));
+      c.dst[kPasses + n] =
+          uniform((int)(unsigned)(uintptr_t)(stage + VkStage<D>::kK + (n * kFwdWaves * 64 + wave * 64) * 16));
+    }
+    return c;
+  }
+  CT_DEVICE FwdCopies stage_copies(int s, int last, lds_addr stage) const {
+    const auto scalar64 = [](const char* ptr) {
+      const unsigned long long b = (unsigned long long)(uintptr_t)ptr;
+      const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
+      const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
+      return ((unsigned long long)hi << 32) | (unsigned long long)lo;
+    };
+    FwdCopies c = stage_destinations(stage);
+    c.v_source = scalar64(vbase + (size_t)s * kKeyTile * row_stride_bytes);
+    c.k_source = scalar64(kbase + (size_t)min(s + 2, last) * kKeyTile * row_stride_bytes);
+    return c;
+  }
+  // the segment ids that go with the K rows of tile s + 2
+  CT_DEVICE void issue_ids_two_ahead(int s, int last, lds_addr lds0) const {
+    if (s + 2 <= last && threadIdx.x < 16)
+      dma16_s(segb + (s + 2) * kKeyTile, threadIdx.x * 16, lds0 + VkStage<D>::seg_slot(s + 2));
+  }
 };
 
 // What a query tile reads from memory before its first key tile can be fetched, read ahead by the
@@ -498,7 +670,7 @@ struct FwdAhead {
 // return. The request is unconditional (the last tile of a workgroup names itself again): a
 // conditional one would keep the old Q registers alive through the whole tile.
 template <int D, int HS>
-CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int next_b,
+CT_DEVICE void attn_fwd_item_phased(const AttnParams& p, FwdAhead<D, HS>& ahead, int next_b,
                              int next_qt, int kvh, int slice, const lds_addr lds0,
                              const RowFragOffsets<D / 8>& ro,
                              const TrFragOffsets<D / 8, KSlots::kAccum>& to) {
@@ -693,6 +865,342 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
   __builtin_amdgcn_s_barrier();
 }
 
+// store_rows_t for the accumulator in a[0:63] (D = 128), one 32-column block in registers at a time.
+CT_DEVICE void fwd_store_rows(float row_scale, lds_addr patch, bf16* gbase, size_t row_stride) {
+  constexpr int D = 128, CPR = D / 8;
+  int l = lane_id();
+  asm volatile("" : "+v"(l));  // (as in store_rows_t: the patch addresses are formed here)
+  const int j = l & 31, half = l >> 5;
+  auto block = [&](auto db_tag) {
+    constexpr int db = decltype(db_tag)::value;
+    const f32x16 acc = fwd_acc_read<db>();
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      const int d0 = db * 32 + 8 * qd + 4 * half;
+      bf16x4 pk;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pk[e] = (bf16)(acc[4 * qd + e] * row_scale);
+      lds_store<bf16x4>(patch + tile_byte_offset<CPR>(j, d0 >> 3) + (d0 & 4) * 2, pk);
+    }
+  };
+  block(std::integral_constant<int, 0>{});
+  block(std::integral_constant<int, 1>{});
+  block(std::integral_constant<int, 2>{});
+  block(std::integral_constant<int, 3>{});
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int n = 0; n < 32 * CPR / 64; ++n) {
+    const int e = l + 64 * n;
+    const int row = e / CPR, c = e % CPR;
+    const u32x4 val = lds_load<u32x4>(patch + tile_byte_offset<CPR>(row, c));
+    store_global16(gbase + (size_t)row * row_stride + c * 8, val);
+  }
+}
+
+// One query tile, interleaved form (D = 128). Arguments as attn_fwd_item_phased.
+template <int D, int HS>
+CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int next_b,
+                             int next_qt, int kvh, int slice, const lds_addr lds0,
+                             const RowFragOffsets<D / 8>& ro,
+                             const TrFragOffsets<D / 8, KSlots::kAccum>& to) {
+  static_assert(D == 128, "the interleaved statements are written for D = 128");
+  constexpr int kStage = VkStage<D>::kBytes;
+  constexpr int kV = VkStage<D>::kV, kK = VkStage<D>::kK;
+  const QueryTileContext<D, HS, kFwdWaves> ctx(p, ahead.b, kvh, slice, ahead.qt, ahead.bounds, ahead.seg_q,
+                                                ahead.end_q);
+
+  const int w = threadIdx.x >> 6;
+  const size_t q_row_stride = (size_t)p.Hq * D;
+  const size_t kv_row_stride = (size_t)p.Hkv * D;
+
+  fwd_acc_zero();
+  float m_run = kNegInf;  // softmax reference (a recent running max), log2 domain
+  float l_run = 0.f;      // this lane's share of the running sum (f32: the LSE is held to 1e-3)
+
+  const VkFetcher<D> fetch(ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride);
+  int t = ctx.first;
+  const int last = ctx.last;
+  const bool any_tile = t <= last;
+  KeyTileBounds kb = {0, 0, 0}, nb = {0, 0, 0};  // bounds of tiles t and t + 1
+  bool visit = false;       // does this wavefront see tile t (its scores are in the buffer of t)
+  bool visit_prev = false;  // ... tile t - 1 (P^T in the other buffer, PV product still to do)
+  if (any_tile) {
+    // K rows of the first two tiles (they belong to stages first - 2 and first - 1), and the V rows
+    // of the first: its place in stage `first` is free already, only the K half of that stage has
+    // to wait until K(first) has been read
+    fetch.issue_k(t, lds0, lds0);
+    if (t + 1 <= last) fetch.issue_k(t + 1, lds0 + kStage, lds0);
+    fetch.issue_v(t, lds0);
+    kb = key_tile_bounds(ctx.meta_b, t);
+    if (t + 1 <= last) nb = key_tile_bounds(ctx.meta_b, t + 1);
+    visit = ctx.wave_visits(kb, t);
+  }
+  // Which of the 64 tiles from `chart_base` on this wavefront sees (bit j of `seen`: tile
+  // chart_base + j) and sees in full, without a mask (`plain`): lane j looks at tile chart_base + j.
+  int chart_base = 0;
+  unsigned long long seen = 0, plain = 0;
+  auto chart = [&](int base) {
+    chart_base = base;
+    const int tj = base + lane_id_here();
+    bool sees = false, full = false;
+    if (tj >= ctx.first && tj <= last) {
+      const int* a = ctx.meta_b + (size_t)(2 * tj) * kMetaW;
+      const int* c = a + kMetaW;
+      const int a_min = a[kMinNz], c_min = c[kMinNz];
+      const int k_min = a_min == 0 ? c_min : (c_min == 0 ? a_min : min(a_min, c_min));
+      const int k_max = max(a[kMaxId], c[kMaxId]);
+      const int k_uniform = (a[kUniform] == c[kUniform]) ? a[kUniform] : 0;
+      sees = blocks_interact(ctx.mine.min_nz, ctx.mine.max_id, ctx.mine.end_max, k_min, k_max, tj * kKeyTile);
+      const bool need_seg = ctx.mine.uniform == 0 || ctx.mine.uniform != k_uniform;
+      const bool need_causal = tj * kKeyTile + kKeyTile - 1 > ctx.mine.end_min;
+      full = sees && !need_seg && !need_causal;
+    }
+    seen = __ballot(sees);
+    plain = __ballot(full);
+  };
+  // (charted here: its loads travel with the first copies)
+  if (any_tile) chart(t - 1);
+  // the next tile's bounds: scalar loads behind this tile's first copies; nothing here uses them
+  ahead.request_bounds(p, next_b, kvh, slice, next_qt);
+  // (the Q rows are touched only now: the first copies above needed nothing but the bounds)
+  bf16x8 qf[D / 16];
+#pragma unroll
+  for (int ks = 0; ks < D / 16; ++ks) qf[ks] = scale_bf16x8(as_bf16x8(ahead.q[ks]), p.scale);
+  dma_wait_all();
+  __syncthreads();
+  if (visit) fwd_qk_b<kK>(ro, qf);  // (statement "b" writes buffer a: the first tile counts even)
+  // every wavefront has read K(first): the first step's copies may replace it
+  __builtin_amdgcn_s_barrier();
+
+  // The running reference m_run only follows the true maximum when that has grown by more than
+  // kRescaleSlack (log2 units): probabilities are then at most 2^slack, well inside bf16 / f32
+  // range, the normalisation by the row sum is unchanged, and the accumulator is rescaled on few
+  // tiles instead of most.
+  auto must_rescale = [&](float mx) { return __any(mx > m_run + kRescaleSlack) != 0; };
+  auto rescale = [&](float mx) {
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = (m_new == kNegInf) ? 0.f : m_new;
+    const float alpha = exp2_fast(m_run - m_use);  // m_run = -inf -> 0
+    l_run *= alpha;
+    // (rows without a finite reference have seen no key yet: their sums are still zero, and on a
+    // query tile's first key tile that is every row)
+    if (__any(m_run != kNegInf)) fwd_acc_scale(alpha);
+    m_run = m_new;
+  };
+
+  // The step of tile t. PARITY = (t - first) & 1: the scores of tile t are in buffer a (0) or b
+  // (1), stage t - 1 (V(t - 1), K(t + 1)) is in LDS buffer 1 - PARITY, stage t goes to PARITY.
+  auto step = [&](auto parity_tag) {
+    constexpr int PARITY = decltype(parity_tag)::value;
+    constexpr int V_OFF = (1 - PARITY) * kStage + kV, K_OFF = (1 - PARITY) * kStage + kK;
+    const bool visit_next = t < last && ctx.wave_visits(nb, t + 1);
+    // the copies of stage t: inside the first statement where the step runs the interleaved ones
+    const bool interleaved = visit_prev && visit && visit_next;
+    if (interleaved) {
+      fetch.issue_ids_two_ahead(t, last, lds0);
+    } else {
+      if (t != ctx.first) fetch.issue_v(t, lds0 + PARITY * kStage);  // (V(first) went with the first copies)
+      if (t + 2 <= last) fetch.issue_k(t + 2, lds0 + PARITY * kStage, lds0);
+    }
+
+    if (visit) {
+      // Masks: what the summaries leave open for this tile. A key tile with one shared id X turns
+      // the id test into a per-query predicate (seg_q == X), which folds into the visible-end
+      // bound; only a key tile that mixes ids needs the per-key comparison.
+      const int k_uniform = uniform(kb.uniform);
+      const bool need_seg = ctx.mine.uniform == 0 || ctx.mine.uniform != k_uniform;
+      const bool need_causal = t * kKeyTile + kKeyTile - 1 > ctx.mine.end_min;
+      if (need_seg || need_causal) {
+        const int seg_cmp = ctx.row_valid() ? ctx.seg_q : -1;
+        if (k_uniform == 0) {
+          unsigned allow[2];
+          tile_mask(lds0 + VkStage<D>::seg_slot(t), t, seg_cmp, ctx.end_q, true, allow);
+          if constexpr (PARITY == 0) fwd_mask_bits_a(allow[0], allow[1]);
+          else fwd_mask_bits_b(allow[0], allow[1]);
+        } else {
+          // (no key of this tile is visible to a query of another id)
+          const int rel = seg_cmp != k_uniform ? -1 : ctx.end_q - t * kKeyTile - 4 * (lane_id_here() >> 5);
+          if constexpr (PARITY == 0) fwd_mask_causal_a(rel);
+          else fwd_mask_causal_b(rel);
+        }
+      }
+    }
+
+    if (interleaved) {
+      const auto copies = fetch.stage_copies(t, last, lds0 + PARITY * kStage);
+      float mx;
+      if constexpr (PARITY == 0) mx = fwd_max_a<V_OFF>(to, copies);
+      else mx = fwd_max_b<V_OFF>(to, copies);
+      if (must_rescale(mx)) {
+        if constexpr (PARITY == 0) fwd_pv_late_a<V_OFF>(to);
+        else fwd_pv_late_b<V_OFF>(to);
+        rescale(mx);
+        const float m_use = (m_run == kNegInf) ? 0.f : m_run;
+        float psum = 0.f;
+        if constexpr (PARITY == 0) {
+          fwd_exp_only_a(m_use, psum);
+          fwd_qk_a<K_OFF>(ro, qf);
+        } else {
+          fwd_exp_only_b(m_use, psum);
+          fwd_qk_b<K_OFF>(ro, qf);
+        }
+        l_run += psum;
+      } else {
+        const float m_use = (m_run == kNegInf) ? 0.f : m_run;
+        float psum = 0.f;
+        if constexpr (PARITY == 0) {
+          fwd_exp_a_a<V_OFF>(to, m_use, psum);
+          fwd_exp_b_a<K_OFF>(ro, qf, m_use, psum);
+        } else {
+          fwd_exp_a_b<V_OFF>(to, m_use, psum);
+          fwd_exp_b_b<K_OFF>(ro, qf, m_use, psum);
+        }
+        l_run += psum;
+      }
+    } else {
+      if (visit_prev) {
+        if constexpr (PARITY == 0) fwd_pv_a<V_OFF>(to);
+        else fwd_pv_b<V_OFF>(to);
+      }
+      if (visit) {
+        float mx;
+        if constexpr (PARITY == 0) mx = fwd_max_only_a();
+        else mx = fwd_max_only_b();
+        if (must_rescale(mx)) rescale(mx);
+        const float m_use = (m_run == kNegInf) ? 0.f : m_run;
+        float psum = 0.f;
+        if constexpr (PARITY == 0) fwd_exp_only_a(m_use, psum);
+        else fwd_exp_only_b(m_use, psum);
+        l_run += psum;
+      }
+      if (visit_next) {
+        if constexpr (PARITY == 0) fwd_qk_a<K_OFF>(ro, qf);
+        else fwd_qk_b<K_OFF>(ro, qf);
+      }
+    }
+    // bounds of tile t + 2, first needed one step from now: requested here, as loaded, so that the
+    // scalar loads complete under the two waits below instead of in front of the next statement
+    // (every statement starts by waiting for the wavefront's LDS and scalar loads)
+    KeyTileWords ahead_words = key_tile_words_request(ctx.meta_b, min(t + 2, last));
+    dma_wait_all();  // stage t
+    __builtin_amdgcn_s_barrier();
+    key_tile_words_wait(ahead_words);
+    visit_prev = visit;
+    visit = visit_next;
+    kb = nb;
+    nb = key_tile_bounds(ahead_words);
+    ++t;
+  };
+  // A step without decisions, for a stretch of tiles that this wavefront sees in full (no masks)
+  // between two tiles that it sees: what step() works out per tile (bounds, who sees what, which
+  // masks) is known for the whole stretch, and its scalar work, about 150 instructions that both
+  // wavefronts of a SIMD run at the same time while the matrix pipe waits, shrinks to the copy
+  // sources and the loop count.
+  unsigned long long v_source = 0, k_source = 0;  // sources of the copies of the plain step of tile t
+  const unsigned long long tile_bytes = (unsigned long long)kKeyTile * kv_row_stride * 2;
+  auto plain_step = [&](auto parity_tag) {
+    constexpr int PARITY = decltype(parity_tag)::value;
+    constexpr int V_OFF = (1 - PARITY) * kStage + kV, K_OFF = (1 - PARITY) * kStage + kK;
+    fetch.issue_ids_two_ahead(t, last, lds0);
+    auto copies = fetch.stage_destinations(lds0 + PARITY * kStage);
+    copies.v_source = v_source;
+    copies.k_source = k_source;
+    float mx;
+    if constexpr (PARITY == 0) mx = fwd_max_a<V_OFF>(to, copies);
+    else mx = fwd_max_b<V_OFF>(to, copies);
+    if (must_rescale(mx)) {
+      if constexpr (PARITY == 0) fwd_pv_late_a<V_OFF>(to);
+      else fwd_pv_late_b<V_OFF>(to);
+      rescale(mx);
+      const float m_use = (m_run == kNegInf) ? 0.f : m_run;
+      float psum = 0.f;
+      if constexpr (PARITY == 0) {
+        fwd_exp_only_a(m_use, psum);
+        fwd_qk_a<K_OFF>(ro, qf);
+      } else {
+        fwd_exp_only_b(m_use, psum);
+        fwd_qk_b<K_OFF>(ro, qf);
+      }
+      l_run += psum;
+    } else {
+      const float m_use = (m_run == kNegInf) ? 0.f : m_run;
+      float psum = 0.f;
+      if constexpr (PARITY == 0) {
+        fwd_exp_a_a<V_OFF>(to, m_use, psum);
+        fwd_exp_b_a<K_OFF>(ro, qf, m_use, psum);
+      } else {
+        fwd_exp_a_b<V_OFF>(to, m_use, psum);
+        fwd_exp_b_b<K_OFF>(ro, qf, m_use, psum);
+      }
+      l_run += psum;
+    }
+    v_source += tile_bytes;
+    if (t + 3 <= last) k_source += tile_bytes;  // (the K tile two ahead of the next step, held at `last`)
+    dma_wait_all();  // stage t
+    __builtin_amdgcn_s_barrier();
+    ++t;
+  };
+
+
+  while (t <= last) {
+    // a stretch of plain steps from tile t on: tiles u with u - 1 seen, u plain, u + 1 seen
+    if (t - chart_base >= 63) chart(t - 1);
+    const unsigned long long stretch = ((seen << 1) & plain & (seen >> 1)) >> (t - chart_base);
+    int n = (int)__builtin_ctzll(~stretch);
+    if (n > 0) {
+      v_source = (unsigned long long)(uintptr_t)(fetch.vbase + (size_t)t * tile_bytes);
+      k_source = (unsigned long long)(uintptr_t)(fetch.kbase + (size_t)min(t + 2, last) * tile_bytes);
+      if (((t - ctx.first) & 1) != 0) {
+        plain_step(std::integral_constant<int, 1>{});
+        --n;
+      }
+      for (; n >= 2; n -= 2) {
+        plain_step(std::integral_constant<int, 0>{});
+        plain_step(std::integral_constant<int, 1>{});
+      }
+      if (n != 0) plain_step(std::integral_constant<int, 0>{});
+      // back to the general step: tile t - 1 and tile t are seen, and their bounds are read again
+      visit_prev = true;
+      visit = true;
+      kb = key_tile_bounds(ctx.meta_b, t);
+      nb = key_tile_bounds(ctx.meta_b, min(t + 1, last));
+      continue;
+    }
+    if (((t - ctx.first) & 1) == 0) step(std::integral_constant<int, 0>{});
+    else step(std::integral_constant<int, 1>{});
+  }
+  // What is left is the PV product of the last tile, and no later wait of this query tile is a
+  // wait for memory: the next tile's rows are requested here and land under that product, the
+  // stores of O and the next tile's first copies.
+  ahead.request_rows(p, kvh, slice);
+  if (any_tile && visit_prev) {
+    // stage `last` is in LDS buffer (last - first) & 1, P^T(last) in the score buffer of that
+    // parity: the statement that reads it is the one of the opposite name
+    if (((last - ctx.first) & 1) == 0) fwd_pv_b<kV>(to);
+    else fwd_pv_a<kStage + kV>(to);
+  }
+  // Every copy of this tile has been waited for, so only LDS traffic has to settle before the
+  // stages become store patches (a wait for memory here would wait for the next tile's loads).
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+
+  const float l_tot = pair_sum(l_run);
+  const bool has = l_tot > 0.f;
+  const float inv = has ? 1.f / l_tot : 0.f;
+  if (ctx.active) {
+    const int le = lane_id_here();
+    const size_t stat = ((size_t)ctx.work.b * p.S + ctx.work.rb * 32 + (le & 31)) * p.Hq + ctx.work.h;
+    if (le < 32) p.lse[stat] = has ? (__logf(l_tot) + m_run * kLn2) : 0.f;
+    const lds_addr patch = lds0 + w * 32 * D * 2;
+    bf16* obase = p.out + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
+    fwd_store_rows(inv, patch, obase, q_row_stride);
+  }
+  // The store patches overlap the stages of the next item: its copies may start once every
+  // wavefront has read its patch back (LDS reads only; the global stores stay in flight).
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+}
+
 // Workgroup (group, bin): walks the query tiles of one work bin for one
 // (head slice, KV head) group. The group is the fast index, so with 8 groups a
 // group stays on one XCD (workgroup ids are dealt round robin to the 8 XCDs)
@@ -723,7 +1231,10 @@ attn_fwd_kernel(AttnParams p) {
   }
   for (; it < it_end; ++it) {
     const int next_item = uniform(region[kBins + 1 + min(it + 1, it_end - 1)]);
-    attn_fwd_item<D, HS>(p, ahead, next_item / tpr, next_item % tpr, kvh, slice, lds0, ro, to);
+    if constexpr (D == 128)
+      attn_fwd_item<D, HS>(p, ahead, next_item / tpr, next_item % tpr, kvh, slice, lds0, ro, to);
+    else
+      attn_fwd_item_phased<D, HS>(p, ahead, next_item / tpr, next_item % tpr, kvh, slice, lds0, ro, to);
   }
 }
 

@@ -257,6 +257,40 @@ CT_DEVICE KeyTileBounds key_tile_bounds(const int* meta_b, int t) {
   return out;
 }
 
+// The same in two steps, for a caller that wants the loads to complete under a wait it has anyway:
+// key_tile_words_request issues the scalar loads and returns at once (the compiler does not know
+// that the registers are still in flight, so it neither waits nor moves the loads behind the
+// caller's barrier); the caller calls key_tile_words_wait before key_tile_bounds.
+struct KeyTileWords {
+  i32x4 a, c;  // the first four words of the two row blocks' records
+};
+static_assert(kMinNz == 0 && kMaxId == 1 && kUniform == 2, "the words the requests below read");
+CT_DEVICE KeyTileWords key_tile_words_request(const int* meta_b, int t) {
+  const int* record = meta_b + (size_t)(2 * t) * kMetaW;
+  const unsigned long long b = (unsigned long long)(uintptr_t)record;
+  const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)b);
+  const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(b >> 32));
+  const unsigned long long base = ((unsigned long long)hi << 32) | (unsigned long long)lo;
+  KeyTileWords w;
+  asm volatile("s_load_dwordx4 %0, %2, 0x0\n\ts_load_dwordx4 %1, %2, %3"
+               : "=&s"(w.a), "=&s"(w.c)
+               : "s"(base), "i"(kMetaW * 4));
+  return w;
+}
+// The wait that goes with key_tile_words_request. It takes the words as operands: what is computed
+// from them cannot be scheduled in front of it.
+CT_DEVICE void key_tile_words_wait(KeyTileWords& w) {
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(w.a), "+s"(w.c));
+}
+CT_DEVICE KeyTileBounds key_tile_bounds(const KeyTileWords& w) {
+  const int a_min = w.a[kMinNz], c_min = w.c[kMinNz];
+  KeyTileBounds out;
+  out.min_nz = a_min == 0 ? c_min : (c_min == 0 ? a_min : min(a_min, c_min));
+  out.max_id = max(w.a[kMaxId], w.c[kMaxId]);
+  out.uniform = (w.a[kUniform] == w.c[kUniform]) ? w.a[kUniform] : 0;
+  return out;
+}
+
 struct QueryBlockBounds {
   int min_nz, max_id, uniform, end_min, end_max, kv_first, kv_last;
 };

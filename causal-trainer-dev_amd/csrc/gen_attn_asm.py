@@ -90,6 +90,236 @@ def qk_sequence(ahead, slots):
     return lines + TAIL
 
 
+# ---------------------------------------------------------------------------
+# Forward, interleaved form. A wavefront that runs its softmax arithmetic and its MFMAs in
+# separate stretches leaves the matrix pipe idle during the first and the vector ALU idle during
+# the second; the other wavefront of the SIMD fills only part of that. Here the arithmetic of key
+# tile t sits between the MFMAs of O += V(t-1)^T P(t-1)^T and S(t+1)^T = K(t+1) Q^T of the same
+# wavefront: about five vector instructions fit behind an MFMA without delaying the next one.
+#
+# The scores live in two buffers of 32 registers that only these statements name, v[176:207] ("a")
+# and v[208:239] ("b"); the compiler is kept out of v[176:255] (clobbers on every statement, and a
+# static check of the compiled kernel). The scores of tile t are in buffer a when t counts even
+# from the first tile of the query tile, else in b; S(t+1) is written to the other buffer while
+# the exponentials of tile t are taken in place. The bf16 pairs of P(t) go into the first 16
+# registers of the buffer they came from (pair p reads scores 2p, 2p+1 and writes register p, which
+# an earlier pair has already read), where the PV product of the next step finds them; by the time
+# S(t+2) is written over them that product has been issued.
+#
+# Per key tile, when the tile before and the tile after are there too (FWD_* statements):
+#   max:   first half of the PV product (k-steps 0, 1)   | maximum of S(t)
+#   exp_a: second half of the PV product (k-steps 2, 3)  | exponentials of scores 0..FWD_SPLIT-1
+#   exp_b: S(t+1)                                        | exponentials of the other scores
+# (an asm statement takes at most 30 operands, and the decision to move the running maximum sits
+# between the first two). Otherwise the same arithmetic and the same products as statements of
+# their own (FWD_*_ONLY, FWD_QK, FWD_PV, FWD_PV_LATE), which give the same bits.
+# ---------------------------------------------------------------------------
+FWD_S = {"a": 112, "b": 144}
+FWD_FIRST_PRIVATE = 112
+FWD_RING0 = 176          # four fragment slots of four registers
+FWD_LAST_PRIVATE = 191
+FWD_SPLIT = 10
+
+
+def other(cur):
+    return "b" if cur == "a" else "a"
+
+
+def fwd_slot(slot):
+    lo = FWD_RING0 + 4 * slot
+    return lo, lo + 3
+
+
+def fwd_acc(db):
+    return "a[%d:%d]" % (16 * db, 16 * db + 15)
+
+
+def weave(groups, valu, lead=0):
+    """MFMA groups (wait, MFMA, the fragment reads behind it) with the vector instructions spread
+    evenly behind them; `lead` of them go in front of the first group, under the first reads."""
+    out = list(valu[:lead])
+    rest = valu[lead:]
+    pos = 0
+    for gi, group in enumerate(groups):
+        out += group
+        want = (len(rest) * (gi + 1)) // len(groups)
+        out += rest[pos:want]
+        pos = want
+    return out
+
+
+def fwd_pf(cur, step):
+    """P^T fragment of k-step `step` of the tile before the one in buffer `cur`."""
+    lo = FWD_S[other(cur)] + 4 * step
+    return "v[%d:%d]" % (lo, lo + 3)
+
+
+def fwd_pv_groups(cur, steps):
+    """MFMA groups of O^T[db] += V^T frag(step, db) * P^T[step] for the given k-steps; returns
+    (head reads, groups). Operands by name: lo0-3, hi0-3, voff."""
+    order = [(step, db) for step in steps for db in range(4)]
+    n, ahead, slots = len(order), 4, 4
+
+    def load(i):
+        step, db = order[i]
+        lo, _ = fwd_slot(i % slots)
+        o = "%%[voff]+%d" % (step * 4096)
+        return ["ds_read_b64_tr_b16 v[%d:%d], %%[lo%d] offset:%s" % (lo, lo + 1, db, o),
+                "ds_read_b64_tr_b16 v[%d:%d], %%[hi%d] offset:%s" % (lo + 2, lo + 3, db, o)]
+
+    head = ["s_waitcnt lgkmcnt(0)"]
+    for i in range(min(ahead, n)):
+        head += load(i)
+    groups = []
+    for i in range(n):
+        later = min(ahead - 1, n - 1 - i)
+        step, db = order[i]
+        lo, hi = fwd_slot(i % slots)
+        g = ["s_waitcnt lgkmcnt(%d)" % (2 * later),
+             "v_mfma_f32_32x32x16_bf16 %s, v[%d:%d], %s, %s" % (fwd_acc(db), lo, hi, fwd_pf(cur, step), fwd_acc(db))]
+        if i + ahead < n:
+            g += load(i + ahead)
+        groups.append(g)
+    return head, groups
+
+
+def fwd_qk_groups(cur):
+    """MFMA groups of S(t+1)^T = K Q^T into the buffer other than `cur`. Operands by name: rp0-7
+    fragment pointers (k-step), q0-7 query fragments, koff."""
+    nxt = FWD_S[other(cur)]
+    n, ahead, slots = 16, 4, 4
+
+    def load(i):
+        ks, kb = divmod(i, 2)
+        lo, hi = fwd_slot(i % slots)
+        return ["ds_read_b128 v[%d:%d], %%[rp%d] offset:%%[koff]+%d" % (lo, hi, ks, kb * 8192)]
+
+    head = ["s_waitcnt lgkmcnt(0)"]
+    for i in range(ahead):
+        head += load(i)
+    groups = []
+    for i in range(n):
+        later = min(ahead - 1, n - 1 - i)
+        ks, kb = divmod(i, 2)
+        lo, hi = fwd_slot(i % slots)
+        dst = "v[%d:%d]" % (nxt + 16 * kb, nxt + 16 * kb + 15)
+        g = ["s_waitcnt lgkmcnt(%d)" % later,
+             "v_mfma_f32_32x32x16_bf16 %s, v[%d:%d], %%[q%d], %s" % (dst, lo, hi, ks, "0" if ks == 0 else dst)]
+        if i + ahead < n:
+            g += load(i + ahead)
+        groups.append(g)
+    return head, groups
+
+
+def fwd_exp_ops(cur, lo, hi):
+    """P = exp2(S c - m) in place for scores lo..hi-1 of buffer `cur` (lo, hi even), the running
+    sum in score order, and the bf16 pairs; ordered so that nothing reads the result of the
+    transcendental instruction directly in front of it. Operands: %[m] the reference, %[psum] the
+    sum, %[c] log2 e (scalar)."""
+    s0 = FWD_S[cur]
+    ops = []
+    for k in range(lo, hi + 2):
+        if k < hi:
+            ops.append("v_fma_f32 v%d, v%d, %%[c], -%%[m]" % (s0 + k, s0 + k))
+        if lo <= k - 1 < hi:
+            ops.append("v_exp_f32_e32 v%d, v%d" % (s0 + k - 1, s0 + k - 1))
+        if lo <= k - 2 < hi:
+            i = k - 2
+            ops.append("v_add_f32_e32 %%[psum], %%[psum], v%d" % (s0 + i))
+            if i % 2 == 1:
+                ops.append("v_cvt_pk_bf16_f32 v%d, v%d, v%d" % (s0 + i // 2, s0 + i - 1, s0 + i))
+    return ops
+
+
+def fwd_max_ops(cur):
+    """%[mx] = log2 e times the maximum of the lane pair's scores in buffer `cur`; %[tmp] scratch."""
+    s0 = FWD_S[cur]
+    ops = ["v_max3_f32 %%[mx], v%d, v%d, v%d" % (s0, s0 + 1, s0 + 2)]
+    for j in range(3, 31, 2):
+        ops.append("v_max3_f32 %%[mx], %%[mx], v%d, v%d" % (s0 + j, s0 + j + 1))
+    ops.append("v_max_f32_e32 %%[mx], %%[mx], v%d" % (s0 + 31))
+    ops += ["v_mov_b32_e32 %[tmp], %[mx]", "s_nop 1", "v_permlane32_swap_b32 %[mx], %[tmp]",
+            "v_max_f32_e32 %[mx], %[mx], %[tmp]", "v_mul_f32_e32 %[mx], %[c], %[mx]"]
+    return ops
+
+
+def flatten(head, groups):
+    return head + [ln for g in groups for ln in g]
+
+
+def fwd_statements(cur):
+    head_pv01, pv01 = fwd_pv_groups(cur, (0, 1))
+    head_pv23, pv23 = fwd_pv_groups(cur, (2, 3))
+    head_pv, pv = fwd_pv_groups(cur, (0, 1, 2, 3))
+    head_qk, qk = fwd_qk_groups(cur)
+    key_offset = lambda i: 32 * (i // 16) + 8 * ((i % 16) // 4) + (i % 16) % 4
+    s0 = FWD_S[cur]
+    causal = []
+    for i in range(32):
+        causal += ["v_cmp_le_i32_e32 vcc, %d, %%[rel]" % key_offset(i),
+                   "v_cndmask_b32_e32 v%d, %%[ninf], v%d, vcc" % (s0 + i, s0 + i)]
+    bits = []
+    for i in range(32):
+        # bit i % 16 of the block's word into the sign bit: negative = allowed
+        bits += ["v_lshlrev_b32_e32 %%[tmp], %d, %%[bits%d]" % (31 - i % 16, i // 16),
+                 "v_cmp_gt_i32_e32 vcc, 0, %[tmp]",
+                 "v_cndmask_b32_e32 v%d, %%[ninf], v%d, vcc" % (s0 + i, s0 + i)]
+    return {
+        # the three interleaved statements
+        "MAX": head_pv01 + weave(fwd_with_copies(pv01, 2), fwd_max_ops(cur)),
+        "EXP_A": head_pv23 + weave(pv23, fwd_exp_ops(cur, 0, FWD_SPLIT)),
+        "EXP_B": head_qk + weave(qk, fwd_exp_ops(cur, FWD_SPLIT, 32), lead=6) + TAIL,
+        # the same pieces on their own
+        "MAX_ONLY": fwd_max_ops(cur),
+        "EXP_ONLY": fwd_exp_ops(cur, 0, 32),
+        "PV": flatten(head_pv, pv) + TAIL,
+        "PV_LATE": flatten(head_pv23, pv23) + TAIL,
+        "QK": flatten(head_qk, qk) + TAIL,
+        # masks: scores of pairs that are not allowed become -inf. CAUSAL: key offset in the tile
+        # <= %[rel] (per lane); BITS: bit r of %[bits0] / %[bits1] set = register r of the block allowed
+        "MASK_CAUSAL": causal,
+        "MASK_BITS": bits,
+    }
+
+
+def fwd_with_copies(groups, passes):
+    """The step's global -> LDS copies of this wavefront (V rows of this tile, then K rows of the
+    tile after next: `passes` pieces of 1 KB each) placed behind the MFMAs: their issue then costs
+    the matrix pipe nothing. Copy g: m0 = %[d<g>] (LDS destination, scalar), source = scalar base
+    %[vsrc] (g < passes) or %[ksrc] plus the lane's byte offset %[off<g % passes>]. m0 is set one
+    MFMA ahead of its copy; the last copy closes the statement."""
+    out = [list(g) for g in groups]
+    n = 2 * passes
+    assert n <= len(groups)
+    for g in range(n):
+        load = "global_load_lds_dwordx4 %%[off%d], %%[%s]" % (g % passes, "vsrc" if g < passes else "ksrc")
+        out[g].append("s_mov_b32 m0, %%[d%d]" % g)
+        if g + 1 < len(groups):
+            out[g + 1] = out[g + 1][:2] + [load] + out[g + 1][2:]
+        else:
+            out.append([load])
+    return out
+
+
+def fwd_accumulator_statements():
+    """The output accumulator O^T (128 x 32 queries) lives in a[0:63], which only these statements
+    and the PV products name. ZERO; SCALE: every element times %[alpha] (per lane: the row's
+    factor), eight elements in flight through the fragment ring; the read-out uses CT_DKVW_READ."""
+    zero = ["v_accvgpr_write_b32 a%d, 0" % r for r in range(64)]
+    scale = []
+    ring = list(range(FWD_RING0, FWD_RING0 + 8))
+    for base in range(0, 64, 8):
+        scale += ["v_accvgpr_read_b32 v%d, a%d" % (ring[e], base + e) for e in range(8)]
+        scale += ["v_mul_f32_e32 v%d, %%[alpha], v%d" % (ring[e], ring[e]) for e in range(8)]
+        scale += ["v_accvgpr_write_b32 a%d, v%d" % (base + e, ring[e]) for e in range(8)]
+    return {"ZERO": zero, "SCALE": scale + ["s_nop 1"]}
+
+
+def fwd_private_clobbers():
+    return ", ".join(['"v%d"' % r for r in range(FWD_FIRST_PRIVATE, FWD_LAST_PRIVATE + 1)] +
+                     ['"a%d"' % r for r in range(64)])
+
+
 DKV_SLOTS = 5
 DKV_SCRATCH0 = 256 - 4 * DKV_SLOTS - 1  # one address temporary, then the fragment slots
 
@@ -497,13 +727,19 @@ def clobbers():
     wide = ", ".join('"v%d"' % r for r in range(W_FIRST, 256))
     accs = ", ".join('"a%d"' % r for r in range(256))
     return ("#define CT_ATTN_ASM_SCRATCH %s\n\n#define CT_DKV_ASM_SCRATCH %s\n\n#define CT_DKVW_ASM_SCRATCH %s\n\n"
-            "#define CT_DKVW_ACCUMULATORS %s\n" % (regs, dkv, wide, accs))
+            "#define CT_DKVW_ACCUMULATORS %s\n\n#define CT_FWD_PRIVATE %s\n" % (regs, dkv, wide, accs,
+                                                                             fwd_private_clobbers()))
 
 
 if __name__ == "__main__":
     print("// Generated by gen_attn_asm.py -- do not edit by hand.")
     print(emit(pv_sequence(4, 4), "CT_ATTN_PV_SEQUENCE"))
     print(emit(qk_sequence(4, 4), "CT_ATTN_QK_SEQUENCE"))
+    for cur in ("a", "b"):
+        for name, lines in fwd_statements(cur).items():
+            print(emit(lines, "CT_FWD_%s_%s" % (name, cur.upper())))
+    for name, lines in fwd_accumulator_statements().items():
+        print(emit(lines, "CT_FWD_ACC_%s" % name))
     print(emit(dq_sdp_half_sequence(), "CT_DQ_SDP_HALF_SEQUENCE"))
     print(emit(dq_acc_half_sequence(), "CT_DQ_ACC_HALF_SEQUENCE"))
     print(emit(dkv_sdp_sequence(), "CT_DKV_SDP_SEQUENCE"))

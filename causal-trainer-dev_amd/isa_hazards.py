@@ -145,6 +145,38 @@ def private_accumulators(assembly: str, kernel: str) -> list[str]:
     return problems
 
 
+def private_registers(assembly: str, kernel: str, lowest: int, highest: int) -> list[str]:
+    """Checks a kernel whose inline-assembly statements keep values in the vector registers
+    v[lowest:highest] and in accumulation registers from one statement to the next without telling
+    the compiler (the interleaved forward: score buffers, fragment ring, output accumulator):
+    outside those statements the compiled code must not name any of them."""
+
+    problems, inside, in_asm, found = [], False, False, False
+    for number, line in enumerate(assembly.splitlines(), 1):
+        text = line.strip()
+        label = re.match(r"([A-Za-z_][\w$]*):", text)
+        if label:
+            inside = kernel in label.group(1)
+            found = found or inside
+            continue
+        if not inside:
+            continue
+        if "#ASMSTART" in text:
+            in_asm = True
+        elif "#ASMEND" in text:
+            in_asm = False
+        elif not in_asm and not text.startswith((";", ".")):
+            code = text.split(";")[0]
+            if re.search(r"\ba\[?\d", code) or "accvgpr" in code:
+                problems.append(f"{kernel}: line {number} '{text}' uses an accumulation register outside the assembly statements")
+            if any(lowest <= register <= highest for register in _vector_registers(code)):
+                problems.append(f"{kernel}: line {number} '{text}' uses a vector register of v[{lowest}:{highest}] "
+                                "outside the assembly statements")
+    if not found:
+        problems.append(f"{kernel}: not found in the assembly")
+    return problems
+
+
 def block_mix(assembly: str, kernel: str) -> list[dict]:
     """Instruction mix of every basic block of `kernel` (the first function whose label contains the
     name): a list of {"label", "valu", "exp", "max3", "mfma", "salu", "lds", "vmem"} in program order.
@@ -229,6 +261,8 @@ def scan_library() -> dict[str, list[str]]:
     for path, text in zip(sources, texts):
         if path.name == "ct_attn.hip":
             findings[path.name] += private_accumulators(text, "attn_dkv_wide_kernel")
+            for heads in (1, 2, 4):
+                findings[path.name] += private_registers(text, f"attn_fwd_kernelILi128ELi{heads}E", 112, 191)
     return findings
 
 
