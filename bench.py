@@ -194,10 +194,14 @@ def attention_step_for(ct, config, inputs, **backward_pins):
     metadata = ct.prepare_attention_metadata(inputs["segment_ids"], mesh=None, profile=profile,
                                              attention_end=inputs["attention_end"])
     q, k, v, dout = inputs["q"], inputs["k"], inputs["v"], inputs["dout"]
+    # The steps stand for the layers of a model over one packing: like the tile metadata, the
+    # backward's scratch buffer and the dK/dV work list in it are shared (built by the first call).
+    workspace = ct.BackwardWorkspace()
 
     def step():
         out, lse = ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
-        ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=config.scale, **backward_pins)
+        ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=config.scale, workspace=workspace,
+                              **backward_pins)
 
     return step, metadata, pairs
 
@@ -332,16 +336,17 @@ def bench_forward_backward_split(ct, torch, config, attention, steps, warmup, pr
                                              attention_end=inputs["attention_end"])
     q, k, v, dout = inputs["q"], inputs["k"], inputs["v"], inputs["dout"]
     out, lse = ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
+    workspace = ct.BackwardWorkspace()  # as in the step of the headline: shared by the calls
 
     def forward():
         ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
 
     def backward():
-        ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=config.scale)
+        ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=config.scale, workspace=workspace)
 
     def both():
         o, l = ct.attention_forward_with_lse(q, k, v, metadata, scale=config.scale)
-        ct.attention_backward(q, k, v, metadata, o, l, dout, scale=config.scale)
+        ct.attention_backward(q, k, v, metadata, o, l, dout, scale=config.scale, workspace=workspace)
 
     result = {}
     no_events = lambda: ct.profiling.KernelTimer(only=())  # a timer that records nothing

@@ -8,6 +8,7 @@ from . import _lib, workloads  # noqa: F401
 from .efficient_attention import (  # noqa: F401
     AttentionKernelProfile,
     AttentionMetadata,
+    BackwardWorkspace,
     attention_backward,
     attention_forward_with_lse,
     default_attention_scale,

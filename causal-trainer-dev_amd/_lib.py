@@ -27,6 +27,7 @@ ATTN_BWD_DKV_NARROW = 1
 ATTN_BWD_DKV_WIDE = 2
 ATTN_BWD_DQ_RECOMPUTE = 0x10
 ATTN_BWD_DQ_FROM_DS = 0x20
+ATTN_BWD_WORK_LIST_KEPT = 0x100
 
 
 class CtError(RuntimeError):

@@ -460,8 +460,8 @@ static int launch_schedule(hipStream_t stream, const AttnParams& p, int kvh_side
 // Recompute form: the work list; dQ per query tile (evaluates S and dP itself and computes delta
 // and -lse / scale for its rows on the way); dK/dV per key tile; the sum of split chunks.
 template <int D>
-static int dispatch_bwd_recompute(hipStream_t stream, const AttnParams& p, bool wide) {
-  int rc = launch_schedule<D>(stream, p, p.Hkv);
+static int dispatch_bwd_recompute(hipStream_t stream, const AttnParams& p, bool wide, bool list_kept) {
+  int rc = list_kept ? 0 : launch_schedule<D>(stream, p, p.Hkv);
   if (rc) return rc;
   switch (heads_per_group(p.Hq, p.Hkv)) {
     case 4: rc = launch_dq<D, 4>(stream, p); break;
@@ -477,7 +477,7 @@ static int dispatch_bwd_recompute(hipStream_t stream, const AttnParams& p, bool 
 // Stored-dS form: row statistics; the work list; then per pass of KV heads the dK/dV kernel, which
 // leaves its dS blocks in the region, and dQ as a product over those blocks; the sum of split chunks.
 template <int D>
-static int dispatch_bwd_blocks(hipStream_t stream, AttnParams p, int kvh_per_pass, bool wide) {
+static int dispatch_bwd_blocks(hipStream_t stream, AttnParams p, int kvh_per_pass, bool wide, bool list_kept) {
   {
     const long tiles = (long)p.B * p.Hq * (p.S / (D == 128 ? 64 : 128));
     LaunchScope scope("attn_bwd_stats_kernel", stream);
@@ -486,7 +486,7 @@ static int dispatch_bwd_blocks(hipStream_t stream, AttnParams p, int kvh_per_pas
     int rc = scope.done();
     if (rc) return rc;
   }
-  int rc = launch_schedule<D>(stream, p, kvh_per_pass);
+  int rc = list_kept ? 0 : launch_schedule<D>(stream, p, kvh_per_pass);
   if (rc) return rc;
   for (int base = 0; base < p.Hkv; base += kvh_per_pass) {
     p.kvh_base = base;
@@ -660,7 +660,8 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   p.Hkv = a->kv_heads;
   p.scale = round_to_bf16(a->scale);
   const int kernel_choice = a->variant & 0xf, path_choice = a->variant & 0xf0;
-  CT_REQUIRE((a->variant & ~0xff) == 0 && kernel_choice <= CT_ATTN_BWD_DKV_WIDE &&
+  const bool list_kept = (a->variant & CT_ATTN_BWD_WORK_LIST_KEPT) != 0;
+  CT_REQUIRE((a->variant & ~(0xff | CT_ATTN_BWD_WORK_LIST_KEPT)) == 0 && kernel_choice <= CT_ATTN_BWD_DKV_WIDE &&
                  (path_choice == 0 || path_choice == CT_ATTN_BWD_DQ_RECOMPUTE || path_choice == CT_ATTN_BWD_DQ_FROM_DS),
              "ct_attn_bwd: unknown variant 0x%x", a->variant);
   // The wide dK/dV kernel does not store dS: asking for it settles the dQ form as well.
@@ -694,10 +695,11 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   if (plan.spill) {
     p.ds = ws + plan.ds;
     p.ds_row_blocks = plan.row_blocks;
-    return a->head_dim == 128 ? dispatch_bwd_blocks<128>(s, p, plan.kvh_per_pass, false)
-                              : dispatch_bwd_blocks<64>(s, p, plan.kvh_per_pass, false);
+    return a->head_dim == 128 ? dispatch_bwd_blocks<128>(s, p, plan.kvh_per_pass, false, list_kept)
+                              : dispatch_bwd_blocks<64>(s, p, plan.kvh_per_pass, false, list_kept);
   }
   const bool wide = a->head_dim == 128 &&
                     (wide_forced || (kernel_choice == 0 && a->seq >= kWideDkvFromSeq));
-  return a->head_dim == 128 ? dispatch_bwd_recompute<128>(s, p, wide) : dispatch_bwd_recompute<64>(s, p, wide);
+  return a->head_dim == 128 ? dispatch_bwd_recompute<128>(s, p, wide, list_kept)
+                            : dispatch_bwd_recompute<64>(s, p, wide, list_kept);
 }

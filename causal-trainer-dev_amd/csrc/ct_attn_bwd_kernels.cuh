@@ -527,6 +527,11 @@ __global__ __launch_bounds__(256) void attn_dkv_reduce_kernel(AttnParams p) {
   const int l = lane_id(), w = threadIdx.x >> 6;
   const int nrb = p.S / 32;
   const int kvh = blockIdx.x % p.Hkv, entry = blockIdx.x / p.Hkv;
+  // This is the last kernel of a backward call: it leaves the dQ kernel's work counters at zero,
+  // so that a later call on the same workspace can keep the work list and skip the kernel that
+  // builds it (and clears the counters).
+  if (blockIdx.x == 0)
+    for (int i = threadIdx.x; i < kDqCounters; i += blockDim.x) p.dq_counters[i] = 0;
   if (entry >= uniform(p.dkv_header[0])) return;
   const int2 work_entry = p.dkv_entries[entry];
   const int tile = uniform(work_entry.x), packed = uniform(work_entry.y);

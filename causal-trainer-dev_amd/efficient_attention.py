@@ -183,8 +183,33 @@ _DKV_KERNELS = {None: 0, "narrow": _lib.ATTN_BWD_DKV_NARROW, "wide": _lib.ATTN_B
 _DQ_FORMS = {None: 0, "recompute": _lib.ATTN_BWD_DQ_RECOMPUTE, "from_ds": _lib.ATTN_BWD_DQ_FROM_DS}
 
 
+class BackwardWorkspace:
+    """Scratch of the attention backward kept from call to call.
+
+    The dK/dV work list that the backward builds in its scratch buffer depends on the tile metadata,
+    the head counts and the form of the backward only. Layers that share one packing can share one
+    of these objects (``attention_backward(..., workspace=...)``,
+    ``efficient_attention(..., backward_workspace=...)``): the first call builds the list, later
+    calls with the same metadata, shape and form tell the library to keep it
+    (``CT_ATTN_BWD_WORK_LIST_KEPT``), which saves a launch per call. The calls that share one must
+    run on one stream, one after the other."""
+
+    def __init__(self):
+        self._buffer = None
+        self._built_for = None
+
+    def _acquire(self, nbytes, device, key):
+        if self._buffer is None or self._buffer.numel() < nbytes or self._buffer.device != device:
+            self._buffer = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self._built_for = None
+        return self._buffer, self._built_for == key
+
+    def _built(self, key):
+        self._built_for = key
+
+
 def _attn_backward(query, key, value, metadata, out, lse, dout, scale, with_delta=False, dkv_kernel=None,
-                   dq_form=None, workspace_bytes=None):
+                   dq_form=None, workspace_bytes=None, kept=None):
     batch, sequence, q_heads, head_dim = query.shape
     lib = _lib.load()
     dq = torch.empty_like(query)
@@ -201,7 +226,16 @@ def _attn_backward(query, key, value, metadata, out, lse, dout, scale, with_delt
                                  "exceed 64 GiB)")
         else:
             workspace_bytes = int(lib.ct_attn_bwd_workspace_bytes(*shape))
-    workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=query.device)
+    variant = _DKV_KERNELS[dkv_kernel] | _DQ_FORMS[dq_form]
+    if kept is None:
+        workspace = torch.empty(workspace_bytes, dtype=torch.uint8, device=query.device)
+    else:
+        # (the version counter of the metadata tensor changes when it is written in place)
+        built_for = (metadata.tile_bounds.data_ptr(), metadata.tile_bounds._version, shape, variant,
+                     workspace_bytes, float(scale))
+        workspace, list_kept = kept._acquire(workspace_bytes, query.device, built_for)
+        if list_kept:
+            variant |= _lib.ATTN_BWD_WORK_LIST_KEPT
     args = _lib.AttnBwdArgs(
         q=query.data_ptr(), k=key.data_ptr(), v=value.data_ptr(),
         segment_ids=metadata.query_segment_ids.data_ptr(),
@@ -211,10 +245,12 @@ def _attn_backward(query, key, value, metadata, out, lse, dout, scale, with_delt
         dq=dq.data_ptr(), dk=dk.data_ptr(), dv=dv.data_ptr(), delta=delta.data_ptr(),
         workspace=workspace.data_ptr(), workspace_bytes=workspace_bytes,
         batch=batch, seq=sequence, q_heads=q_heads, kv_heads=key.shape[2], head_dim=head_dim,
-        scale=scale, variant=_DKV_KERNELS[dkv_kernel] | _DQ_FORMS[dq_form],
+        scale=scale, variant=variant,
     )
     with torch.cuda.device(query.device):
         _lib.check(lib.ct_attn_bwd(_lib.current_stream(), args))
+    if kept is not None:
+        kept._built(built_for)
     if with_delta:
         return dq, dk, dv, delta.view(batch, q_heads, sequence)
     return dq, dk, dv
@@ -224,27 +260,31 @@ class _EfficientAttention(torch.autograd.Function):
     """Custom VJP with the reference's residual (q, k, v, metadata, O, LSE) (:1831-1863)."""
 
     @staticmethod
-    def forward(ctx, query, key, value, metadata, scale):
+    def forward(ctx, query, key, value, metadata, scale, backward_workspace=None):
         out, lse = _attn_forward(query, key, value, metadata, scale)
         ctx.save_for_backward(query, key, value, out, lse)
         ctx.attention_metadata = metadata
         ctx.scale = scale
+        ctx.backward_workspace = backward_workspace
         return out
 
     @staticmethod
     def backward(ctx, output_cotangent):
         query, key, value, out, lse = ctx.saved_tensors
         dout = output_cotangent.to(torch.bfloat16).contiguous()
-        dq, dk, dv = _attn_backward(query, key, value, ctx.attention_metadata, out, lse, dout, ctx.scale)
-        return dq, dk, dv, None, None
+        dq, dk, dv = _attn_backward(query, key, value, ctx.attention_metadata, out, lse, dout, ctx.scale,
+                                    kept=ctx.backward_workspace)
+        return dq, dk, dv, None, None, None
 
 
 def efficient_attention(query, key, value, metadata, *, mesh=None, profile=None, scale=None,
-                        causal=True):
+                        causal=True, backward_workspace=None):
     """Segment-isolated causal attention forward with its analytic custom VJP.
 
     query ``[B, S, Hq, D]``, key / value ``[B, S, Hkv, D]``, all bf16 on a ROCm
     device; returns ``[B, S, Hq, D]`` bf16. Gradients flow to query, key, value.
+    ``backward_workspace`` (this build's addition, a :class:`BackwardWorkspace`) lets the layers of
+    a model that share ``metadata`` share the scratch buffer of the backward and the work list in it.
     """
 
     if not isinstance(causal, bool):
@@ -276,7 +316,7 @@ def efficient_attention(query, key, value, metadata, *, mesh=None, profile=None,
     _validate_metadata(metadata, query_shape, resolved_profile)
     resolved_scale = default_attention_scale(query_shape[-1]) if scale is None else _python_scalar(scale)
     return _EfficientAttention.apply(
-        query.contiguous(), key.contiguous(), value.contiguous(), metadata, resolved_scale
+        query.contiguous(), key.contiguous(), value.contiguous(), metadata, resolved_scale, backward_workspace
     )
 
 
@@ -288,7 +328,7 @@ def attention_forward_with_lse(query, key, value, metadata, *, scale=None):
 
 
 def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=None, with_delta=False,
-                       dkv_kernel=None, dq_form=None, workspace_bytes=None):
+                       dkv_kernel=None, dq_form=None, workspace_bytes=None, workspace=None):
     """Backward only, from the saved residuals: returns ``(dq, dk, dv)``; with ``with_delta`` also the
     scratch ``-delta = -rowsum(out * dout)`` as the kernels leave it, head-major ``[B, Hq, S]``.
 
@@ -296,16 +336,18 @@ def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=Non
     kernel or a form of the backward for this call (``ct_attn_bwd_args.variant``); ``None`` leaves
     the choice to the library, which is what training code does (dQ recomputes; the dK/dV kernel goes
     by sequence length). ``workspace_bytes`` overrides the size of the scratch buffer (default: what
-    the library asks for the chosen form)."""
+    the library asks for the chosen form); ``workspace`` (a :class:`BackwardWorkspace`) keeps the
+    buffer, and with it the dK/dV work list, from one call to the next."""
 
     resolved = default_attention_scale(query.shape[-1]) if scale is None else float(scale)
     return _attn_backward(query, key, value, metadata, out, lse, dout.contiguous(), resolved, with_delta,
-                          dkv_kernel, dq_form, workspace_bytes)
+                          dkv_kernel, dq_form, workspace_bytes, workspace)
 
 
 __all__ = [
     "AttentionKernelProfile",
     "AttentionMetadata",
+    "BackwardWorkspace",
     "attention_backward",
     "attention_forward_with_lse",
     "default_attention_scale",

@@ -145,6 +145,14 @@ int32_t ct_attn_fwd(void* stream, const ct_attn_fwd_args* args);
 #define CT_ATTN_BWD_DKV_WIDE 2
 #define CT_ATTN_BWD_DQ_RECOMPUTE 0x10
 #define CT_ATTN_BWD_DQ_FROM_DS 0x20
+/* The dK/dV work list depends on the tile metadata, the head counts and the form of the backward
+ * only, not on the tensors: a caller that runs the backward of several layers over one packing
+ * (same tile_meta, shape, variant and workspace size) can keep the list. With this flag the call
+ * does not build it: the head of `workspace` must be as the previous ct_attn_bwd call on this
+ * workspace left it (every call leaves the list in place and the work counters of the dQ kernel at
+ * zero). One launch and 0.01 ms less per call; anything else in the workspace may be overwritten
+ * between the calls. */
+#define CT_ATTN_BWD_WORK_LIST_KEPT 0x100
 
 typedef struct ct_attn_bwd_args {
   const uint16_t* q;

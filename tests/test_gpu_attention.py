@@ -171,6 +171,41 @@ def test_default_choices_of_the_backward(ct, gpu, seq, expected):
         _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5, dq_form="from_ds", dkv_kernel="wide")
 
 
+@pytest.mark.parametrize("form", ["recompute", "from_ds"])
+def test_kept_work_list(ct, gpu, form):
+    """Layers that share a packing can share the backward's scratch buffer and the dK/dV work list
+    in it (CT_ATTN_BWD_WORK_LIST_KEPT through ct.BackwardWorkspace): the first call builds the list,
+    the next ones launch one kernel less and give the same bits, also with other tensors; another
+    packing builds it again."""
+
+    from causal_trainer_dev_amd import profiling
+
+    rng = np.random.default_rng(77)
+    batch, seq, q_heads, kv_heads, dim = 2, 1024, 4, 2, 128
+    scale = dim ** -0.5
+    layouts = [_layout(rng, batch, seq, max_len=700), _layout(rng, batch, seq, max_len=300)]
+    profile = ct.resolve_attention_profile((batch, seq, q_heads, dim), (batch, seq, kv_heads, dim), None,
+                                           has_attention_end=False)
+    kept = ct.BackwardWorkspace()
+    launches = []
+    for ids, layers in ((layouts[0], 3), (layouts[1], 2)):
+        metadata = ct.prepare_attention_metadata(torch.from_numpy(ids).to(gpu), mesh=None, profile=profile)
+        for layer in range(layers):
+            q, dout = (_bf16(rng.standard_normal((batch, seq, q_heads, dim))).to(gpu) for _ in range(2))
+            k, v = (_bf16(rng.standard_normal((batch, seq, kv_heads, dim))).to(gpu) for _ in range(2))
+            out, lse = ct.attention_forward_with_lse(q, k, v, metadata, scale=scale)
+            print("layout", len(launches), "layer", layer, form, flush=True)
+            expected = ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=scale, dq_form=form)
+            with profiling.KernelTimer() as timer:
+                got = ct.attention_backward(q, k, v, metadata, out, lse, dout, scale=scale, dq_form=form,
+                                            workspace=kept)
+            launches.append(sorted(timer.durations_ms()))
+            for a, b in zip(expected, got):
+                assert torch.equal(a, b)
+    built = ["attn_dkv_schedule_kernel" in names for names in launches]
+    assert built == [True, False, False, True, False], launches
+
+
 @pytest.mark.parametrize("scale", [0.0, 1e-37, -0.09, 1.0])
 @pytest.mark.parametrize("dim", [64, 128])
 def test_any_finite_scale(ct, gpu, bwd_variant, scale, dim):
