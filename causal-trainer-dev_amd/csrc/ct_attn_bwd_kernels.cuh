@@ -47,6 +47,42 @@ CT_DEVICE void dq_arith(f32x16& s, const f32x16& dp, float lse2, float delta_q) 
   }
 }
 
+// The 32 rows of a wavefront (one head, D elements each) as the k-contiguous MFMA fragments of its
+// lanes: row l % 32, chunks 2 ks + l / 32. Loaded directly in that form an instruction touches 32
+// rows with 32 bytes each, and the address unit of a compute unit, which handles a few cache lines
+// per cycle, needs 8-12 k cycles for the three tensors of a dQ tile (measured: a tenth of the
+// kernel at short segments). Here the lanes run along the rows instead (an instruction covers 64 /
+// CPR whole rows), and the chunks go through the wavefront's LDS patch (swizzled tile layout) to
+// the lanes that need them.
+template <int D>
+struct RowBlockLoader {
+  static constexpr int CPR = D / 8;              // 16-byte chunks per row
+  static constexpr int kRowsPerLoad = 64 / CPR;  // rows one instruction covers
+  static constexpr int kLoads = 32 / kRowsPerLoad;
+  u32x4 raw[kLoads];
+  // `first_row`: row 0 of the block for this wavefront's head; row stride in elements
+  CT_DEVICE void request(const bf16* first_row, size_t row_stride) {
+    const int l = lane_id_here();
+    const bf16* mine = first_row + (size_t)(l / CPR) * row_stride + (l % CPR) * 8;
+#pragma unroll
+    for (int n = 0; n < kLoads; ++n) raw[n] = load_global16(mine + (size_t)(n * kRowsPerLoad) * row_stride);
+  }
+  // (LDS operations of one wavefront complete in order: the reads see the writes, and the next
+  // block's writes come after these reads)
+  template <class Fragment>
+  CT_DEVICE void to_fragments(lds_addr patch, Fragment* fragments) {
+    const int l = lane_id_here();
+#pragma unroll
+    for (int n = 0; n < kLoads; ++n)
+      lds_store<u32x4>(patch + tile_byte_offset<CPR>(l / CPR + n * kRowsPerLoad, l % CPR), raw[n]);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks)
+      fragments[ks] = lds_load<Fragment>(patch + tile_byte_offset<CPR>(l & 31, 2 * ks + (l >> 5)));
+    __builtin_amdgcn_wave_barrier();
+  }
+};
+
 // One query tile (4 / HS row blocks x HS heads of one KV head), start to finish.
 template <int D, int HS>
 CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int qt, const lds_addr lds_base) {
@@ -65,18 +101,8 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
   const size_t stat_t = ((size_t)ctx.work.b * p.Hq + ctx.work.h) * p.S + ctx.pos;  // head-major
   const float lse2 = p.lse[ctx.stat_off] * kLog2e;
 
-  bf16x8 qf[D / 16], dof[D / 16];
-  u32x4 of[D / 16];  // this row's half of `out`, for delta
-#pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) {
-    qf[ks] = scale_bf16x8(as_bf16x8(load_global16(p.q + ctx.q_off + 16 * ks + 8 * half)), p.scale);
-    dof[ks] = as_bf16x8(load_global16(p.dout + ctx.q_off + 16 * ks + 8 * half));
-    of[ks] = load_global16(p.out + ctx.q_off + 16 * ks + 8 * half);
-  }
-  f32x16 dqacc[D / 32];
-#pragma unroll
-  for (int db = 0; db < D / 32; ++db) dqacc[db] = zero16();
-
+  // The first key tile's copies go first (stage 0), the rows of Q, dO and O behind them; their
+  // way into fragments leads through this wavefront's patch in stage 1, which nothing uses yet.
   const KvFetcher<D> fetch(ctx.kbase, ctx.vbase, ctx.segb, kv_row_stride);
   int t = ctx.first;
   KeyTileBounds kb = {0, 0, 0};
@@ -84,6 +110,24 @@ CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int 
     fetch.issue(t, lds0);
     kb = key_tile_bounds(ctx.meta_b, t);
   }
+  bf16x8 qf[D / 16], dof[D / 16];
+  u32x4 of[D / 16];  // this row's half of `out`, for delta
+  {
+    const size_t block_off = (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
+    const lds_addr patch = lds0 + kStage + uniform(w) * 32 * D * 2;
+    RowBlockLoader<D> q_rows, do_rows, o_rows;
+    q_rows.request(p.q + block_off, q_row_stride);
+    do_rows.request(p.dout + block_off, q_row_stride);
+    o_rows.request(p.out + block_off, q_row_stride);
+    q_rows.to_fragments(patch, qf);
+    do_rows.to_fragments(patch, dof);
+    o_rows.to_fragments(patch, of);
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks) qf[ks] = scale_bf16x8(qf[ks], p.scale);
+  }
+  f32x16 dqacc[D / 32];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db) dqacc[db] = zero16();
   dma_wait_all();
   __syncthreads();
 
