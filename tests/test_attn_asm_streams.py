@@ -99,12 +99,16 @@ class Model:
 
 
 def _sequences(gen):
-    return {
+    sequences = {
         "pv": gen.pv_sequence(4, 4), "qk": gen.qk_sequence(4, 4), "dq_sdp_half": gen.dq_sdp_half_sequence(),
         "dq_acc_half": gen.dq_acc_half_sequence(), "dkv_sdp": gen.dkv_sdp_sequence(), "dkv_acc": gen.dkv_acc_sequence(),
         "dkvw_step": gen.dkvw_step_sequence(), "dkvw_masked": gen.dkvw_step_sequence(masked=True),
         "dkvw_run": gen.dkvw_run_sequence(),
     }
+    for cur in ("a", "b"):
+        for name, lines in gen.fwd_statements(cur).items():
+            sequences["fwd_%s_%s" % (name.lower(), cur)] = lines
+    return sequences
 
 
 def test_fragment_rings_and_wait_counts(gen):
@@ -172,6 +176,112 @@ def test_wide_stream_structure(gen):
     assert len(narrowed) == 2
     for i in narrowed:
         assert lines[i + 1].startswith("global_load_lds") and lines[i + 2] == "s_mov_b64 exec, -1"
+
+
+def _vector_alu(lines):
+    return [line for line in lines if line.startswith("v_") and not line.startswith("v_mfma")]
+
+
+@pytest.mark.parametrize("cur", ["a", "b"])
+def test_forward_interleaved_statements(gen, cur):
+    """The forward's three statements per key tile: MFMA counts, how much vector work sits behind
+    an MFMA, that the statements without MFMAs run the very same vector instructions (the two forms
+    of a step must give the same bits), where the bf16 pairs go, and the copies."""
+
+    statements = gen.fwd_statements(cur)
+    s0, other = gen.FWD_S[cur], gen.FWD_S[gen.other(cur)]
+    mfmas = {name: [line for line in lines if line.startswith("v_mfma")] for name, lines in statements.items()}
+    assert [len(mfmas[name]) for name in ("MAX", "EXP_A", "EXP_B", "PV", "PV_LATE", "QK")] == [8, 8, 16, 16, 8, 16]
+    # about five vector instructions fit behind an MFMA (microbenchmark): no statement asks for more
+    for name in ("MAX", "EXP_A", "EXP_B"):
+        assert len(_vector_alu(statements[name])) / len(mfmas[name]) <= 5.0, name
+    total = sum(len(_vector_alu(statements[name])) for name in ("MAX", "EXP_A", "EXP_B"))
+    assert total / 32 <= 4.3, total
+
+    # the same vector instructions with and without the MFMAs; for the exponentials, which the
+    # interleaved form cuts into two statements (so the software pipeline drains once in between),
+    # the same instructions per score and the same order of the additions into the sum
+    assert _vector_alu(statements["MAX"]) == _vector_alu(statements["MAX_ONLY"])
+    split = _vector_alu(statements["EXP_A"]) + _vector_alu(statements["EXP_B"])
+    assert sorted(split) == sorted(_vector_alu(statements["EXP_ONLY"]))
+    additions = lambda lines: [line for line in lines if line.startswith("v_add_f32")]
+    assert additions(split) == additions(_vector_alu(statements["EXP_ONLY"]))
+    # the products of the two forms are the same MFMAs in the same order
+    assert mfmas["MAX"] + mfmas["EXP_A"] == mfmas["PV"] and mfmas["EXP_A"] == mfmas["PV_LATE"]
+    assert mfmas["EXP_B"] == mfmas["QK"]
+
+    for exponent in (_vector_alu(statements["EXP_ONLY"]), split):
+        # nothing reads the result of a transcendental instruction directly behind it
+        for before, after in zip(exponent, exponent[1:]):
+            if before.startswith("v_exp_f32"):
+                written = _registers(_split(before)[1][0])
+                assert not written & set().union(*[_registers(op) for op in _split(after)[1][1:]]), (before, after)
+        # the sum runs in score order; score i: fma, exp2, add, and its pair's packing, in that order
+        adds = [line for line in exponent if line.startswith("v_add_f32")]
+        assert [_split(line)[1][2] for line in adds] == ["v%d" % (s0 + i) for i in range(32)]
+        position = {line: index for index, line in enumerate(exponent)}
+        pack_of = lambda pair: position["v_cvt_pk_bf16_f32 v%d, v%d, v%d" % (s0 + pair, s0 + 2 * pair, s0 + 2 * pair + 1)]
+        for i in range(32):
+            register = s0 + i
+            fma = position["v_fma_f32 v%d, v%d, %%[c], -%%[m]" % (register, register)]
+            exp2 = position["v_exp_f32_e32 v%d, v%d" % (register, register)]
+            add = position["v_add_f32_e32 %%[psum], %%[psum], v%d" % register]
+            assert fma < exp2 < add < pack_of(i // 2), i
+            # the pair's packing overwrites score i // 2, whose own packing (pair i // 4) is done
+            assert pack_of(i // 4) <= pack_of(i // 2), i
+        assert sum(line.startswith("v_cvt_pk_bf16_f32") for line in exponent) == 16
+
+    # P^T of the tile before: the first 16 registers of the other buffer, k-step by k-step; the
+    # next tile's scores go to the other buffer and only the last statement writes there
+    for index, line in enumerate(mfmas["PV"]):
+        step = index // 4
+        assert _split(line)[1][2] == "v[%d:%d]" % (other + 4 * step, other + 4 * step + 3), line
+        assert _split(line)[1][0] == _split(line)[1][3] == "a[%d:%d]" % (16 * (index % 4), 16 * (index % 4) + 15)
+    for index, line in enumerate(mfmas["QK"]):
+        block = index % 2
+        assert _split(line)[1][0] == "v[%d:%d]" % (other + 16 * block, other + 16 * block + 15), line
+    for name in ("MAX", "EXP_A", "MAX_ONLY", "EXP_ONLY", "MASK_CAUSAL", "MASK_BITS"):
+        for line in statements[name]:
+            if line.startswith(("v_", "ds_read")):
+                destination = _registers(_split(line)[1][0])
+                assert not destination & set(range(other, other + 32)), (name, line)
+    # no statement names a register outside the private window (and its operands)
+    for name, lines in statements.items():
+        for line in lines:
+            named = set().union(*[_registers(op) for op in _split(line)[1]]) if " " in line else set()
+            assert all(gen.FWD_FIRST_PRIVATE <= r <= gen.FWD_LAST_PRIVATE for r in named), (name, line)
+
+    # the step's four copies ride in the first statement: V pieces, then K pieces, each with m0 set
+    # at least one instruction ahead and nothing else touching m0 in between
+    first = statements["MAX"]
+    copies = [i for i, line in enumerate(first) if line.startswith("global_load_lds")]
+    assert [first[i] for i in copies] == ["global_load_lds_dwordx4 %%[off%d], %%[%s]" % (g % 2, "vsrc" if g < 2 else "ksrc")
+                                          for g in range(4)]
+    settings = [i for i, line in enumerate(first) if line.startswith("s_mov_b32 m0")]
+    assert [first[i] for i in settings] == ["s_mov_b32 m0, %%[d%d]" % g for g in range(4)]
+    for g in range(4):
+        assert settings[g] + 1 < copies[g] and (g == 3 or copies[g] < settings[g + 1])
+    for name in ("EXP_A", "EXP_B", "PV", "PV_LATE", "QK"):
+        assert not any("m0" in line or line.startswith("global_") for line in statements[name]), name
+
+
+def test_forward_masks(gen):
+    """The mask statements: one compare and one select per score, the key offset of a score register
+    as the accumulator layout has it (block 32 kb, then 8 (r / 4) + r % 4)."""
+
+    for cur in ("a", "b"):
+        s0 = gen.FWD_S[cur]
+        causal = gen.fwd_statements(cur)["MASK_CAUSAL"]
+        assert len(causal) == 64
+        for i in range(32):
+            offset = 32 * (i // 16) + 8 * ((i % 16) // 4) + (i % 16) % 4
+            assert causal[2 * i] == "v_cmp_le_i32_e32 vcc, %d, %%[rel]" % offset
+            assert causal[2 * i + 1] == "v_cndmask_b32_e32 v%d, %%[ninf], v%d, vcc" % (s0 + i, s0 + i)
+        bits = gen.fwd_statements(cur)["MASK_BITS"]
+        assert len(bits) == 96
+        for i in range(32):
+            assert bits[3 * i] == "v_lshlrev_b32_e32 %%[tmp], %d, %%[bits%d]" % (31 - i % 16, i // 16)
+            assert bits[3 * i + 2] == "v_cndmask_b32_e32 v%d, %%[ninf], v%d, vcc" % (s0 + i, s0 + i)
 
 
 def test_committed_include_is_what_the_generator_prints(gen):
