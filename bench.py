@@ -362,11 +362,14 @@ def bench_forward_backward_split(ct, torch, config, attention, steps, warmup, pr
 
 
 def bench_backward_forms(ct, torch, config, attention, steps, warmup, preamble_steps):
-    """The same step with the other forms of the backward pinned (ct_attn_bwd_args.variant), for the
-    record: dQ from dS blocks that the dK/dV kernel stores, and the wide dK/dV kernel."""
+    """The same step with the forms of the backward pinned (ct_attn_bwd_args.variant), for the
+    record: dQ from dS blocks that the dK/dV kernel stores (what the library chooses by itself at
+    this shape, given the workspace), dQ from a second evaluation of S and dP beside the narrow and
+    beside the wide dK/dV kernel."""
 
     forms = {}
     for name, pins in (("dq_from_ds", dict(dq_form="from_ds")),
+                       ("dq_recompute", dict(dq_form="recompute", dkv_kernel="narrow")),
                        ("dq_recompute_dkv_wide", dict(dq_form="recompute", dkv_kernel="wide"))):
         step, _, _ = attention_step_for(ct, config, attention["inputs"], **pins)
         elapsed, kernels, _ = timed_with_table(torch, ct, step, steps, warmup, preamble=preamble_steps)
@@ -697,6 +700,10 @@ def main():
             "allowed_pairs": attention["pairs"],
             "flops_per_step": attention["flops"]["total"],
             "seed": config.seed,
+            # which form of the backward the library chose by itself (`backward_forms` has them all)
+            "backward_form": ("dQ from stored dS blocks" if any(k["kernel"] == "attn_dq_blocks_kernel"
+                                                                for k in attention["kernels"])
+                              else "dQ recomputes S and dP"),
         },
         "pct_bf16_mfma_peak": 100.0 * attention["tflops"] / PEAK_BF16_TFLOPS,
         "roofline": {

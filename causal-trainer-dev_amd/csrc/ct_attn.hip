@@ -668,7 +668,15 @@ extern "C" int32_t ct_attn_bwd(void* stream, const ct_attn_bwd_args* a) {
   const bool wide_forced = kernel_choice == CT_ATTN_BWD_DKV_WIDE && a->head_dim == 128;
   CT_REQUIRE(!(wide_forced && path_choice == CT_ATTN_BWD_DQ_FROM_DS),
              "ct_attn_bwd: the wide dK/dV kernel has no stored-dS form");
-  const bool allow_blocks = path_choice == CT_ATTN_BWD_DQ_FROM_DS;
+  // Left to the library (no form asked for), the stored-dS form runs where it measured faster and
+  // costs nothing the caller has not offered: rows of up to kFromDsUpToSeq positions, the narrow
+  // dK/dV kernel, and a workspace that holds the dS blocks of all KV heads at once.
+  bool allow_blocks = path_choice == CT_ATTN_BWD_DQ_FROM_DS;
+  if (path_choice == 0 && !wide_forced && a->seq <= kFromDsUpToSeq) {
+    const BwdPlan offered = bwd_plan(a->batch, a->seq, a->q_heads, a->kv_heads, a->head_dim,
+                                     a->attention_end != nullptr, a->workspace_bytes, true);
+    allow_blocks = offered.spill && offered.kvh_per_pass == a->kv_heads && a->workspace_bytes >= offered.total;
+  }
   const BwdPlan plan = bwd_plan(a->batch, a->seq, a->q_heads, a->kv_heads, a->head_dim,
                                 a->attention_end != nullptr, a->workspace_bytes, allow_blocks);
   if (a->workspace_bytes < plan.total)

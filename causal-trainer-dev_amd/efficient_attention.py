@@ -179,6 +179,10 @@ def _attn_forward(query, key, value, metadata, scale):
     return out, lse
 
 
+# Left to itself (dq_form=None) the backward offers the library the larger workspace of the
+# stored-dS form for rows of up to 4096 positions, if that is at most 4 GiB.
+_FROM_DS_UP_TO_SEQ = 4096
+_FROM_DS_WORKSPACE_CAP = 4 << 30
 _DKV_KERNELS = {None: 0, "narrow": _lib.ATTN_BWD_DKV_NARROW, "wide": _lib.ATTN_BWD_DKV_WIDE}
 _DQ_FORMS = {None: 0, "recompute": _lib.ATTN_BWD_DQ_RECOMPUTE, "from_ds": _lib.ATTN_BWD_DQ_FROM_DS}
 
@@ -218,12 +222,15 @@ def _attn_backward(query, key, value, metadata, out, lse, dout, scale, with_delt
     delta = torch.empty_like(lse)
     shape = (batch, sequence, query.shape[2], key.shape[2], head_dim)
     if workspace_bytes is None:
+        stored = int(lib.ct_attn_bwd_workspace_bytes_from_ds(*shape, int(metadata.attention_end is not None)))
         if dq_form == "from_ds":
-            workspace_bytes = int(lib.ct_attn_bwd_workspace_bytes_from_ds(
-                *shape, int(metadata.attention_end is not None)))
+            workspace_bytes = stored
             if workspace_bytes == 0:
                 raise ValueError("dq_form='from_ds' is not available for this shape (dS blocks of one KV head "
                                  "exceed 64 GiB)")
+        elif dq_form is None and sequence <= _FROM_DS_UP_TO_SEQ and 0 < stored <= _FROM_DS_WORKSPACE_CAP:
+            # the library then takes the stored-dS form, which is the faster one at such rows
+            workspace_bytes = stored
         else:
             workspace_bytes = int(lib.ct_attn_bwd_workspace_bytes(*shape))
     variant = _DKV_KERNELS[dkv_kernel] | _DQ_FORMS[dq_form]
@@ -334,8 +341,9 @@ def attention_backward(query, key, value, metadata, out, lse, dout, *, scale=Non
 
     ``dkv_kernel`` (``"narrow"`` / ``"wide"``) and ``dq_form`` (``"recompute"`` / ``"from_ds"``) pin a
     kernel or a form of the backward for this call (``ct_attn_bwd_args.variant``); ``None`` leaves
-    the choice to the library, which is what training code does (dQ recomputes; the dK/dV kernel goes
-    by sequence length). ``workspace_bytes`` overrides the size of the scratch buffer (default: what
+    the choice to the library, which is what training code does (the dK/dV kernel goes by sequence
+    length; dQ comes from stored dS blocks at rows of up to 4096 positions when their workspace is at
+    most 4 GiB, and from a recomputing kernel otherwise). ``workspace_bytes`` overrides the size of the scratch buffer (default: what
     the library asks for the chosen form); ``workspace`` (a :class:`BackwardWorkspace`) keeps the
     buffer, and with it the dK/dV work list, from one call to the next."""
 

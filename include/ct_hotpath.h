@@ -134,13 +134,16 @@ int32_t ct_attn_fwd(void* stream, const ct_attn_fwd_args* args);
  * NARROW = two wavefronts per SIMD with 32 keys each, WIDE = one wavefront per SIMD with 64
  * keys, the (dK, dV) sums in the accumulation registers and each step one generated
  * instruction stream (left open: WIDE from 16384 positions on, NARROW below). Bits 4-7, how dQ
- * is formed: RECOMPUTE (also what 0 means) = a query-stationary kernel evaluates S and dP a
- * second time (the reference's _local_attention_dq, src/kernels/efficient_attention.py:985-1267);
- * FROM_DS = the dK/dV kernel (NARROW) stores its bf16 dS blocks in the workspace and dQ is the
- * product of those blocks with K: 14 D instead of 18 D executed flops per pair for 4 bytes of
- * HBM traffic per pair and head; measured at par with RECOMPUTE on packed 4096-token rows and
- * slower on long rows, hence not the default; needs ct_attn_bwd_workspace_bytes_from_ds. All
- * give the same results within the operator's tolerances (not bitwise: summation orders differ). */
+ * is formed: RECOMPUTE = a query-stationary kernel evaluates S and dP a second time (the
+ * reference's _local_attention_dq, src/kernels/efficient_attention.py:985-1267); FROM_DS = the
+ * dK/dV kernel (NARROW) stores its bf16 dS blocks in the workspace and dQ is the product of those
+ * blocks with K: 14 D instead of 18 D executed flops per pair for 4 bytes of HBM traffic per
+ * pair and head; measured 1-3 % faster than RECOMPUTE on packed 4096-token rows and 15 % slower
+ * on 32768-token rows; needs ct_attn_bwd_workspace_bytes_from_ds. Left open (0): FROM_DS for
+ * rows of at most 4096 positions if the caller's workspace holds the dS blocks of all KV heads
+ * (workspace_bytes >= ct_attn_bwd_workspace_bytes_from_ds and that size is the one-pass size),
+ * else RECOMPUTE: a caller chooses by the workspace it offers. All give the same results within
+ * the operator's tolerances (not bitwise: summation orders differ). */
 #define CT_ATTN_BWD_DKV_NARROW 1
 #define CT_ATTN_BWD_DKV_WIDE 2
 #define CT_ATTN_BWD_DQ_RECOMPUTE 0x10

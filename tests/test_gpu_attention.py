@@ -132,13 +132,15 @@ def test_forward_backward_match_oracle(ct, gpu, case, bwd_variant):
     _check_against_oracle(results, q, k, v, dout, ids, ends, scale)
 
 
-@pytest.mark.parametrize("seq,expected", [(8192, "narrow"), (16384, "wide")])
+@pytest.mark.parametrize("seq,expected", [(4096, "from_ds"), (8192, "narrow"), (16384, "wide")])
 def test_default_choices_of_the_backward(ct, gpu, seq, expected):
-    """Left to itself the backward recomputes S and dP in its dQ kernel, beside the wide dK/dV
-    kernel from 16384 positions on and the narrow one below. Every kernel is deterministic, so the
-    default's results are bitwise those of the form it should have chosen (and, the summation
-    orders being different, not the others'). The stored-dS form has to be asked for, with a
-    workspace that holds at least one KV head's blocks."""
+    """Left to itself the backward takes dQ from stored dS blocks at rows of up to 4096 positions (the
+    Python operator then offers the workspace for it) and recomputes S and dP in its dQ kernel
+    above, beside the wide dK/dV kernel from 16384 positions on and the narrow one below. Every
+    kernel is deterministic, so the default's results are bitwise those of the form it should have
+    chosen (and, the summation orders being different, not the others'). With the small workspace
+    the default recomputes at any length; asked for by name, the stored-dS form needs a workspace
+    that holds at least one KV head's blocks."""
 
     rng = np.random.default_rng(seq)
     ids = _layout(rng, 1, seq, max_len=3000)
@@ -157,14 +159,22 @@ def test_default_choices_of_the_backward(ct, gpu, seq, expected):
     for name, pins in runs.items():
         print("seq", seq, name, flush=True)
         results[name] = _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5, **pins)
-    other = "wide" if expected == "narrow" else "narrow"
     for index in (2, 3, 4):
         assert torch.equal(results["default"][index], results[expected][index])
         assert ref.relative_l2(results["narrow"][index], results["wide"][index]) <= 1e-2
         assert ref.relative_l2(results["from_ds"][index], results["narrow"][index]) <= 1e-2
-    for index in (3, 4):
-        assert not torch.equal(results["default"][index], results[other][index])
     assert not torch.equal(results["from_ds"][2], results["narrow"][2])
+    if expected == "from_ds":
+        # (dK and dV come from the same kernel in both forms; dQ tells them apart)
+        assert not torch.equal(results["default"][2], results["narrow"][2])
+        print("seq", seq, "default with the small workspace", flush=True)
+        recomputed = _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5, dq_form=None, workspace_bytes=small)
+        for index in (2, 3, 4):
+            assert torch.equal(recomputed[index], results["narrow"][index])
+    else:
+        other = "wide" if expected == "narrow" else "narrow"
+        for index in (3, 4):
+            assert not torch.equal(results["default"][index], results[other][index])
     with pytest.raises(ct._lib.CtError, match="stored-dS form needs"):
         _run_gpu(ct, gpu, q, k, v, dout, ids, None, 128 ** -0.5, dq_form="from_ds", workspace_bytes=small)
     with pytest.raises(ct._lib.CtError, match="no stored-dS form"):
