@@ -47,42 +47,6 @@ CT_DEVICE void dq_arith(f32x16& s, const f32x16& dp, float lse2, float delta_q) 
   }
 }
 
-// The 32 rows of a wavefront (one head, D elements each) as the k-contiguous MFMA fragments of its
-// lanes: row l % 32, chunks 2 ks + l / 32. Loaded directly in that form an instruction touches 32
-// rows with 32 bytes each, and the address unit of a compute unit, which handles a few cache lines
-// per cycle, needs 8-12 k cycles for the three tensors of a dQ tile (measured: a tenth of the
-// kernel at short segments). Here the lanes run along the rows instead (an instruction covers 64 /
-// CPR whole rows), and the chunks go through the wavefront's LDS patch (swizzled tile layout) to
-// the lanes that need them.
-template <int D>
-struct RowBlockLoader {
-  static constexpr int CPR = D / 8;              // 16-byte chunks per row
-  static constexpr int kRowsPerLoad = 64 / CPR;  // rows one instruction covers
-  static constexpr int kLoads = 32 / kRowsPerLoad;
-  u32x4 raw[kLoads];
-  // `first_row`: row 0 of the block for this wavefront's head; row stride in elements
-  CT_DEVICE void request(const bf16* first_row, size_t row_stride) {
-    const int l = lane_id_here();
-    const bf16* mine = first_row + (size_t)(l / CPR) * row_stride + (l % CPR) * 8;
-#pragma unroll
-    for (int n = 0; n < kLoads; ++n) raw[n] = load_global16(mine + (size_t)(n * kRowsPerLoad) * row_stride);
-  }
-  // (LDS operations of one wavefront complete in order: the reads see the writes, and the next
-  // block's writes come after these reads)
-  template <class Fragment>
-  CT_DEVICE void to_fragments(lds_addr patch, Fragment* fragments) {
-    const int l = lane_id_here();
-#pragma unroll
-    for (int n = 0; n < kLoads; ++n)
-      lds_store<u32x4>(patch + tile_byte_offset<CPR>(l / CPR + n * kRowsPerLoad, l % CPR), raw[n]);
-    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks)
-      fragments[ks] = lds_load<Fragment>(patch + tile_byte_offset<CPR>(l & 31, 2 * ks + (l >> 5)));
-    __builtin_amdgcn_wave_barrier();
-  }
-};
-
 // One query tile (4 / HS row blocks x HS heads of one KV head), start to finish.
 template <int D, int HS>
 CT_DEVICE void attn_dq_item(const AttnParams& p, int b, int kvh, int slice, int qt, const lds_addr lds_base) {

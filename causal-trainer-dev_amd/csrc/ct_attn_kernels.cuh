@@ -566,7 +566,11 @@ struct VkStage {
   static constexpr int kBytes = 2 * kTileBytes;
   static constexpr int kSegRing = 2 * kBytes;  // after both stages
   static constexpr int kSegSlotBytes = kKeyTile * 4;
-  static constexpr int kTotalBytes = kSegRing + 4 * kSegSlotBytes;
+  // behind the id ring: per wavefront, the patch through which its O rows go to memory (a place of
+  // its own, so that the next query tile's first copies can be on their way meanwhile)
+  static constexpr int kStorePatches = kSegRing + 4 * kSegSlotBytes;
+  static constexpr int kStorePatchBytes = 32 * D * 2;
+  static constexpr int kTotalBytes = kStorePatches + kFwdWaves * kStorePatchBytes;
   // offset of the slot that holds the ids of key tile t
   static CT_DEVICE int seg_slot(int t) { return kSegRing + (t & 3) * kSegSlotBytes; }
 };
@@ -642,7 +646,23 @@ struct FwdAhead {
   int b, qt;
   typename Context::TileBounds bounds;
   int seg_q, end_q;
-  u32x4 q[D / 16];
+  RowBlockLoader<D> q_rows;  // whole rows per instruction; they become fragments in the tile's prologue
+  // the K rows of the tile's first two key tiles are on their way to the two stages, the V rows of
+  // its first key tile to stage 0 (the tile before issued them behind its last key tile)
+  bool first_copies_issued = false;
+  // key tiles of tile (b, qt), from the bounds
+  CT_DEVICE void key_range(const AttnParams& p, int& first, int& last) const {
+    constexpr int PB = Context::PB;
+    const int nrb = p.S / 32;
+    first = INT_MAX;
+    last = -1;
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+      if (qt * PB + i >= nrb) break;
+      first = min(first, uniform(bounds.kv_first[i]));
+      last = max(last, uniform(bounds.kv_last[i]));
+    }
+  }
   CT_DEVICE void request_bounds(const AttnParams& p, int b_, int kvh, int slice, int qt_) {
     b = b_;
     qt = qt_;
@@ -659,9 +679,8 @@ struct FwdAhead {
     // (always a load: a value formed here instead would first have to wait for the load before
     // it, which may still own the register; the context ignores it without visible ends)
     end_q = (p.end ? p.end : p.seg)[position];
-    const bf16* rows = p.q + (position * p.Hq + work.h) * D + 8 * (l >> 5);
-#pragma unroll
-    for (int ks = 0; ks < D / 16; ++ks) q[ks] = load_global16(rows + 16 * ks);
+    const size_t first = (size_t)b * p.S + min(work.rb, p.S / 32 - 1) * 32;
+    q_rows.request(p.q + (first * p.Hq + work.h) * D, (size_t)p.Hq * D);
   }
 };
 
@@ -707,8 +726,9 @@ CT_DEVICE void attn_fwd_item_phased(const AttnParams& p, FwdAhead<D, HS>& ahead,
   ahead.request_bounds(p, next_b, kvh, slice, next_qt);
   // (the Q rows are touched only now: the first copies above needed nothing but the bounds)
   bf16x8 qf[D / 16];
+  ahead.q_rows.to_fragments(lds0 + (VkStage<D>::kStorePatches + w * VkStage<D>::kStorePatchBytes), qf);
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) qf[ks] = scale_bf16x8(as_bf16x8(ahead.q[ks]), p.scale);
+  for (int ks = 0; ks < D / 16; ++ks) qf[ks] = scale_bf16x8(qf[ks], p.scale);
   dma_wait_all();
   __syncthreads();
   if (visit) scores_t<D>(kStage + VkStage<D>::kK, ro, qf, s);
@@ -900,7 +920,7 @@ CT_DEVICE void fwd_store_rows(float row_scale, lds_addr patch, bf16* gbase, size
 // One query tile, interleaved form (D = 128). Arguments as attn_fwd_item_phased.
 template <int D, int HS>
 CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int next_b,
-                             int next_qt, int kvh, int slice, const lds_addr lds0,
+                             int next_qt, bool more, int kvh, int slice, const lds_addr lds0,
                              const RowFragOffsets<D / 8>& ro,
                              const TrFragOffsets<D / 8, KSlots::kAccum>& to) {
   static_assert(D == 128, "the interleaved statements are written for D = 128");
@@ -928,9 +948,11 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
     // K rows of the first two tiles (they belong to stages first - 2 and first - 1), and the V rows
     // of the first: its place in stage `first` is free already, only the K half of that stage has
     // to wait until K(first) has been read
-    fetch.issue_k(t, lds0, lds0);
-    if (t + 1 <= last) fetch.issue_k(t + 1, lds0 + kStage, lds0);
-    fetch.issue_v(t, lds0);
+    if (!ahead.first_copies_issued) {
+      fetch.issue_k(t, lds0, lds0);
+      if (t + 1 <= last) fetch.issue_k(t + 1, lds0 + kStage, lds0);
+      fetch.issue_v(t, lds0);
+    }
     kb = key_tile_bounds(ctx.meta_b, t);
     if (t + 1 <= last) nb = key_tile_bounds(ctx.meta_b, t + 1);
     visit = ctx.wave_visits(kb, t);
@@ -964,8 +986,9 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
   ahead.request_bounds(p, next_b, kvh, slice, next_qt);
   // (the Q rows are touched only now: the first copies above needed nothing but the bounds)
   bf16x8 qf[D / 16];
+  ahead.q_rows.to_fragments(lds0 + (VkStage<D>::kStorePatches + w * VkStage<D>::kStorePatchBytes), qf);
 #pragma unroll
-  for (int ks = 0; ks < D / 16; ++ks) qf[ks] = scale_bf16x8(as_bf16x8(ahead.q[ks]), p.scale);
+  for (int ks = 0; ks < D / 16; ++ks) qf[ks] = scale_bf16x8(qf[ks], p.scale);
   dma_wait_all();
   __syncthreads();
   if (visit) fwd_qk_b<kK>(ro, qf);  // (statement "b" writes buffer a: the first tile counts even)
@@ -1170,8 +1193,25 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
     else step(std::integral_constant<int, 1>{});
   }
   // What is left is the PV product of the last tile, and no later wait of this query tile is a
-  // wait for memory: the next tile's rows are requested here and land under that product, the
-  // stores of O and the next tile's first copies.
+  // wait for memory. Every wavefront is past its last read of K rows, so the next query tile's
+  // first two K tiles can take their places in the stages now, and its rows are requested behind
+  // them: all of that lands under the last product and the stores of O. (`ahead` names the next
+  // tile since the prologue.)
+  int next_first = 0, next_last = -1;
+  VkFetcher<D> next_fetch = fetch;
+  ahead.first_copies_issued = false;
+  if (more) {
+    ahead.key_range(p, next_first, next_last);
+    if (next_first <= next_last) {
+      const size_t row0 = ((size_t)ahead.b * p.S * p.Hkv + kvh) * D;
+      next_fetch.kbase = reinterpret_cast<const char*>(p.k + row0);
+      next_fetch.vbase = reinterpret_cast<const char*>(p.v + row0);
+      next_fetch.segb = p.seg + (size_t)ahead.b * p.S;
+      next_fetch.issue_k(next_first, lds0, lds0);
+      if (next_first + 1 <= next_last) next_fetch.issue_k(next_first + 1, lds0 + kStage, lds0);
+      ahead.first_copies_issued = true;
+    }
+  }
   ahead.request_rows(p, kvh, slice);
   if (any_tile && visit_prev) {
     // stage `last` is in LDS buffer (last - first) & 1, P^T(last) in the score buffer of that
@@ -1179,10 +1219,12 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
     if (((last - ctx.first) & 1) == 0) fwd_pv_b<kV>(to);
     else fwd_pv_a<kStage + kV>(to);
   }
-  // Every copy of this tile has been waited for, so only LDS traffic has to settle before the
-  // stages become store patches (a wait for memory here would wait for the next tile's loads).
+  // Every wavefront has read its V rows once it is past this barrier (LDS traffic only: a wait for
+  // memory here would wait for the next tile's loads): the V rows of the next tile's first key
+  // tile may follow.
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_s_barrier();
+  if (ahead.first_copies_issued) next_fetch.issue_v(next_first, lds0);
 
   const float l_tot = pair_sum(l_run);
   const bool has = l_tot > 0.f;
@@ -1191,14 +1233,12 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
     const int le = lane_id_here();
     const size_t stat = ((size_t)ctx.work.b * p.S + ctx.work.rb * 32 + (le & 31)) * p.Hq + ctx.work.h;
     if (le < 32) p.lse[stat] = has ? (__logf(l_tot) + m_run * kLn2) : 0.f;
-    const lds_addr patch = lds0 + w * 32 * D * 2;
+    // (the patch is this wavefront's alone: its next use, one query tile on, follows these reads
+    // in the wavefront's own order, so no barrier closes the tile)
+    const lds_addr patch = lds0 + (VkStage<D>::kStorePatches + w * VkStage<D>::kStorePatchBytes);
     bf16* obase = p.out + (((size_t)ctx.work.b * p.S + ctx.work.rb * 32) * p.Hq + ctx.work.h) * D;
     fwd_store_rows(inv, patch, obase, q_row_stride);
   }
-  // The store patches overlap the stages of the next item: its copies may start once every
-  // wavefront has read its patch back (LDS reads only; the global stores stay in flight).
-  __builtin_amdgcn_s_waitcnt(0xC07F);
-  __builtin_amdgcn_s_barrier();
 }
 
 // Workgroup (group, bin): walks the query tiles of one work bin for one
@@ -1232,7 +1272,7 @@ attn_fwd_kernel(AttnParams p) {
   for (; it < it_end; ++it) {
     const int next_item = uniform(region[kBins + 1 + min(it + 1, it_end - 1)]);
     if constexpr (D == 128)
-      attn_fwd_item<D, HS>(p, ahead, next_item / tpr, next_item % tpr, kvh, slice, lds0, ro, to);
+      attn_fwd_item<D, HS>(p, ahead, next_item / tpr, next_item % tpr, it + 1 < it_end, kvh, slice, lds0, ro, to);
     else
       attn_fwd_item_phased<D, HS>(p, ahead, next_item / tpr, next_item % tpr, kvh, slice, lds0, ro, to);
   }

@@ -357,6 +357,42 @@ CT_DEVICE bf16x8 pack_acc8(const f32x16& c, int t) {
 CT_DEVICE u32x4 load_global16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
 CT_DEVICE void store_global16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
 
+// The 32 rows of a wavefront (one head, D elements each) as the k-contiguous MFMA fragments of its
+// lanes: row l % 32, chunks 2 ks + l / 32. Loaded directly in that form an instruction touches 32
+// rows with 32 bytes each, and the address unit of a compute unit, which handles a few cache lines
+// per cycle, needs 8-12 k cycles for the three tensors of a dQ tile (measured: a tenth of that
+// kernel at short segments). Here the lanes run along the rows instead (an instruction covers 64 /
+// CPR whole rows), and the chunks go through the wavefront's LDS patch (swizzled tile layout) to
+// the lanes that need them.
+template <int D>
+struct RowBlockLoader {
+  static constexpr int CPR = D / 8;              // 16-byte chunks per row
+  static constexpr int kRowsPerLoad = 64 / CPR;  // rows one instruction covers
+  static constexpr int kLoads = 32 / kRowsPerLoad;
+  u32x4 raw[kLoads];
+  // `first_row`: row 0 of the block for this wavefront's head; row stride in elements
+  CT_DEVICE void request(const bf16* first_row, size_t row_stride) {
+    const int l = lane_id_here();
+    const bf16* mine = first_row + (size_t)(l / CPR) * row_stride + (l % CPR) * 8;
+#pragma unroll
+    for (int n = 0; n < kLoads; ++n) raw[n] = load_global16(mine + (size_t)(n * kRowsPerLoad) * row_stride);
+  }
+  // (LDS operations of one wavefront complete in order: the reads see the writes, and the next
+  // block's writes come after these reads)
+  template <class Fragment>
+  CT_DEVICE void to_fragments(lds_addr patch, Fragment* fragments) {
+    const int l = lane_id_here();
+#pragma unroll
+    for (int n = 0; n < kLoads; ++n)
+      lds_store<u32x4>(patch + tile_byte_offset<CPR>(l / CPR + n * kRowsPerLoad, l % CPR), raw[n]);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int ks = 0; ks < D / 16; ++ks)
+      fragments[ks] = lds_load<Fragment>(patch + tile_byte_offset<CPR>(l & 31, 2 * ks + (l >> 5)));
+    __builtin_amdgcn_wave_barrier();
+  }
+};
+
 // 4-byte store to uniform_base + lane_offset + IMM bytes (scalar base, 32-bit lane offset): no
 // per-store vector address arithmetic. The scalar base may have just been written by a vector
 // instruction (v_readfirstlane): a memory instruction that reads such a register needs 5 wait
