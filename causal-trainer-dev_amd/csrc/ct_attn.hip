@@ -2,9 +2,9 @@
 #include <atomic>
 #include <algorithm>
 
-#include "ct_attn_bwd_kernels.cuh"
-#include "ct_attn_dkv_wide.cuh"
-#include "ct_attn_kernels.cuh"
+#include "ct_attn_bwd_kernels.hip.h"
+#include "ct_attn_dkv_wide.hip.h"
+#include "ct_attn_kernels.hip.h"
 #include "ct_error.h"
 
 #include <string.h>

@@ -13,7 +13,7 @@
 // Every output tile has a single owner: no atomics, fixed summation order.
 #pragma once
 
-#include "ct_attn_kernels.cuh"
+#include "ct_attn_kernels.hip.h"
 
 namespace ct {
 

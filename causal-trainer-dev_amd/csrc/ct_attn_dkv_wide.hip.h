@@ -12,7 +12,7 @@
 // (wavefront w here covers the 32-key blocks 2w and 2w + 1 of the tile).
 #pragma once
 
-#include "ct_attn_bwd_kernels.cuh"
+#include "ct_attn_bwd_kernels.hip.h"
 
 namespace ct {
 

@@ -25,8 +25,8 @@
 #include <type_traits>
 
 #include "ct_attn_asm.inc"
-#include "ct_attn_meta.cuh"
-#include "ct_common.cuh"
+#include "ct_attn_meta.hip.h"
+#include "ct_common.hip.h"
 
 namespace ct {
 

@@ -33,7 +33,7 @@
 
 #include <limits.h>
 
-#include "ct_common.cuh"
+#include "ct_common.hip.h"
 
 namespace ct {
 

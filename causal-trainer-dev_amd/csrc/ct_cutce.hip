@@ -24,7 +24,7 @@
 #include <mutex>
 
 #include "ct_error.h"
-#include "ct_gemm.cuh"
+#include "ct_gemm.hip.h"
 
 namespace ct {
 

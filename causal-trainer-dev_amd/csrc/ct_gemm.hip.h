@@ -28,7 +28,7 @@
 
 #include <type_traits>
 
-#include "ct_common.cuh"
+#include "ct_common.hip.h"
 #include "ct_gemm_asm.inc"
 
 namespace ct {
