@@ -147,27 +147,6 @@ CT_DEVICE void scores_t(int tile_off, const RowFrags& ro, const bf16x8* qf, f32x
   }
 }
 
-// allowed(query of this lane, key held by register r of block kb)?  Writes a
-// 32-bit mask per block: bit r set = allowed.
-CT_DEVICE void tile_mask(lds_addr segk, int tile, int seg_q, int end_q, bool row_valid,
-                         unsigned* allow) {
-  const int half = lane_id() >> 5;
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb) {
-    unsigned bits = 0;
-#pragma unroll
-    for (int qd = 0; qd < 4; ++qd) {
-      const int k0 = kb * 32 + 8 * qd + 4 * half;
-      const i32x4 sk = lds_load<i32x4>(segk + k0 * 4);
-      const int key = tile * kKeyTile + k0;
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        bits |= (unsigned)(sk[e] == seg_q && key + e <= end_q) << (4 * qd + e);
-    }
-    allow[kb] = row_valid ? bits : 0u;
-  }
-}
-
 // Sets the scores of disallowed (query, key) pairs of a transposed score tile to -inf.
 // The pair rule is seg_k == seg_q != 0 and key <= end_q (src/modeling/attention.py:67-97);
 // each half is only evaluated where the tile's summaries do not already prove it:
@@ -452,6 +431,11 @@ struct FwdCopies {
   CT_DEVICE void fwd_qk_##NAME(const RowFragOffsets<16>& ro, const bf16x8* qf) {                             \
     asm volatile(CT_FWD_QK_##UPPER : : CT_FWD_ROW_PTRS(ro, qf), [koff] "i"(K_OFF) : "memory", CT_FWD_PRIVATE); \
   }                                                                                                           \
+  /* the same with the output accumulator cleared behind the MFMAs (a query tile's first scores) */          \
+  template <int K_OFF>                                                                                        \
+  CT_DEVICE void fwd_qk_zero_##NAME(const RowFragOffsets<16>& ro, const bf16x8* qf) {                        \
+    asm volatile(CT_FWD_QK_ZERO_##UPPER : : CT_FWD_ROW_PTRS(ro, qf), [koff] "i"(K_OFF) : "memory", CT_FWD_PRIVATE); \
+  }                                                                                                           \
   /* -inf where the key's offset in the tile exceeds rel (per lane) */                                        \
   CT_DEVICE void fwd_mask_causal_##NAME(int rel) {                                                            \
     asm volatile(CT_FWD_MASK_CAUSAL_##UPPER                                                                   \
@@ -459,12 +443,12 @@ struct FwdCopies {
                  : [rel] "v"(rel), [ninf] "v"(kNegInf)                                                        \
                  : "memory", "vcc", CT_FWD_PRIVATE);                                                          \
   }                                                                                                           \
-  /* -inf where bit r of bits0 / bits1 (register r of key block 0 / 1) is clear */                            \
-  CT_DEVICE void fwd_mask_bits_##NAME(unsigned bits0, unsigned bits1) {                                       \
-    int tmp;                                                                                                  \
-    asm volatile(CT_FWD_MASK_BITS_##UPPER                                                                     \
-                 : [tmp] "=&v"(tmp)                                                                           \
-                 : [bits0] "v"(bits0), [bits1] "v"(bits1), [ninf] "v"(kNegInf)                                \
+  /* -inf where the key's id differs from seg (per lane); ids: the lane's address of the id of key */        \
+  /* 4 * (lane / 32) of the tile in the id ring                                                      */        \
+  CT_DEVICE void fwd_mask_ids_##NAME(lds_addr ids, int seg) {                                                 \
+    asm volatile(CT_FWD_MASK_IDS_##UPPER                                                                      \
+                 :                                                                                            \
+                 : [idp] "v"(ids), [segq] "v"(seg), [ninf] "v"(kNegInf)                                       \
                  : "memory", "vcc", CT_FWD_PRIVATE);                                                          \
   }
 CT_FWD_STATEMENTS(a, A)
@@ -933,7 +917,6 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
   const size_t q_row_stride = (size_t)p.Hq * D;
   const size_t kv_row_stride = (size_t)p.Hkv * D;
 
-  fwd_acc_zero();
   float m_run = kNegInf;  // softmax reference (a recent running max), log2 domain
   float l_run = 0.f;      // this lane's share of the running sum (f32: the LSE is held to 1e-3)
 
@@ -991,7 +974,10 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
   for (int ks = 0; ks < D / 16; ++ks) qf[ks] = scale_bf16x8(qf[ks], p.scale);
   dma_wait_all();
   __syncthreads();
-  if (visit) fwd_qk_b<kK>(ro, qf);  // (statement "b" writes buffer a: the first tile counts even)
+  // (statement "b" writes buffer a: the first tile counts even; the output accumulator is cleared
+  // behind its MFMAs, or on its own where this wavefront does not see the first tile)
+  if (visit) fwd_qk_zero_b<kK>(ro, qf);
+  else fwd_acc_zero();
   // every wavefront has read K(first): the first step's copies may replace it
   __builtin_amdgcn_s_barrier();
 
@@ -1036,10 +1022,17 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
       if (need_seg || need_causal) {
         const int seg_cmp = ctx.row_valid() ? ctx.seg_q : -1;
         if (k_uniform == 0) {
-          unsigned allow[2];
-          tile_mask(lds0 + VkStage<D>::seg_slot(t), t, seg_cmp, ctx.end_q, true, allow);
-          if constexpr (PARITY == 0) fwd_mask_bits_a(allow[0], allow[1]);
-          else fwd_mask_bits_b(allow[0], allow[1]);
+          // the ids of the tile's keys against the row's (-1 for a padding row matches none), then,
+          // where the tile reaches past the smallest visible end, the keys' offsets against the row's end
+          const int half = lane_id_here() >> 5;
+          const lds_addr ids = lds0 + (VkStage<D>::seg_slot(t) + 16 * half);
+          if constexpr (PARITY == 0) fwd_mask_ids_a(ids, seg_cmp);
+          else fwd_mask_ids_b(ids, seg_cmp);
+          if (need_causal) {
+            const int rel = ctx.end_q - t * kKeyTile - 4 * half;
+            if constexpr (PARITY == 0) fwd_mask_causal_a(rel);
+            else fwd_mask_causal_b(rel);
+          }
         } else {
           // (no key of this tile is visible to a query of another id)
           const int rel = seg_cmp != k_uniform ? -1 : ctx.end_q - t * kKeyTile - 4 * (lane_id_here() >> 5);

@@ -258,12 +258,22 @@ def fwd_statements(cur):
     for i in range(32):
         causal += ["v_cmp_le_i32_e32 vcc, %d, %%[rel]" % key_offset(i),
                    "v_cndmask_b32_e32 v%d, %%[ninf], v%d, vcc" % (s0 + i, s0 + i)]
-    bits = []
-    for i in range(32):
-        # bit i % 16 of the block's word into the sign bit: negative = allowed
-        bits += ["v_lshlrev_b32_e32 %%[tmp], %d, %%[bits%d]" % (31 - i % 16, i // 16),
-                 "v_cmp_gt_i32_e32 vcc, 0, %[tmp]",
-                 "v_cndmask_b32_e32 v%d, %%[ninf], v%d, vcc" % (s0 + i, s0 + i)]
+    # ids: the tile's 64 key ids sit in LDS in key order; %[idp] is this lane's address of key
+    # 4 * (lane / 32), so the quad of registers 4 q .. 4 q + 3 of block kb is the 16 bytes at
+    # offset 4 * (32 kb + 8 q). Quads go through the fragment ring (four in flight).
+    ids = ["s_waitcnt lgkmcnt(0)"]
+    quad_regs = lambda q: FWD_RING0 + 4 * (q % 4)
+    quad_read = lambda q: "ds_read_b128 v[%d:%d], %%[idp] offset:%d" % (
+        quad_regs(q), quad_regs(q) + 3, 4 * (32 * (q // 4) + 8 * (q % 4)))
+    ids += [quad_read(q) for q in range(4)]
+    for q in range(8):
+        ids.append("s_waitcnt lgkmcnt(%d)" % min(3, 7 - q))
+        for e in range(4):
+            i = 4 * q + e
+            ids += ["v_cmp_eq_u32_e32 vcc, %%[segq], v%d" % (quad_regs(q) + e),
+                    "v_cndmask_b32_e32 v%d, %%[ninf], v%d, vcc" % (s0 + i, s0 + i)]
+        if q + 4 < 8:
+            ids.append(quad_read(q + 4))
     return {
         # the three interleaved statements
         "MAX": head_pv01 + weave(fwd_with_copies(pv01, 2), fwd_max_ops(cur)),
@@ -275,10 +285,13 @@ def fwd_statements(cur):
         "PV": flatten(head_pv, pv) + TAIL,
         "PV_LATE": flatten(head_pv23, pv23) + TAIL,
         "QK": flatten(head_qk, qk) + TAIL,
-        # masks: scores of pairs that are not allowed become -inf. CAUSAL: key offset in the tile
-        # <= %[rel] (per lane); BITS: bit r of %[bits0] / %[bits1] set = register r of the block allowed
+        # the first scores of a query tile, with the clearing of the output accumulator behind the MFMAs
+        "QK_ZERO": head_qk + weave(qk, fwd_accumulator_statements()["ZERO"]) + TAIL,
+        # masks: scores of pairs that are not allowed become -inf. CAUSAL: allowed = key offset in the
+        # tile <= %[rel] (per lane)
         "MASK_CAUSAL": causal,
-        "MASK_BITS": bits,
+        # IDS: the key's id (read here from the id ring in LDS) differs from %[segq] (per lane)
+        "MASK_IDS": ids,
     }
 
 

@@ -44,7 +44,7 @@ def _split(line):
 class Model:
     def __init__(self):
         self.pending = []          # (destination registers) of LDS reads in flight, in issue order
-        self.unread = {}           # register -> index of the LDS read whose data no MFMA has used yet
+        self.unread = {}           # register -> index of the LDS read whose data nothing has used yet
         self.mfmas = 0
         self.last_mfma_write = {}  # register -> number of the MFMA that last wrote it
         self.problems = []
@@ -59,7 +59,7 @@ class Model:
                 dest = _registers(ops[0])
                 stale = [r for r in dest if r in self.unread]
                 if stale:
-                    self.problems.append(f"line {number} '{line}' overwrites a fragment no MFMA has read")
+                    self.problems.append(f"line {number} '{line}' overwrites LDS data nothing has read")
                 if dest & self.busy():
                     self.problems.append(f"line {number} '{line}' writes registers of a read still in flight")
                 self.pending.append(dest)
@@ -86,6 +86,7 @@ class Model:
                 if sources & self.busy():
                     self.problems.append(f"line {number} '{line}' reads registers of an LDS read still in flight")
                 for r in sources:
+                    self.unread.pop(r, None)       # (ids read from LDS are consumed by compares)
                     written = self.last_mfma_write.get(r)
                     # an MFMA result is read by the vector ALU only after two more MFMAs have been
                     # issued: the producer has then left the matrix pipe
@@ -130,7 +131,7 @@ def test_model_catches_the_mistakes_it_is_meant_for(gen):
     lost = [line for line in good]
     mfma = next(i for i, line in enumerate(lost) if line.startswith("v_mfma"))
     del lost[mfma]
-    assert any("no MFMA has read" in p for p in Model().run(lost).problems)
+    assert any("nothing has read" in p for p in Model().run(lost).problems)
     # arithmetic directly behind the MFMA that produces its input
     wide = gen.dkvw_step_sequence()
     s0 = gen.W_S[0]
@@ -240,7 +241,7 @@ def test_forward_interleaved_statements(gen, cur):
     for index, line in enumerate(mfmas["QK"]):
         block = index % 2
         assert _split(line)[1][0] == "v[%d:%d]" % (other + 16 * block, other + 16 * block + 15), line
-    for name in ("MAX", "EXP_A", "MAX_ONLY", "EXP_ONLY", "MASK_CAUSAL", "MASK_BITS"):
+    for name in ("MAX", "EXP_A", "MAX_ONLY", "EXP_ONLY", "MASK_CAUSAL", "MASK_IDS"):
         for line in statements[name]:
             if line.startswith(("v_", "ds_read")):
                 destination = _registers(_split(line)[1][0])
@@ -267,7 +268,8 @@ def test_forward_interleaved_statements(gen, cur):
 
 def test_forward_masks(gen):
     """The mask statements: one compare and one select per score, the key offset of a score register
-    as the accumulator layout has it (block 32 kb, then 8 (r / 4) + r % 4)."""
+    as the accumulator layout has it (block 32 kb, then 8 (r / 4) + r % 4, plus 4 for the lanes of
+    the upper half)."""
 
     for cur in ("a", "b"):
         s0 = gen.FWD_S[cur]
@@ -277,11 +279,40 @@ def test_forward_masks(gen):
             offset = 32 * (i // 16) + 8 * ((i % 16) // 4) + (i % 16) % 4
             assert causal[2 * i] == "v_cmp_le_i32_e32 vcc, %d, %%[rel]" % offset
             assert causal[2 * i + 1] == "v_cndmask_b32_e32 v%d, %%[ninf], v%d, vcc" % (s0 + i, s0 + i)
-        bits = gen.fwd_statements(cur)["MASK_BITS"]
-        assert len(bits) == 96
-        for i in range(32):
-            assert bits[3 * i] == "v_lshlrev_b32_e32 %%[tmp], %d, %%[bits%d]" % (31 - i % 16, i // 16)
-            assert bits[3 * i + 2] == "v_cndmask_b32_e32 v%d, %%[ninf], v%d, vcc" % (s0 + i, s0 + i)
+        # ids: run the statement on a model of the id ring (key k's id at byte 4 k; the lane's pointer
+        # is the address of key 4 * half): every score must be compared with the id of its own key,
+        # and no register may be read before the wait that covers its load
+        for half in (0, 1):
+            registers, landed, in_flight = {}, set(), []
+            compared = {}
+            pending_compare = None
+            for line in gen.fwd_statements(cur)["MASK_IDS"]:
+                name, operands = _split(line)
+                if name == "s_waitcnt":
+                    allowed = int(operands[0][len("lgkmcnt("):-1])
+                    while len(in_flight) > allowed:
+                        landed |= in_flight.pop(0)
+                elif name == "ds_read_b128":
+                    offset = int(operands[2][len("offset:"):]) if len(operands) > 2 else int(line.split("offset:")[1])
+                    quad = sorted(_registers(operands[0]))
+                    assert len(quad) == 4 and offset % 16 == 0
+                    for e, register in enumerate(quad):
+                        registers[register] = 4 * half + offset // 4 + e     # the key whose id it holds
+                    landed -= set(quad)
+                    in_flight.append(set(quad))
+                elif name == "v_cmp_eq_u32_e32":
+                    assert operands[:2] == ["vcc", "%[segq]"]
+                    (register,) = _registers(operands[2])
+                    assert register in landed, line
+                    pending_compare = registers[register]
+                elif name == "v_cndmask_b32_e32":
+                    (score,) = _registers(operands[0])
+                    assert operands[1] == "%[ninf]" and _registers(operands[2]) == {score} and operands[3] == "vcc"
+                    compared[score - s0] = pending_compare
+                    pending_compare = None
+                else:
+                    raise AssertionError(line)
+            assert compared == {i: 32 * (i // 16) + 8 * ((i % 16) // 4) + (i % 16) % 4 + 4 * half for i in range(32)}
 
 
 def test_committed_include_is_what_the_generator_prints(gen):
