@@ -924,6 +924,7 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
   int t = ctx.first;
   const int last = ctx.last;
   const bool any_tile = t <= last;
+  const bool k_rows_on_their_way = ahead.first_copies_issued;
   KeyTileBounds kb = {0, 0, 0}, nb = {0, 0, 0};  // bounds of tiles t and t + 1
   bool visit = false;       // does this wavefront see tile t (its scores are in the buffer of t)
   bool visit_prev = false;  // ... tile t - 1 (P^T in the other buffer, PV product still to do)
@@ -931,7 +932,8 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
     // K rows of the first two tiles (they belong to stages first - 2 and first - 1), and the V rows
     // of the first: its place in stage `first` is free already, only the K half of that stage has
     // to wait until K(first) has been read
-    if (!ahead.first_copies_issued) {
+    // (a query tile that follows another in this workgroup had its K rows copied by that one)
+    if (!k_rows_on_their_way) {
       fetch.issue_k(t, lds0, lds0);
       if (t + 1 <= last) fetch.issue_k(t + 1, lds0 + kStage, lds0);
       fetch.issue_v(t, lds0);
@@ -974,6 +976,9 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
   for (int ks = 0; ks < D / 16; ++ks) qf[ks] = scale_bf16x8(qf[ks], p.scale);
   dma_wait_all();
   __syncthreads();
+  // Every wavefront is past the last PV product of the query tile before: the V rows of this one's
+  // first key tile may take their place (first read one step from now, behind that step's wait).
+  if (any_tile && k_rows_on_their_way) fetch.issue_v(t, lds0);
   // (statement "b" writes buffer a: the first tile counts even; the output accumulator is cleared
   // behind its MFMAs, or on its own where this wavefront does not see the first tile)
   if (visit) fwd_qk_zero_b<kK>(ro, qf);
@@ -1189,16 +1194,15 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
   // wait for memory. Every wavefront is past its last read of K rows, so the next query tile's
   // first two K tiles can take their places in the stages now, and its rows are requested behind
   // them: all of that lands under the last product and the stores of O. (`ahead` names the next
-  // tile since the prologue.)
-  int next_first = 0, next_last = -1;
-  VkFetcher<D> next_fetch = fetch;
+  // tile since the prologue. Its V rows wait for the barrier in its own prologue: until then a
+  // wavefront may still read this tile's.)
   ahead.first_copies_issued = false;
   if (more) {
+    int next_first, next_last;
     ahead.key_range(p, next_first, next_last);
     if (next_first <= next_last) {
-      const size_t row0 = ((size_t)ahead.b * p.S * p.Hkv + kvh) * D;
-      next_fetch.kbase = reinterpret_cast<const char*>(p.k + row0);
-      next_fetch.vbase = reinterpret_cast<const char*>(p.v + row0);
+      VkFetcher<D> next_fetch = fetch;
+      next_fetch.kbase = reinterpret_cast<const char*>(p.k + ((size_t)ahead.b * p.S * p.Hkv + kvh) * D);
       next_fetch.segb = p.seg + (size_t)ahead.b * p.S;
       next_fetch.issue_k(next_first, lds0, lds0);
       if (next_first + 1 <= next_last) next_fetch.issue_k(next_first + 1, lds0 + kStage, lds0);
@@ -1212,12 +1216,6 @@ CT_DEVICE void attn_fwd_item(const AttnParams& p, FwdAhead<D, HS>& ahead, int ne
     if (((last - ctx.first) & 1) == 0) fwd_pv_b<kV>(to);
     else fwd_pv_a<kStage + kV>(to);
   }
-  // Every wavefront has read its V rows once it is past this barrier (LDS traffic only: a wait for
-  // memory here would wait for the next tile's loads): the V rows of the next tile's first key
-  // tile may follow.
-  __builtin_amdgcn_s_waitcnt(0xC07F);
-  __builtin_amdgcn_s_barrier();
-  if (ahead.first_copies_issued) next_fetch.issue_v(next_first, lds0);
 
   const float l_tot = pair_sum(l_run);
   const bool has = l_tot > 0.f;
