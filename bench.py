@@ -206,7 +206,7 @@ def attention_step_for(ct, config, inputs, **backward_pins):
     return step, metadata, pairs
 
 
-ROOFLINE_ATTENTION_KERNELS = ("attn_fwd_kernel", "attn_dq_kernel", "attn_dkv_kernel")
+ROOFLINE_ATTENTION_KERNELS = ("attn_fwd_kernel", "attn_dq_kernel", "attn_dkv_kernel", "attn_dkv_wide_kernel")
 ROOFLINE_CUTCE_KERNELS = ("cutce_stats_kernel", "cutce_dhidden_kernel", "cutce_dhead_kernel", "cutce_dlogits_kernel",
                           "cutce_grads_kernel")
 
@@ -220,7 +220,8 @@ def kernel_table(config, pairs, kernels):
     else:
         # dQ recomputes S and dP: algorithmic work split by which kernel owns the result:
         # dQ kernel 4*D*Hq*pairs (dP, dQ), dK/dV kernel 6*D*Hq*pairs (S, dV, dK)
-        per_kernel_flops = {"attn_fwd_kernel": 4 * unit, "attn_dq_kernel": 4 * unit, "attn_dkv_kernel": 6 * unit}
+        per_kernel_flops = {"attn_fwd_kernel": 4 * unit, "attn_dq_kernel": 4 * unit, "attn_dkv_kernel": 6 * unit,
+                            "attn_dkv_wide_kernel": 6 * unit}
     per_kernel_bytes = {
         # O and dO read once, lse read, two statistics written
         "attn_bwd_stats_kernel": config.batch * config.seq * config.q_heads * (4 * config.head_dim + 12),

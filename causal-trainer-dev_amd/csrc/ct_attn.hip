@@ -411,14 +411,15 @@ template <int D>
 static int launch_dkv(hipStream_t stream, const AttnParams& p, bool wide) {
   const size_t smem = QdoStage<D>::kTotalBytes;
   const int grid = p.dkv_max_entries * p.kvh_count;  // entries beyond the list's length exit at once
-  LaunchScope scope3("attn_dkv_kernel", stream);
   if constexpr (D == 128) {
     if (wide) {
       CT_ENSURE_LDS("ct_attn_bwd", &attn_dkv_wide_kernel, DkvWideLds::kTotalBytes);
+      LaunchScope scope("attn_dkv_wide_kernel", stream);
       hipLaunchKernelGGL(attn_dkv_wide_kernel, dim3(grid), dim3(128), DkvWideLds::kTotalBytes, stream, p);
-      return scope3.done();
+      return scope.done();
     }
   }
+  LaunchScope scope3("attn_dkv_kernel", stream);
   if (p.ds) {
     CT_ENSURE_LDS("ct_attn_bwd", (&attn_dkv_kernel<D, true>), smem);
     hipLaunchKernelGGL((attn_dkv_kernel<D, true>), dim3(grid), dim3(256), smem, stream, p);

@@ -288,8 +288,8 @@ using DkvTrFrags = std::conditional_t<(D / 8 >= 16), TrFragCompact<D / 8, KSlots
 
 // X (32 rows of an LDS tile) times register fragments: C[row, key] = sum_d X[row, d] F[key, d].
 template <int D>
-CT_DEVICE f32x16 rows_times_frags(int tile_off, const DkvRowFrags<D>& ro, const bf16x8* frags) {
-  f32x16 c = zero16();
+CT_DEVICE f32x16 rows_times_frags(int tile_off, const DkvRowFrags<D>& ro, const bf16x8* frags,
+                                  f32x16 c = zero16()) {
 #pragma unroll
   for (int ks = 0; ks < D / 16; ++ks) c = mfma32(ro.load(tile_off, 0, ks), frags[ks], c);
   return c;
@@ -304,7 +304,7 @@ template <int STAGE_OFF>
 CT_DEVICE void dkv_sdp_sequence_128(const RowFragOffsets<16>& ro, const bf16x8* kf, unsigned v_off,
                                     f32x16& s, f32x16& dp) {
   asm volatile(CT_DKV_SDP_SEQUENCE
-               : "=&v"(s), "=&v"(dp)
+               : "+v"(s), "+v"(dp)
                : "v"(ro.ptr[0]), "v"(ro.ptr[1]), "v"(ro.ptr[2]), "v"(ro.ptr[3]), "v"(ro.ptr[4]),
                  "v"(ro.ptr[5]), "v"(ro.ptr[6]), "v"(ro.ptr[7]), "v"(kf[0]), "v"(kf[1]), "v"(kf[2]),
                  "v"(kf[3]), "v"(kf[4]), "v"(kf[5]), "v"(kf[6]), "v"(kf[7]), "s"(v_off), "i"(STAGE_OFF)
@@ -690,25 +690,38 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
     if (more) qb_bounds = query_block_bounds(meta_b, qb_next);
     const bool visit = blocks_interact(q_min, q_max, q_end_max, my_min, my_max, my_rb * 32);
     if (visit) {
+      // The row offsets below depend on the lane only; hoisted out of the loop they become
+      // spilled registers whose reloads wait for every copy in flight. Recompute them here.
+      int half_here = half;
+      asm volatile("" : "+v"(half_here));
+      // Both products start from the per-row terms of their 16 query rows instead of zero (the
+      // statistics pass left -lse / scale and -delta): the sums S - lse / scale and dP - delta
+      // come out of the matrix pipe, and no vector instruction adds them.
       f32x16 s, dp;
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int r0 = 8 * qd + 4 * half_here;
+        const f32x4 lse4 = lds_load<f32x4>(stage + QdoStage<D>::kLse + r0 * 4);
+        const f32x4 del4 = lds_load<f32x4>(stage + QdoStage<D>::kDelta + r0 * 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s[4 * qd + e] = lse4[e];
+          dp[4 * qd + e] = del4[e];
+        }
+      }
       if constexpr (D == 128) {
         // (fragment pointers built here from the lane id: held across the loop they would
         // push the kernel over its register budget)
         const RowFragOffsets<16> rp = RowFragOffsets<16>::expand(RowFragCompact<16>(lds0, lane_id_here()));
         dkv_sdp_sequence_128<CUR * kStage>(rp, kf, (unsigned)vpatch_off, s, dp);
       } else {
-        s = rows_times_frags<D>(CUR * kStage + QdoStage<D>::kQ, ro, kf);
-        dp = zero16();
+        s = rows_times_frags<D>(CUR * kStage + QdoStage<D>::kQ, ro, kf, s);
 #pragma unroll
         for (int ks = 0; ks < D / 16; ++ks)
           dp = mfma32(ro.load(CUR * kStage + QdoStage<D>::kDo, 0, ks), ro.load(vpatch_off, 0, ks), dp);
       }
       const bool interior = tile_is_interior(q_uni, q_end_min, my_uni, my_rb * 32 + 31);
       f32x16 prob;
-      // The row offsets below depend on the lane only; hoisted out of the loop they become
-      // spilled registers whose reloads wait for every copy in flight. Recompute them here.
-      int half_here = half;
-      asm volatile("" : "+v"(half_here));
       if (!interior) {
         // Masked scores become -inf (their probability is then exactly 0). Written with
         // bitwise logic and selects only: the per-element tests must not turn into branches.
@@ -732,17 +745,10 @@ __global__ __launch_bounds__(256, 2) void attn_dkv_kernel(AttnParams p) {
         }
       }
 #pragma unroll
-      for (int qd = 0; qd < 4; ++qd) {
-        const int r0 = 8 * qd + 4 * half_here;
-        const f32x4 lse4 = lds_load<f32x4>(stage + QdoStage<D>::kLse + r0 * 4);
-        const f32x4 del4 = lds_load<f32x4>(stage + QdoStage<D>::kDelta + r0 * 4);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = 4 * qd + e;
-          const float pr = exp2_fast((s[r] + lse4[e]) * scale_log2e);  // lse4 = -lse / scale
-          prob[r] = pr;
-          dp[r] = pr * (dp[r] + del4[e]);                              // del4 = -delta
-        }
+      for (int r = 0; r < 16; ++r) {
+        const float pr = exp2_fast(s[r] * scale_log2e);  // s = S - lse / scale
+        prob[r] = pr;
+        dp[r] = pr * dp[r];                              // dp = dP - delta
       }
       if constexpr (SPILL) {
         // The block as the lanes hold it: the two operands of the dK product (8 query rows of one

@@ -348,9 +348,10 @@ def dkv_sdp_sequence():
     DKV_SLOTS registers quads: a read is issued as soon as the MFMA that used its slot has been
     issued, so reads stay DKV_SLOTS fragments in front of their MFMAs.
 
-    operands: %0 S, %1 dP (written), %2-%9 row-fragment pointers (k-step), %10-%17 K fragments
-    (registers), %18 byte offset of this wavefront's V rows (scalar), %19 byte offset of the
-    stage (Q tile; the dO tile follows 8192 bytes later).
+    operands: %0 S, %1 dP (read and written: the chains start from what the caller put there, the
+    per-row terms -lse / scale and -delta), %2-%9 row-fragment pointers (k-step), %10-%17 K
+    fragments (registers), %18 byte offset of this wavefront's V rows (scalar), %19 byte offset of
+    the stage (Q tile; the dO tile follows 8192 bytes later).
     """
     steps = 8
     total = 3 * steps  # read r = 3 ks + which; which: 0 Q, 1 dO, 2 V
@@ -376,12 +377,11 @@ def dkv_sdp_sequence():
         do_slot = dkv_slot((3 * ks + 1) % DKV_SLOTS)
         v_slot = dkv_slot((3 * ks + 2) % DKV_SLOTS)
         lines.append("s_waitcnt lgkmcnt(%d)" % (state["issued"] - (3 * ks + 1)))
-        lines.append("v_mfma_f32_32x32x16_bf16 %%0, v[%d:%d], %%%d, %s" % (q_slot[0], q_slot[1], 10 + ks,
-                                                                        "0" if ks == 0 else "%0"))
+        lines.append("v_mfma_f32_32x32x16_bf16 %%0, v[%d:%d], %%%d, %%0" % (q_slot[0], q_slot[1], 10 + ks))
         lines += load_next()
         lines.append("s_waitcnt lgkmcnt(%d)" % (state["issued"] - (3 * ks + 3)))
-        lines.append("v_mfma_f32_32x32x16_bf16 %%1, v[%d:%d], v[%d:%d], %s" % (do_slot[0], do_slot[1], v_slot[0],
-                                                                              v_slot[1], "0" if ks == 0 else "%1"))
+        lines.append("v_mfma_f32_32x32x16_bf16 %%1, v[%d:%d], v[%d:%d], %%1" % (do_slot[0], do_slot[1], v_slot[0],
+                                                                               v_slot[1]))
         lines += load_next()
         lines += load_next()
     return lines + DKV_TAIL
