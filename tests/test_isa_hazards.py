@@ -85,8 +85,9 @@ def test_library_sources_have_no_scalar_base_hazard(ct):
 def test_steady_state_paths_keep_their_instruction_budget(ct):
     """Vector ALU instructions per MFMA on the paths an all-allowed key tile takes, read off the
     compiled head-dimension-128 kernels. What the arithmetic alone needs per score is fma + exp2 + add
-    (+ half a max3 and half a bf16 packing) in the forward, and add, mul, exp2, add, mul (+ a
-    packing each for P and dS) in the backward: 4.0, 3.5 and 3.5 per MFMA. The kernels with two
+    (+ half a max3 and half a bf16 packing) in the forward, fma, exp2, sub, mul (+ half a packing)
+    in dQ, and mul, exp2, mul (+ a packing each for P and dS; the sums with the per-row terms come
+    out of the matrix pipe) in dK/dV: 4.0, 3.0 and 2.0 per MFMA. The kernels with two
     wavefronts per SIMD add the rebuilding of their swizzled fragment addresses per tile (their 16
     pointers do not fit beside the accumulators), which is the rest. The bounds hold these paths
     where they are; masked tiles and the per-item prologue and epilogue come on top (measured
@@ -125,6 +126,6 @@ def test_steady_state_paths_keep_their_instruction_budget(ct):
     dq_valu, dq_salu = loop_ratio("attn_dq_kernelILi128ELi4E", 48)
     dkv_valu, dkv_salu = loop_ratio("attn_dkv_kernelILi128ELb0E", 32)
     stored_valu, _ = loop_ratio("attn_dkv_kernelILi128ELb1E", 32, stores_per_block=2)   # + the dS store
-    assert dq_valu <= 4.0 and dkv_valu <= 5.2 and stored_valu <= 5.3, (dq_valu, dkv_valu, stored_valu)
+    assert dq_valu <= 4.0 and dkv_valu <= 4.1 and stored_valu <= 4.2, (dq_valu, dkv_valu, stored_valu)
     # scalar instructions of those blocks: bounds, branches, copy bookkeeping
-    assert dq_salu <= 2.0 and dkv_salu <= 2.2, (dq_salu, dkv_salu)
+    assert dq_salu <= 2.0 and dkv_salu <= 2.0, (dq_salu, dkv_salu)
