@@ -167,13 +167,26 @@ class _CutCE(torch.autograd.Function):
 def pallas_cut_linear_cross_entropy(hidden_states, lm_head_kernel, targets, weights, *, mesh=None,
                                     sparse_compaction: bool = False,
                                     lm_head_trainable: bool = True, local_chunk_size: int = 0,
-                                    logits_cache: bool = True):
+                                    logits_cache: bool = True, head_layout: str = "dv"):
     """Return ``(nll_sum, weight_sum)``; logits are only ever kept in the bounded cache
     described in the module docstring (``logits_cache=False`` disables it).
 
     hidden_states ``[B, S, d]``, lm_head_kernel ``[d, V]`` (same float dtype, bf16),
     targets int32 ``[B, S]``, weights f32 ``[B, S]``; a row is ignored iff its weight is 0.
+
+    ``head_layout="vd"``: lm_head_kernel is ``[V, d]`` (a checkpoint's ``[out, in]`` layout, which the
+    reference transposes once at load, src/causal_trainer/checkpointing/huggingface.py:1-6). The
+    kernels read ``[d, V]`` with the vocabulary contiguous, so this layout costs a transposing copy
+    of the head per call and one of its gradient in the backward (2 B read + 2 B written per element
+    each, about 0.4 ms per GB on this part); its gradient comes back as ``[V, d]``.
     """
+
+    if head_layout not in ("dv", "vd"):
+        raise ValueError("head_layout must be 'dv' ([hidden, vocab]) or 'vd' ([vocab, hidden])")
+    if head_layout == "vd":
+        if lm_head_kernel.ndim != 2:
+            raise ValueError("lm_head_kernel must have shape [vocab, hidden]")
+        lm_head_kernel = lm_head_kernel.t()   # (made contiguous below; autograd transposes the gradient back)
 
     local_chunk_size = _integer(local_chunk_size, "local_chunk_size must be a static non-negative integer")
     if local_chunk_size < 0:

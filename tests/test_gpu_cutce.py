@@ -119,6 +119,32 @@ def test_weight_patterns(ct, gpu, pattern):
         assert not with_c[3].any() and not with_c[4].any()
 
 
+def test_head_layout_vocab_major(ct, gpu):
+    """The operator with the head given as [V, d] (a checkpoint's layout): the same loss and hidden
+    gradient as with [d, V], bit for bit (the kernels see the same transposed copy), and the head's
+    gradient in the layout the head came in."""
+
+    hidden, head, targets, weights = _case(5, 600, 128, 700)
+    hidden3 = hidden.reshape(2, 300, 128).to(gpu).requires_grad_(True)
+    targets2, weights2 = targets.reshape(2, 300).to(gpu), weights.reshape(2, 300).to(gpu)
+    outcomes = {}
+    for layout in ("dv", "vd"):
+        kernel = (head if layout == "dv" else head.t().contiguous()).to(gpu).requires_grad_(True)
+        nll, weight_sum = ct.pallas_cut_linear_cross_entropy(hidden3, kernel, targets2, weights2, head_layout=layout)
+        (dh, dw) = torch.autograd.grad(nll, (hidden3, kernel))
+        outcomes[layout] = (float(nll), float(weight_sum), dh.cpu(), dw.cpu())
+    assert outcomes["dv"][:2] == outcomes["vd"][:2]
+    assert torch.equal(outcomes["dv"][2], outcomes["vd"][2])
+    assert outcomes["vd"][3].shape == (700, 128) and torch.equal(outcomes["dv"][3], outcomes["vd"][3].t())
+    _, dh_pure, dw_pure = ref.full_logits_loss_and_grads(hidden, head, targets, weights, 1.0)
+    assert relative_l2(outcomes["vd"][2].reshape(600, 128), dh_pure) <= GRAD_RTOL
+    assert relative_l2(outcomes["vd"][3].t(), dw_pure) <= GRAD_RTOL
+    with pytest.raises(ValueError, match="head_layout"):
+        ct.pallas_cut_linear_cross_entropy(hidden3, head.to(gpu), targets2, weights2, head_layout="rows")
+    with pytest.raises(ValueError, match="hidden, vocab"):
+        ct.pallas_cut_linear_cross_entropy(hidden3, head.to(gpu), targets2, weights2, head_layout="vd")
+
+
 def test_small_workspace_walks_vocabulary_slabs(ct, gpu):
     case = _case(9, 900, 256, 1500)
     lib = ct._lib.load()
