@@ -894,25 +894,33 @@ CT_DEVICE void store_slot_rows_t(const f32x16* acc, float row_scale, lds_addr pa
   int l = lane_id();
   asm volatile("" : "+v"(l));
   const int row_of_lane = ds_slot_row(l & 31), half = l >> 5;
-#pragma unroll
-  for (int db = 0; db < D / 32; ++db) {
-#pragma unroll
-    for (int qd = 0; qd < 4; ++qd) {
-      const int d0 = db * 32 + 8 * qd + 4 * half;
+  using Patch = PatchRows<D>;
+  const lds_addr store_base = Patch::store_base(patch, row_of_lane, half);
+  const unsigned row_swizzle = Patch::row_swizzle(row_of_lane);
+  auto block = [&](auto db_tag) {
+    constexpr int db = decltype(db_tag)::value;
+    auto quad = [&](auto qd_tag) {
+      constexpr int qd = decltype(qd_tag)::value;
       bf16x4 pk;
 #pragma unroll
       for (int e = 0; e < 4; ++e) pk[e] = (bf16)(acc[db][4 * qd + e] * row_scale);
-      lds_store<bf16x4>(patch + tile_byte_offset<CPR>(row_of_lane, d0 >> 3) + (d0 & 4) * 2, pk);
-    }
+      lds_store<bf16x4>(store_base + Patch::template chunk_term<db * 4 + qd>(row_swizzle), pk);
+    };
+    quad(std::integral_constant<int, 0>{});
+    quad(std::integral_constant<int, 1>{});
+    quad(std::integral_constant<int, 2>{});
+    quad(std::integral_constant<int, 3>{});
+  };
+  block(std::integral_constant<int, 0>{});
+  block(std::integral_constant<int, 1>{});
+  if constexpr (D > 64) {
+    block(std::integral_constant<int, 2>{});
+    block(std::integral_constant<int, 3>{});
   }
+  static_assert(D == 64 || D == 128, "two or four 32-column blocks");
+  (void)CPR;
   __builtin_amdgcn_wave_barrier();
-#pragma unroll
-  for (int n = 0; n < 32 * CPR / 64; ++n) {
-    const int e = l + 64 * n;
-    const int row = e / CPR, c = e % CPR;
-    const u32x4 val = lds_load<u32x4>(patch + tile_byte_offset<CPR>(row, c));
-    store_global16(gbase + (size_t)row * row_stride + c * 8, val);
-  }
+  Patch::to_global(patch, l, gbase, row_stride);
 }
 
 // s_waitcnt vmcnt(n) for a wave-uniform n that is one of the few values the walk produces.
