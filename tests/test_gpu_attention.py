@@ -132,6 +132,39 @@ def test_forward_backward_match_oracle(ct, gpu, case, bwd_variant):
     _check_against_oracle(results, q, k, v, dout, ids, ends, scale)
 
 
+def test_several_query_tiles_per_workgroup_with_empty_ones(ct, gpu, bwd_variant):
+    """Rows long enough for every forward workgroup to walk several query tiles one after the other
+    (a tile's first K rows are copied while the tile before it finishes), with stretches of padding
+    that leave whole 64-row tiles without a single key between tiles that have many, over three
+    batch rows: the hand-over between tiles, including to and from a tile with nothing to do."""
+
+    rng = np.random.default_rng(77)
+    batch, seq = 3, 2048
+    ids = np.zeros((batch, seq), np.int32)
+    for row in range(batch):
+        position, segment = int(rng.integers(0, 200)), 1
+        while position < seq:
+            length = int(rng.integers(1, 300))
+            if rng.random() < 0.3:
+                position += int(rng.integers(64, 260))      # padding: up to four whole tiles
+                continue
+            ids[row, position:position + length] = segment
+            position += length
+            segment += 1
+    blocks = ids.reshape(batch, seq // 64, 64)
+    assert ((blocks == 0).all(-1).sum(-1) >= 2).all()       # every row has tiles without any key
+    q = _bf16(rng.standard_normal((batch, seq, 4, 128)))
+    k = _bf16(rng.standard_normal((batch, seq, 1, 128)))
+    v = _bf16(rng.standard_normal((batch, seq, 1, 128)))
+    dout = _bf16(rng.standard_normal((batch, seq, 4, 128)))
+    scale = 128 ** -0.5
+    results = _run_gpu(ct, gpu, q, k, v, dout, ids, None, scale)
+    _check_against_oracle(results, q, k, v, dout, ids, None, scale)
+    again = _run_gpu(ct, gpu, q, k, v, dout, ids, None, scale)
+    for first, second in zip(results, again):
+        assert torch.equal(first, second)
+
+
 @pytest.mark.parametrize("seq,expected", [(4096, "from_ds"), (8192, "narrow"), (16384, "wide")])
 def test_default_choices_of_the_backward(ct, gpu, seq, expected):
     """Left to itself the backward takes dQ from stored dS blocks at rows of up to 4096 positions (the

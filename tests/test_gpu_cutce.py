@@ -132,7 +132,7 @@ def test_head_layout_vocab_major(ct, gpu):
         kernel = (head if layout == "dv" else head.t().contiguous()).to(gpu).requires_grad_(True)
         nll, weight_sum = ct.pallas_cut_linear_cross_entropy(hidden3, kernel, targets2, weights2, head_layout=layout)
         (dh, dw) = torch.autograd.grad(nll, (hidden3, kernel))
-        outcomes[layout] = (float(nll), float(weight_sum), dh.cpu(), dw.cpu())
+        outcomes[layout] = (float(nll.detach()), float(weight_sum.detach()), dh.cpu(), dw.cpu())
     assert outcomes["dv"][:2] == outcomes["vd"][:2]
     assert torch.equal(outcomes["dv"][2], outcomes["vd"][2])
     assert outcomes["vd"][3].shape == (700, 128) and torch.equal(outcomes["dv"][3], outcomes["vd"][3].t())
