@@ -146,6 +146,13 @@ def test_cutce_argument_errors(ct):
     for invalid in (True, 1.5, "128", -1):
         with pytest.raises((TypeError, ValueError), match="local_chunk_size"):
             fn(hidden, head, targets, weights, local_chunk_size=invalid)
+    # the head as [vocab, hidden]: named by the option, checked like the other layout
+    with pytest.raises(ValueError, match="head_layout"):
+        fn(hidden, head, targets, weights, head_layout="vocab_major")
+    with pytest.raises(ValueError, match=r"\[hidden, vocab\]"):
+        fn(hidden, head, targets, weights, head_layout="vd")
+    with pytest.raises(RuntimeError, match="only on a ROCm GPU"):
+        fn(hidden, head.T.contiguous(), targets, weights, head_layout="vd")
     with pytest.raises(RuntimeError, match="only on a ROCm GPU"):
         fn(hidden, head, targets, weights)
 
